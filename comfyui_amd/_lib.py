@@ -1,0 +1,107 @@
+"""ctypes binding of libhdmoe.so (the C ABI declared in include/hdmoe.h).
+
+The library is the only compute path of this package: if it is missing the import
+of this module raises, there is no fallback.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libhdmoe.so")
+
+W_BF16 = 0
+W_E4M3FN = 1
+MAX_EXPERTS = 16
+E_NULL, E_SHAPE, E_WORKSPACE, E_LAUNCH = -1, -2, -3, -4
+TOPK = 2
+
+c_void_p = ctypes.c_void_p
+c_int = ctypes.c_int
+c_int64 = ctypes.c_int64
+c_size_t = ctypes.c_size_t
+
+
+class FfnWeights(ctypes.Structure):
+    """hdmoe_ffn_weights"""
+    _fields_ = [
+        ("w1", c_void_p), ("w2", c_void_p), ("w3", c_void_p),
+        ("scale_w1", c_void_p), ("scale_w2", c_void_p), ("scale_w3", c_void_p),
+        ("scale_in1", c_void_p), ("scale_in2", c_void_p), ("scale_in3", c_void_p),
+    ]
+
+
+class LayerArgs(ctypes.Structure):
+    """hdmoe_layer_args"""
+    _fields_ = [
+        ("T", c_int), ("D", c_int), ("H", c_int), ("Hs", c_int), ("E", c_int), ("weight_dtype", c_int),
+        ("x", c_void_p), ("gate_w", c_void_p),
+        ("experts", ctypes.POINTER(FfnWeights)), ("shared", ctypes.POINTER(FfnWeights)),
+        ("out", c_void_p), ("workspace", c_void_p), ("workspace_bytes", c_size_t),
+        ("topk_idx", c_void_p), ("topk_weight", c_void_p),
+    ]
+
+
+class LayerLayout(ctypes.Structure):
+    """hdmoe_layer_layout"""
+    _fields_ = [(n, c_size_t) for n in
+                ("topk_idx", "topk_weight", "counts", "offsets", "perm", "inv_perm", "dispatch_ws",
+                 "a", "h", "y", "total")]
+
+
+# name -> (restype, argtypes); every symbol include/hdmoe.h declares
+SIGNATURES = {
+    "hdmoe_version": (c_int, []),
+    "hdmoe_last_error": (ctypes.c_char_p, []),
+    "hdmoe_gate_top2": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),
+    "hdmoe_dispatch_workspace_bytes": (c_size_t, [c_int, c_int]),
+    "hdmoe_dispatch": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t,
+                               c_void_p]),
+    "hdmoe_quant_fp8": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_void_p, c_void_p]),
+    "hdmoe_quant_permute_fp8": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                                        ctypes.POINTER(c_void_p), c_void_p, c_void_p]),
+    "hdmoe_permute_bf16": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p]),
+    "hdmoe_grouped_swiglu": (c_int, [c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                                     ctypes.POINTER(FfnWeights), c_void_p, c_void_p]),
+    "hdmoe_grouped_down": (c_int, [c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                                   ctypes.POINTER(FfnWeights), c_void_p, c_void_p]),
+    "hdmoe_linear": (c_int, [c_int, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "hdmoe_silu_mul_bf16": (c_int, [c_void_p, c_void_p, c_int64, c_void_p, c_void_p]),
+    "hdmoe_scale_to_bf16": (c_int, [c_int, c_void_p, c_int64, c_void_p, c_void_p, c_void_p]),
+    "hdmoe_combine": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p]),
+    "hdmoe_layer_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int, c_int]),
+    "hdmoe_moe_ffn": (c_int, [ctypes.POINTER(LayerArgs), c_void_p]),
+    "hdmoe_layer_layout_get": (c_int, [c_int, c_int, c_int, c_int, c_int, c_int, ctypes.POINTER(LayerLayout)]),
+}
+
+
+class HdmoeError(RuntimeError):
+    def __init__(self, code, message):
+        super().__init__(f"libhdmoe error {code}: {message}")
+        self.code = code
+
+
+def _load():
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"{LIB_PATH} is missing. Build it with `python -m comfyui_amd.build` (needs hipcc); "
+            "comfyui_amd has no other compute path.")
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    return lib
+
+
+lib = _load()
+
+
+def check(rc):
+    """Raise HdmoeError for a negative return code of an entry point."""
+    if rc != 0:
+        raise HdmoeError(rc, lib.hdmoe_last_error().decode("utf-8", "replace"))
+
+
+def ptr(t):
+    """Device (or host) address of a tensor, None -> NULL."""
+    return None if t is None else t.data_ptr()

@@ -1,0 +1,60 @@
+"""Compile comfyui_amd/csrc/*.hip into comfyui_amd/libhdmoe.so for gfx950 with hipcc.
+
+hipcc cross-compiles without a GPU present. Run as `python -m comfyui_amd.build`
+(or through __graft_entry__.build()). The library is built in-tree so that the
+Python side can load it with ctypes from a fixed place.
+"""
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB = os.path.join(HERE, "libhdmoe.so")
+SOURCES = ["gate.hip", "dispatch.hip", "elementwise.hip", "gemm.hip", "layer.hip"]
+
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950",
+    "-O3",
+    "-std=c++17",
+    "-fPIC",
+    # never let the compiler form packed fp32 instructions
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wall",
+    "-Wno-unused-function",
+]
+
+
+def build(verbose=True, extra_flags=()):
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    objs = []
+    procs = []
+    for src in SOURCES:
+        obj = os.path.join(CSRC, src.replace(".hip", ".o"))
+        cmd = [hipcc, *HIPCC_FLAGS, *extra_flags, "-c", os.path.join(CSRC, src), "-o", obj]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
+        objs.append(obj)
+    failed = False
+    for src, p in procs:
+        out, _ = p.communicate()
+        out = "\n".join(l for l in out.splitlines() if "packed-fp32-ops" not in l and l.strip())
+        if out and verbose:
+            print(out)
+        if p.returncode != 0:
+            failed = True
+            print(f"FAILED: {src}", file=sys.stderr)
+            if not verbose:
+                print(out, file=sys.stderr)
+    if failed:
+        raise RuntimeError("hipcc failed")
+    cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+    return LIB
+
+
+if __name__ == "__main__":
+    build()

@@ -1,0 +1,147 @@
+// Token dispatch: stable counting sort of the flat expert ids.
+// Replaces the E boolean-mask gathers of MOEFeedForwardSwiGLU.forward
+// (/root/reference/comfy/ldm/hidream/model.py:313-318), which pick, for expert i,
+// the flat slots p = 2t+s with topk_idx[p] == i in ascending p.
+//
+// Two launches over chunks of CHUNK flat slots:
+//   count:   per-chunk expert histogram from wave ballots        -> chunk_counts[chunk][E]
+//   scatter: every block sums the histograms of the chunks before it (and all of
+//            them for the global counts/offsets), then ranks its own slots with
+//            ballot prefix counts inside a wave and an LDS scan across waves, and
+//            writes perm / inv_perm.
+// No atomics, so the result does not depend on scheduling.
+// Traffic: 2T*4 bytes read twice, 2*2T*4 bytes written.
+#include "common.h"
+
+namespace {
+
+constexpr int THREADS = 256;
+constexpr int WAVES = THREADS / 64;
+constexpr int ITEMS = 8;
+constexpr int CHUNK = THREADS * ITEMS;  // flat slots per block
+
+__global__ __launch_bounds__(THREADS) void dispatch_count_kernel(const int32_t* __restrict__ flat, int n,
+                                                                 int E, int32_t* __restrict__ chunk_counts) {
+  __shared__ int32_t wave_cnt[WAVES][HDMOE_MAX_EXPERTS];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int base = blockIdx.x * CHUNK;
+  int32_t cnt = 0;  // lane e (< E) of each wave accumulates the wave's count for expert e
+  for (int it = 0; it < ITEMS; ++it) {
+    const int p = base + it * THREADS + threadIdx.x;
+    const int e = p < n ? flat[p] : -1;  // ids outside [0,E) match no ballot and are dropped
+    for (int q = 0; q < E; ++q) {
+      const unsigned long long m = __ballot(e == q);
+      if (lane == q) cnt += __popcll(m);
+    }
+  }
+  if (lane < E) wave_cnt[wave][lane] = cnt;
+  __syncthreads();
+  if (threadIdx.x < E) {
+    int32_t s = 0;
+    for (int w = 0; w < WAVES; ++w) s += wave_cnt[w][threadIdx.x];
+    chunk_counts[(size_t)blockIdx.x * E + threadIdx.x] = s;
+  }
+}
+
+__global__ __launch_bounds__(THREADS) void dispatch_scatter_kernel(
+    const int32_t* __restrict__ flat, int n, int E, int nchunks, const int32_t* __restrict__ chunk_counts,
+    int32_t* __restrict__ counts, int32_t* __restrict__ offsets, int32_t* __restrict__ perm,
+    int32_t* __restrict__ inv_perm) {
+  __shared__ int32_t total[HDMOE_MAX_EXPERTS];
+  __shared__ int32_t before[HDMOE_MAX_EXPERTS];
+  __shared__ int32_t cursor[HDMOE_MAX_EXPERTS];  // next sorted row per expert for this block
+  __shared__ int32_t wave_cnt[WAVES][HDMOE_MAX_EXPERTS];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+
+  // per expert: rows in earlier chunks, rows overall. Wave w handles experts w, w+WAVES, ...
+  for (int e = wave; e < E; e += WAVES) {
+    int32_t tot = 0, bef = 0;
+    for (int c = lane; c < nchunks; c += 64) {
+      const int32_t v = chunk_counts[(size_t)c * E + e];
+      tot += v;
+      if (c < (int)blockIdx.x) bef += v;
+    }
+    for (int off = 32; off >= 1; off >>= 1) {
+      tot += __shfl_xor(tot, off, 64);
+      bef += __shfl_xor(bef, off, 64);
+    }
+    if (lane == 0) { total[e] = tot; before[e] = bef; }
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int32_t run = 0;
+    for (int e = 0; e < E; ++e) {
+      cursor[e] = run + before[e];
+      if (blockIdx.x == 0) { counts[e] = total[e]; offsets[e] = run; }
+      run += total[e];
+    }
+    if (blockIdx.x == 0) offsets[E] = run;
+  }
+  __syncthreads();
+
+  const int base = blockIdx.x * CHUNK;
+  const unsigned long long lt = (1ull << lane) - 1ull;
+  for (int it = 0; it < ITEMS; ++it) {
+    const int p = base + it * THREADS + threadIdx.x;
+    int e = p < n ? flat[p] : -1;
+    if (e >= E) e = -1;  // never index the LDS tables with a bad id
+    int32_t rank = 0;   // slots of my expert in lower lanes of my wave
+    int32_t mine = 0;   // lane q holds the wave's count for expert q
+    for (int q = 0; q < E; ++q) {
+      const unsigned long long m = __ballot(e == q);
+      if (e == q) rank = __popcll(m & lt);
+      if (lane == q) mine = __popcll(m);
+    }
+    if (lane < E) wave_cnt[wave][lane] = mine;
+    __syncthreads();
+    if (e >= 0) {
+      int32_t pos = cursor[e] + rank;
+      for (int w = 0; w < wave; ++w) pos += wave_cnt[w][e];
+      perm[pos] = p;
+      inv_perm[p] = pos;
+    }
+    __syncthreads();
+    if (threadIdx.x < E) {
+      int32_t s = 0;
+      for (int w = 0; w < WAVES; ++w) s += wave_cnt[w][threadIdx.x];
+      cursor[threadIdx.x] += s;
+    }
+    __syncthreads();
+  }
+}
+
+}  // namespace
+
+extern "C" size_t hdmoe_dispatch_workspace_bytes(int T, int E) {
+  if (T < 0 || E < 1) return 0;
+  const size_t n = (size_t)T * HDMOE_TOPK;
+  const size_t nchunks = (n + CHUNK - 1) / CHUNK;
+  return hdmoe_align_up((nchunks > 0 ? nchunks : 1) * (size_t)E * sizeof(int32_t), 256);
+}
+
+extern "C" int hdmoe_dispatch(const int32_t* topk_idx, int T, int E, int32_t* counts, int32_t* offsets,
+                              int32_t* perm, int32_t* inv_perm, void* workspace, size_t workspace_bytes,
+                              hdmoe_stream_t stream) {
+  HDMOE_REQUIRE_PTR(topk_idx);
+  HDMOE_REQUIRE_PTR(counts);
+  HDMOE_REQUIRE_PTR(offsets);
+  HDMOE_REQUIRE_PTR(perm);
+  HDMOE_REQUIRE_PTR(inv_perm);
+  HDMOE_REQUIRE_PTR(workspace);
+  if (T < 0 || E < 1 || E > HDMOE_MAX_EXPERTS)
+    return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_dispatch: T=%d E=%d (1 <= E <= %d)", T, E, HDMOE_MAX_EXPERTS);
+  if ((size_t)T * HDMOE_TOPK > (size_t)INT32_MAX)
+    return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_dispatch: T=%d too large", T);
+  if (workspace_bytes < hdmoe_dispatch_workspace_bytes(T, E) || (reinterpret_cast<uintptr_t>(workspace) & 3))
+    return hdmoe_fail(HDMOE_E_WORKSPACE, "hdmoe_dispatch: workspace %zu bytes, need %zu (4-byte aligned)",
+                      workspace_bytes, hdmoe_dispatch_workspace_bytes(T, E));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int n = T * HDMOE_TOPK;
+  int nchunks = (n + CHUNK - 1) / CHUNK;
+  if (nchunks < 1) nchunks = 1;  // T == 0 still writes counts = 0 and offsets = 0
+  int32_t* cc = static_cast<int32_t*>(workspace);
+  hipLaunchKernelGGL(dispatch_count_kernel, dim3(nchunks), dim3(THREADS), 0, s, topk_idx, n, E, cc);
+  hipLaunchKernelGGL(dispatch_scatter_kernel, dim3(nchunks), dim3(THREADS), 0, s, topk_idx, n, E, nchunks, cc,
+                     counts, offsets, perm, inv_perm);
+  return hdmoe_check_launch("hdmoe_dispatch");
+}

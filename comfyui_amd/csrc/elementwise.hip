@@ -1,0 +1,286 @@
+// Bandwidth-bound row kernels around the GEMMs: activation quantisation (with and
+// without the dispatch gather), the bf16 gather, SiLU*mul for the unfused path and
+// the weighted combine. One wavefront per row; a lane moves 8 elements (16 bytes of
+// bf16) per 512-element chunk, so every load instruction of a wave covers 1 KiB of
+// one row.
+#include "common.h"
+#include "numfmt.h"
+
+namespace {
+
+constexpr int THREADS = 256;
+constexpr int WAVES = THREADS / 64;
+
+struct ScalePtrs {
+  const float* p[HDMOE_MAX_EXPERTS];
+};
+
+__device__ __forceinline__ float bf16_lo(uint32_t u) { return __uint_as_float(u << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t u) { return __uint_as_float(u & 0xffff0000u); }
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+  return (uint32_t)hdmoe_f32_to_bf16(lo) | ((uint32_t)hdmoe_f32_to_bf16(hi) << 16);
+}
+
+// fp8_linear's activation cast (/root/reference/comfy/ops.py:337-343).
+// inv < 0 selects the scale_input-is-None rule (clamp to +-448, scale 1).
+__device__ __forceinline__ uint32_t quant1(float v, float inv) {
+  float y;
+  if (inv < 0.0f) y = v < -448.0f ? -448.0f : (v > 448.0f ? 448.0f : v);
+  else y = hdmoe_round_bf16(v * inv);  // bf16 tensor times bf16 scalar, rounded to bf16
+  return hdmoe_f32_to_e4m3fn(y);
+}
+
+__device__ __forceinline__ uint32_t quant2x(uint32_t u, float inv) {
+  return quant1(bf16_lo(u), inv) | (quant1(bf16_hi(u), inv) << 8);
+}
+
+__device__ __forceinline__ uint2 quant8(const uint4& v, float inv) {
+  uint2 o;
+  o.x = quant2x(v.x, inv) | (quant2x(v.y, inv) << 16);
+  o.y = quant2x(v.z, inv) | (quant2x(v.w, inv) << 16);
+  return o;
+}
+
+// (1.0 / scale_input).to(bfloat16) as fp32; NULL pointer -> clamp rule marker
+__device__ __forceinline__ float inv_scale(const float* s) {
+  if (s == nullptr) return -1.0f;
+  return hdmoe_round_bf16(__fdiv_rn(1.0f, *s));
+}
+
+__global__ __launch_bounds__(THREADS) void quant_rows_kernel(const uint4* __restrict__ x, long rows, int row16,
+                                                             const float* scale_in, uint2* __restrict__ out) {
+  const int lane = threadIdx.x & 63;
+  const long wave = (long)blockIdx.x * WAVES + (threadIdx.x >> 6);
+  const long nwaves = (long)gridDim.x * WAVES;
+  const float inv = inv_scale(scale_in);
+  for (long r = wave; r < rows; r += nwaves)
+    for (int u = lane; u < row16; u += 64) out[r * row16 + u] = quant8(x[r * row16 + u], inv);
+}
+
+__global__ __launch_bounds__(THREADS) void quant_permute_kernel(const uint4* __restrict__ x,
+                                                                const int32_t* __restrict__ perm,
+                                                                const int32_t* __restrict__ offsets, int rows, int E,
+                                                                int row16, ScalePtrs sp, uint2* __restrict__ out) {
+  const int lane = threadIdx.x & 63;
+  const int wave = blockIdx.x * WAVES + (threadIdx.x >> 6);
+  const int nwaves = gridDim.x * WAVES;
+  for (int r = wave; r < rows; r += nwaves) {
+    const long t = perm[r] / HDMOE_TOPK;
+    int e = 0;
+    while (e + 1 < E && r >= offsets[e + 1]) ++e;
+    const float inv = inv_scale(sp.p[e]);
+    for (int u = lane; u < row16; u += 64) out[(long)r * row16 + u] = quant8(x[t * row16 + u], inv);
+  }
+}
+
+__global__ __launch_bounds__(THREADS) void permute_rows_kernel(const uint4* __restrict__ x,
+                                                               const int32_t* __restrict__ perm, int rows, int row16,
+                                                               uint4* __restrict__ out) {
+  const int lane = threadIdx.x & 63;
+  const int wave = blockIdx.x * WAVES + (threadIdx.x >> 6);
+  const int nwaves = gridDim.x * WAVES;
+  for (int r = wave; r < rows; r += nwaves) {
+    const long t = perm[r] / HDMOE_TOPK;
+    for (int u = lane; u < row16; u += 64) out[(long)r * row16 + u] = x[t * row16 + u];
+  }
+}
+
+// bf16( bf16(silu(a)) * b ); silu evaluated in fp32 as a / (1 + exp(-a))
+__device__ __forceinline__ float silu_mul1(float a, float b) {
+  const float s = hdmoe_round_bf16(a / (1.0f + __expf(-a)));
+  return s * b;
+}
+
+__global__ __launch_bounds__(THREADS) void silu_mul_kernel(const uint4* __restrict__ a, const uint4* __restrict__ b,
+                                                           long n16, uint4* __restrict__ out) {
+  const long stride = (long)gridDim.x * THREADS;
+  for (long i = (long)blockIdx.x * THREADS + threadIdx.x; i < n16; i += stride) {
+    const uint4 va = a[i], vb = b[i];
+    uint4 o;
+    o.x = pack_bf16(silu_mul1(bf16_lo(va.x), bf16_lo(vb.x)), silu_mul1(bf16_hi(va.x), bf16_hi(vb.x)));
+    o.y = pack_bf16(silu_mul1(bf16_lo(va.y), bf16_lo(vb.y)), silu_mul1(bf16_hi(va.y), bf16_hi(vb.y)));
+    o.z = pack_bf16(silu_mul1(bf16_lo(va.z), bf16_lo(vb.z)), silu_mul1(bf16_hi(va.z), bf16_hi(vb.z)));
+    o.w = pack_bf16(silu_mul1(bf16_lo(va.w), bf16_lo(vb.w)), silu_mul1(bf16_hi(va.w), bf16_hi(vb.w)));
+    out[i] = o;
+  }
+}
+
+// (y.view(T,2,D) * w.unsqueeze(-1)).sum(1) + shared at bf16
+// (/root/reference/comfy/ldm/hidream/model.py:319,324): each product is rounded to
+// bf16, the two-term sum is formed in fp32 and rounded, then the shared row is added
+// and the result rounded again.
+__device__ __forceinline__ float comb1(float y0, float y1, float w0, float w1, float sh, bool has_shared) {
+  float s = hdmoe_round_bf16(hdmoe_round_bf16(y0 * w0) + hdmoe_round_bf16(y1 * w1));
+  return has_shared ? s + sh : s;
+}
+
+__device__ __forceinline__ uint32_t comb2(uint32_t y0, uint32_t y1, float w0, float w1, uint32_t sh, bool hs) {
+  return pack_bf16(comb1(bf16_lo(y0), bf16_lo(y1), w0, w1, bf16_lo(sh), hs),
+                   comb1(bf16_hi(y0), bf16_hi(y1), w0, w1, bf16_hi(sh), hs));
+}
+
+__global__ __launch_bounds__(THREADS) void combine_kernel(const uint4* __restrict__ y, const int2* __restrict__ inv_perm,
+                                                          const uint32_t* __restrict__ w, const uint4* __restrict__ shared,
+                                                          int T, int row16, uint4* __restrict__ out) {
+  const int lane = threadIdx.x & 63;
+  const int wave = blockIdx.x * WAVES + (threadIdx.x >> 6);
+  const int nwaves = gridDim.x * WAVES;
+  const bool hs = shared != nullptr;
+  for (int t = wave; t < T; t += nwaves) {
+    const int2 r = inv_perm[t];
+    const uint32_t wp = w[t];
+    const float w0 = bf16_lo(wp), w1 = bf16_hi(wp);
+    const uint4* y0 = y + (long)r.x * row16;
+    const uint4* y1 = y + (long)r.y * row16;
+    for (int u = lane; u < row16; u += 64) {
+      const uint4 a = y0[u], b = y1[u];
+      uint4 sh = make_uint4(0, 0, 0, 0);
+      if (hs) sh = shared[(long)t * row16 + u];
+      uint4 o;
+      o.x = comb2(a.x, b.x, w0, w1, sh.x, hs);
+      o.y = comb2(a.y, b.y, w0, w1, sh.y, hs);
+      o.z = comb2(a.z, b.z, w0, w1, sh.z, hs);
+      o.w = comb2(a.w, b.w, w0, w1, sh.w, hs);
+      out[(long)t * row16 + u] = o;
+    }
+  }
+}
+
+// out = bf16( bf16(src) * bf16(scale) ): the `weight * scale_weight` / `input * scale_weight`
+// products of the scaled-fp8 Linear without fp8 matmul (/root/reference/comfy/ops.py:407-410),
+// whose operands have already been cast to the compute dtype.
+__global__ __launch_bounds__(THREADS) void scale_fp8_to_bf16_kernel(const uint2* __restrict__ src, long n8,
+                                                                    const float* scale, uint4* __restrict__ out) {
+  const float sc = hdmoe_round_bf16(*scale);
+  const long stride = (long)gridDim.x * THREADS;
+  for (long i = (long)blockIdx.x * THREADS + threadIdx.x; i < n8; i += stride) {
+    const uint2 v = src[i];
+    float f[8];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      f[j] = hdmoe_e4m3fn_to_f32((uint8_t)(v.x >> (8 * j))) * sc;
+      f[4 + j] = hdmoe_e4m3fn_to_f32((uint8_t)(v.y >> (8 * j))) * sc;
+    }
+    out[i] = make_uint4(pack_bf16(f[0], f[1]), pack_bf16(f[2], f[3]), pack_bf16(f[4], f[5]), pack_bf16(f[6], f[7]));
+  }
+}
+
+__global__ __launch_bounds__(THREADS) void scale_bf16_kernel(const uint4* __restrict__ src, long n8, const float* scale,
+                                                             uint4* __restrict__ out) {
+  const float sc = hdmoe_round_bf16(*scale);
+  const long stride = (long)gridDim.x * THREADS;
+  for (long i = (long)blockIdx.x * THREADS + threadIdx.x; i < n8; i += stride) {
+    const uint4 v = src[i];
+    out[i] = make_uint4(pack_bf16(bf16_lo(v.x) * sc, bf16_hi(v.x) * sc), pack_bf16(bf16_lo(v.y) * sc, bf16_hi(v.y) * sc),
+                        pack_bf16(bf16_lo(v.z) * sc, bf16_hi(v.z) * sc), pack_bf16(bf16_lo(v.w) * sc, bf16_hi(v.w) * sc));
+  }
+}
+
+inline int row_blocks(long rows) {
+  long b = (rows + WAVES - 1) / WAVES;
+  if (b < 1) b = 1;
+  if (b > HDMOE_NUM_CU * 16) b = HDMOE_NUM_CU * 16;
+  return (int)b;
+}
+
+}  // namespace
+
+extern "C" int hdmoe_quant_fp8(const void* x_bf16, int64_t rows, int D, const float* scale_input_dev, void* out_fp8,
+                               hdmoe_stream_t stream) {
+  HDMOE_REQUIRE_PTR(x_bf16);
+  HDMOE_REQUIRE_PTR(out_fp8);
+  if (rows < 0 || D <= 0 || D % 8 != 0)
+    return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_quant_fp8: rows=%lld D=%d (D must be a positive multiple of 8)",
+                      (long long)rows, D);
+  if (rows == 0) return HDMOE_OK;
+  hipLaunchKernelGGL(quant_rows_kernel, dim3(row_blocks(rows)), dim3(THREADS), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const uint4*>(x_bf16), (long)rows, D / 8, scale_input_dev,
+                     static_cast<uint2*>(out_fp8));
+  return hdmoe_check_launch("hdmoe_quant_fp8");
+}
+
+extern "C" int hdmoe_quant_permute_fp8(const void* x_bf16, const int32_t* perm, const int32_t* offsets, int T, int D,
+                                       int E, const float* const* scale_input, void* a_fp8, hdmoe_stream_t stream) {
+  HDMOE_REQUIRE_PTR(x_bf16);
+  HDMOE_REQUIRE_PTR(perm);
+  HDMOE_REQUIRE_PTR(offsets);
+  HDMOE_REQUIRE_PTR(scale_input);
+  HDMOE_REQUIRE_PTR(a_fp8);
+  if (T < 0 || D <= 0 || D % 8 != 0 || E < 1 || E > HDMOE_MAX_EXPERTS)
+    return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_quant_permute_fp8: T=%d D=%d E=%d", T, D, E);
+  if (T == 0) return HDMOE_OK;
+  ScalePtrs sp;
+  for (int e = 0; e < HDMOE_MAX_EXPERTS; ++e) sp.p[e] = e < E ? scale_input[e] : nullptr;
+  const int rows = T * HDMOE_TOPK;
+  hipLaunchKernelGGL(quant_permute_kernel, dim3(row_blocks(rows)), dim3(THREADS), 0,
+                     static_cast<hipStream_t>(stream), static_cast<const uint4*>(x_bf16), perm, offsets, rows, E,
+                     D / 8, sp, static_cast<uint2*>(a_fp8));
+  return hdmoe_check_launch("hdmoe_quant_permute_fp8");
+}
+
+extern "C" int hdmoe_permute_bf16(const void* x_bf16, const int32_t* perm, int T, int D, void* a_bf16,
+                                  hdmoe_stream_t stream) {
+  HDMOE_REQUIRE_PTR(x_bf16);
+  HDMOE_REQUIRE_PTR(perm);
+  HDMOE_REQUIRE_PTR(a_bf16);
+  if (T < 0 || D <= 0 || D % 8 != 0) return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_permute_bf16: T=%d D=%d", T, D);
+  if (T == 0) return HDMOE_OK;
+  const int rows = T * HDMOE_TOPK;
+  hipLaunchKernelGGL(permute_rows_kernel, dim3(row_blocks(rows)), dim3(THREADS), 0,
+                     static_cast<hipStream_t>(stream), static_cast<const uint4*>(x_bf16), perm, rows, D / 8,
+                     static_cast<uint4*>(a_bf16));
+  return hdmoe_check_launch("hdmoe_permute_bf16");
+}
+
+extern "C" int hdmoe_silu_mul_bf16(const void* a_bf16, const void* b_bf16, int64_t n, void* out_bf16,
+                                   hdmoe_stream_t stream) {
+  HDMOE_REQUIRE_PTR(a_bf16);
+  HDMOE_REQUIRE_PTR(b_bf16);
+  HDMOE_REQUIRE_PTR(out_bf16);
+  if (n < 0 || n % 8 != 0) return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_silu_mul_bf16: n=%lld must be a multiple of 8", (long long)n);
+  if (n == 0) return HDMOE_OK;
+  const long n16 = n / 8;
+  long blocks = (n16 + THREADS - 1) / THREADS;
+  if (blocks > HDMOE_NUM_CU * 16) blocks = HDMOE_NUM_CU * 16;
+  hipLaunchKernelGGL(silu_mul_kernel, dim3((int)blocks), dim3(THREADS), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const uint4*>(a_bf16), static_cast<const uint4*>(b_bf16), n16,
+                     static_cast<uint4*>(out_bf16));
+  return hdmoe_check_launch("hdmoe_silu_mul_bf16");
+}
+
+extern "C" int hdmoe_combine(const void* y_sorted_bf16, const int32_t* inv_perm, const void* topk_weight_bf16,
+                             const void* shared_bf16, int T, int D, void* out_bf16, hdmoe_stream_t stream) {
+  HDMOE_REQUIRE_PTR(y_sorted_bf16);
+  HDMOE_REQUIRE_PTR(inv_perm);
+  HDMOE_REQUIRE_PTR(topk_weight_bf16);
+  HDMOE_REQUIRE_PTR(out_bf16);
+  if (T < 0 || D <= 0 || D % 8 != 0) return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_combine: T=%d D=%d", T, D);
+  if (T == 0) return HDMOE_OK;
+  hipLaunchKernelGGL(combine_kernel, dim3(row_blocks(T)), dim3(THREADS), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const uint4*>(y_sorted_bf16), reinterpret_cast<const int2*>(inv_perm),
+                     static_cast<const uint32_t*>(topk_weight_bf16), static_cast<const uint4*>(shared_bf16), T, D / 8,
+                     static_cast<uint4*>(out_bf16));
+  return hdmoe_check_launch("hdmoe_combine");
+}
+
+extern "C" int hdmoe_scale_to_bf16(int src_dtype, const void* src, int64_t n, const float* scale_dev, void* out_bf16,
+                                   hdmoe_stream_t stream) {
+  HDMOE_REQUIRE_PTR(src);
+  HDMOE_REQUIRE_PTR(scale_dev);
+  HDMOE_REQUIRE_PTR(out_bf16);
+  if (n < 0 || n % 8 != 0) return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_scale_to_bf16: n=%lld must be a multiple of 8", (long long)n);
+  if (src_dtype != HDMOE_W_BF16 && src_dtype != HDMOE_W_E4M3FN)
+    return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_scale_to_bf16: src_dtype=%d", src_dtype);
+  if (n == 0) return HDMOE_OK;
+  const long n8 = n / 8;
+  long blocks = (n8 + THREADS - 1) / THREADS;
+  if (blocks > HDMOE_NUM_CU * 16) blocks = HDMOE_NUM_CU * 16;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (src_dtype == HDMOE_W_E4M3FN)
+    hipLaunchKernelGGL(scale_fp8_to_bf16_kernel, dim3((int)blocks), dim3(THREADS), 0, s, static_cast<const uint2*>(src), n8,
+                       scale_dev, static_cast<uint4*>(out_bf16));
+  else
+    hipLaunchKernelGGL(scale_bf16_kernel, dim3((int)blocks), dim3(THREADS), 0, s, static_cast<const uint4*>(src), n8,
+                       scale_dev, static_cast<uint4*>(out_bf16));
+  return hdmoe_check_launch("hdmoe_scale_to_bf16");
+}

@@ -1,0 +1,202 @@
+// Gate kernel: logits = x . Wg^T, softmax, top-2 with lowest-index tie-break.
+// Replaces MoEGate.forward (/root/reference/comfy/ldm/hidream/model.py:263-283).
+//
+// One token per wavefront. Lane l owns the 8-element groups starting at element
+// l*8 + c*512 (c = 0, 1, ...): a 16-byte load per lane and chunk, so a wave reads
+// 1 KiB of the token row per load instruction, fully coalesced. Each lane keeps
+// its slice of Wg in registers (packed bf16) for the whole kernel, because the
+// slice is the same for every token the wave processes. The E dot products are
+// accumulated in fp32 with fma in ascending element order per lane and reduced
+// across the wave with an xor butterfly (32, 16, 8, 4, 2, 1). That order is fixed
+// on purpose: it is the order the CPU checker restates, which makes logits,
+// scores and therefore the routing reproducible bit for bit.
+//
+// HBM traffic per token: D*2 bytes read, 12 bytes written; the kernel is
+// bandwidth bound (the E x D weight is 20 KiB and stays in registers / L2).
+#include "common.h"
+#include "numfmt.h"
+
+#pragma clang fp contract(off)
+
+namespace {
+
+constexpr int WAVES_PER_BLOCK = 4;
+
+__device__ __forceinline__ float exp_neg(float x) {
+  // exp(x), x <= 0: ln2 split range reduction, degree-5 polynomial, exponent
+  // added through the bit pattern. Only fp32 fma/mul/add, so results do not
+  // depend on a math library.
+  x = x < -80.0f ? -80.0f : x;
+  float n = __builtin_rintf(x * 1.44269504088896341f);
+  float r = __builtin_fmaf(n, -0.693359375f, x);
+  r = __builtin_fmaf(n, 2.12194440e-4f, r);
+  float p = 1.9875691500e-4f;
+  p = __builtin_fmaf(p, r, 1.3981999507e-3f);
+  p = __builtin_fmaf(p, r, 8.3334519073e-3f);
+  p = __builtin_fmaf(p, r, 4.1665795894e-2f);
+  p = __builtin_fmaf(p, r, 1.6666665459e-1f);
+  p = __builtin_fmaf(p, r, 5.0000001201e-1f);
+  float z = r * r;
+  float y = __builtin_fmaf(p, z, r);
+  y = y + 1.0f;
+  return __uint_as_float(__float_as_uint(y) + ((uint32_t)(int32_t)n << 23));
+}
+
+__device__ __forceinline__ float bf16_lo(uint32_t u) { return __uint_as_float(u << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t u) { return __uint_as_float(u & 0xffff0000u); }
+
+__device__ __forceinline__ float dot8(const uint4& a, const uint4& b, float acc) {
+  acc = __builtin_fmaf(bf16_lo(a.x), bf16_lo(b.x), acc);
+  acc = __builtin_fmaf(bf16_hi(a.x), bf16_hi(b.x), acc);
+  acc = __builtin_fmaf(bf16_lo(a.y), bf16_lo(b.y), acc);
+  acc = __builtin_fmaf(bf16_hi(a.y), bf16_hi(b.y), acc);
+  acc = __builtin_fmaf(bf16_lo(a.z), bf16_lo(b.z), acc);
+  acc = __builtin_fmaf(bf16_hi(a.z), bf16_hi(b.z), acc);
+  acc = __builtin_fmaf(bf16_lo(a.w), bf16_lo(b.w), acc);
+  acc = __builtin_fmaf(bf16_hi(a.w), bf16_hi(b.w), acc);
+  return acc;
+}
+
+template <int E>
+__device__ __forceinline__ void finish_token(float (&logit)[E], int lane, int t, int32_t* idx,
+                                             uint16_t* wout) {
+#pragma unroll
+  for (int e = 0; e < E; ++e) {
+    float v = logit[e];
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) v = v + __shfl_xor(v, off, 64);
+    logit[e] = hdmoe_round_bf16(v);  // F.linear output is a bf16 tensor
+  }
+  float mx = logit[0];
+#pragma unroll
+  for (int e = 1; e < E; ++e) mx = logit[e] > mx ? logit[e] : mx;
+  float ex[E];
+  float sum = 0.0f;
+#pragma unroll
+  for (int e = 0; e < E; ++e) {
+    ex[e] = exp_neg(logit[e] - mx);
+    sum = sum + ex[e];
+  }
+  float score[E];
+#pragma unroll
+  for (int e = 0; e < E; ++e) score[e] = hdmoe_round_bf16(__fdiv_rn(ex[e], sum));  // softmax output is bf16
+  // first two of a stable descending sort: strict '>' keeps the lower index on ties
+  int i0 = 0;
+  float s0 = score[0];
+#pragma unroll
+  for (int e = 1; e < E; ++e)
+    if (score[e] > s0) { s0 = score[e]; i0 = e; }
+  int i1 = -1;
+  float s1 = 0.0f;
+#pragma unroll
+  for (int e = 0; e < E; ++e) {
+    if (e == i0) continue;
+    if (i1 < 0 || score[e] > s1) { s1 = score[e]; i1 = e; }
+  }
+  if (lane == 0) {
+    reinterpret_cast<int2*>(idx)[t] = make_int2(i0, i1);
+    reinterpret_cast<uint32_t*>(wout)[t] =
+        (uint32_t)hdmoe_f32_to_bf16(s0) | ((uint32_t)hdmoe_f32_to_bf16(s1) << 16);
+  }
+}
+
+// D == NCHUNK * 512: the lane's Wg slice lives in registers.
+template <int E, int NCHUNK>
+__global__ __launch_bounds__(WAVES_PER_BLOCK * 64) void gate_top2_reg_kernel(
+    const uint4* __restrict__ x, const uint4* __restrict__ wg, int T, int32_t* __restrict__ idx,
+    uint16_t* __restrict__ wout) {
+  const int lane = threadIdx.x & 63;
+  const int wave = blockIdx.x * WAVES_PER_BLOCK + (threadIdx.x >> 6);
+  const int nwaves = gridDim.x * WAVES_PER_BLOCK;
+  constexpr int ROW16 = NCHUNK * 64;  // 16-byte units per row
+  uint4 w[E][NCHUNK];
+#pragma unroll
+  for (int e = 0; e < E; ++e)
+#pragma unroll
+    for (int c = 0; c < NCHUNK; ++c) w[e][c] = wg[(size_t)e * ROW16 + c * 64 + lane];
+
+  int t = wave;
+  if (t >= T) return;
+  uint4 cur[NCHUNK], nxt[NCHUNK];
+#pragma unroll
+  for (int c = 0; c < NCHUNK; ++c) cur[c] = x[(size_t)t * ROW16 + c * 64 + lane];
+  for (; t < T; t += nwaves) {
+    const int tn = t + nwaves;
+    if (tn < T) {
+#pragma unroll
+      for (int c = 0; c < NCHUNK; ++c) nxt[c] = x[(size_t)tn * ROW16 + c * 64 + lane];
+    }
+    float logit[E];
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      float acc = 0.0f;
+#pragma unroll
+      for (int c = 0; c < NCHUNK; ++c) acc = dot8(cur[c], w[e][c], acc);
+      logit[e] = acc;
+    }
+    finish_token<E>(logit, lane, t, idx, wout);
+#pragma unroll
+    for (int c = 0; c < NCHUNK; ++c) cur[c] = nxt[c];
+  }
+}
+
+// Any D that is a multiple of 8: Wg is re-read through the cache hierarchy.
+template <int E>
+__global__ __launch_bounds__(WAVES_PER_BLOCK * 64) void gate_top2_generic_kernel(
+    const uint4* __restrict__ x, const uint4* __restrict__ wg, int T, int D, int32_t* __restrict__ idx,
+    uint16_t* __restrict__ wout) {
+  const int lane = threadIdx.x & 63;
+  const int wave = blockIdx.x * WAVES_PER_BLOCK + (threadIdx.x >> 6);
+  const int nwaves = gridDim.x * WAVES_PER_BLOCK;
+  const int row16 = D / 8;
+  for (int t = wave; t < T; t += nwaves) {
+    float logit[E];
+#pragma unroll
+    for (int e = 0; e < E; ++e) logit[e] = 0.0f;
+    for (int u = lane; u < row16; u += 64) {
+      uint4 xv = x[(size_t)t * row16 + u];
+#pragma unroll
+      for (int e = 0; e < E; ++e) logit[e] = dot8(xv, wg[(size_t)e * row16 + u], logit[e]);
+    }
+    finish_token<E>(logit, lane, t, idx, wout);
+  }
+}
+
+template <int E>
+int launch_gate(const void* x, const void* wg, int T, int D, int32_t* idx, void* w, hipStream_t s) {
+  // about 8 tokens per wave amortise the register-resident weight slice
+  int blocks = (T + WAVES_PER_BLOCK * 8 - 1) / (WAVES_PER_BLOCK * 8);
+  if (blocks < 1) blocks = 1;
+  if (blocks > HDMOE_NUM_CU * 8) blocks = HDMOE_NUM_CU * 8;
+  dim3 grid(blocks), block(WAVES_PER_BLOCK * 64);
+  const uint4* xp = static_cast<const uint4*>(x);
+  const uint4* wp = static_cast<const uint4*>(wg);
+  uint16_t* wo = static_cast<uint16_t*>(w);
+  if (E <= 4 && D == 2560) {
+    hipLaunchKernelGGL((gate_top2_reg_kernel<(E <= 4 ? E : 4), 5>), grid, block, 0, s, xp, wp, T, idx, wo);
+  } else {
+    hipLaunchKernelGGL((gate_top2_generic_kernel<E>), grid, block, 0, s, xp, wp, T, D, idx, wo);
+  }
+  return hdmoe_check_launch("hdmoe_gate_top2");
+}
+
+}  // namespace
+
+extern "C" int hdmoe_gate_top2(const void* x_bf16, const void* gate_w_bf16, int T, int D, int E,
+                               int32_t* topk_idx, void* topk_weight_bf16, hdmoe_stream_t stream) {
+  HDMOE_REQUIRE_PTR(x_bf16);
+  HDMOE_REQUIRE_PTR(gate_w_bf16);
+  HDMOE_REQUIRE_PTR(topk_idx);
+  HDMOE_REQUIRE_PTR(topk_weight_bf16);
+  if (T < 0 || D <= 0 || D % 8 != 0)
+    return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_gate_top2: T=%d D=%d (D must be a positive multiple of 8)", T, D);
+  if (T == 0) return HDMOE_OK;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  switch (E) {
+    case 2: return launch_gate<2>(x_bf16, gate_w_bf16, T, D, topk_idx, topk_weight_bf16, s);
+    case 4: return launch_gate<4>(x_bf16, gate_w_bf16, T, D, topk_idx, topk_weight_bf16, s);
+    case 8: return launch_gate<8>(x_bf16, gate_w_bf16, T, D, topk_idx, topk_weight_bf16, s);
+    case 16: return launch_gate<16>(x_bf16, gate_w_bf16, T, D, topk_idx, topk_weight_bf16, s);
+    default: return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_gate_top2: E=%d not in {2,4,8,16}", E);
+  }
+}

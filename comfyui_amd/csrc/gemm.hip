@@ -1,0 +1,464 @@
+// Grouped "NT" GEMM on the gfx950 matrix cores for the expert feed-forwards:
+//   out[r, n] = epilogue( sum_k a[r, k] * w_g[n, k] ),  r in the row segment of group g.
+// Replaces the per-expert operations.Linear calls of FeedForwardSwiGLU.forward
+// (/root/reference/comfy/ldm/hidream/model.py:237-238) as fp8_linear evaluates them
+// (/root/reference/comfy/ops.py:345-348: fp8 x fp8 products, fp32 accumulation,
+// * scale_input*scale_weight, rounded to bf16) or, for bf16 weights, as a bf16
+// Linear does (ops.py:107-115).
+//
+// Both operands are K-contiguous, which is the layout the MFMA wants: a lane feeds
+// 32 (fp8) or 16 (bf16) consecutive K bytes of one row. Weights take the MFMA "A"
+// slot (rows of the 32x32 result = output features) and tokens the "B" slot (columns
+// = tokens), so a lane ends up with 4 consecutive features of one token per
+// accumulator quad and can store them as one packed word.
+//
+// Block = 512 threads = 8 waves (2 per SIMD), block tile 256 tokens x 256 weight rows,
+// K step 128 bytes, 2 LDS stages of 64 KiB filled by buffer_load ... lds (global ->
+// LDS without passing through registers). Wave (wq, wt) owns weight rows {wq*32..+32}
+// of each 128-row half and tokens {wt*128..+128}: 2x4 MFMA tiles of 32x32, 128 fp32
+// accumulators per lane. In SwiGLU mode the two 128-row halves of the weight tile are
+// the SAME 128 hidden features of w1 (gate) and w3 (up), so silu(gate)*up is formed
+// in registers and the [rows, 2H] intermediate never exists.
+//
+// LDS tile layout: row-major, 128 bytes per row, 16-byte chunks XOR-swizzled with
+// f(row) = ((row>>1)&7) ^ ((row&1)<<2) so that the 16-byte MFMA fragment reads of 8
+// or 16 consecutive rows hit distinct banks. The global->LDS path writes LDS linearly
+// per lane, so the swizzle is applied to the global address each lane fetches.
+//
+// Groups: row segments come from the dispatch offsets on the device (no host sync).
+// The grid is sized for the worst case; a block first decodes (group, m-tile, n-tile)
+// from its index and exits if its index is past the real tile count. Block ids are
+// remapped so that each XCD (ids congruent mod 8) walks a contiguous range of tiles,
+// 4 m-tiles deep, and its L2 sees each operand tile reused by neighbouring blocks.
+#include "common.h"
+#include "numfmt.h"
+
+namespace {
+
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+
+constexpr int BM = 256;        // tokens per block tile
+constexpr int BN = 256;        // weight rows per block tile
+constexpr int BK = 128;        // K bytes per stage
+constexpr int TILE_BYTES = 256 * BK;
+constexpr int STAGE_BYTES = 2 * TILE_BYTES;
+constexpr int STAGES = 2;
+constexpr int SMEM_BYTES = STAGES * STAGE_BYTES;
+constexpr int GROUP_M = 4;     // m-tiles per raster band
+constexpr int NTHREADS = 512;
+constexpr int MAX_GROUPS = HDMOE_MAX_EXPERTS + 1;
+
+enum Mode { FP8_SWIGLU = 0, FP8_PLAIN = 1, BF16_SWIGLU = 2, BF16_PLAIN = 3 };
+
+struct GemmGroup {
+  const uint8_t* a;     // activations; row indices below are relative to this base
+  const uint8_t* b0;    // plain: W [N,K]; swiglu: w1 [H,K]
+  const uint8_t* b1;    // swiglu: w3 [H,K]
+  const float* sb0;     // scale_weight of b0 (fp8)
+  const float* sb1;     // scale_weight of b1 (fp8, swiglu)
+  const float* s_in;    // scale_input of this Linear (fp8), NULL = 1
+  const float* s_next;  // scale_input of the Linear that consumes the output (fp8 swiglu), NULL = clamp rule
+  uint8_t* out;         // [rows, n_out] in the element type of the mode
+  int row_begin;        // >= 0: static segment [row_begin, row_end); < 0: offsets[dyn], offsets[dyn+1]
+  int row_end;
+  int dyn;
+  int n_out;            // output features (H for swiglu, N for plain)
+  int kbytes;           // bytes per row of a and of the weights
+};
+
+struct GemmArgs {
+  GemmGroup g[MAX_GROUPS];
+  const int32_t* offsets;
+  int G;
+};
+
+__device__ __forceinline__ int swz(int row) { return ((row >> 1) & 7) ^ ((row & 1) << 2); }
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, bytes, 0x00020000);
+}
+
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
+template <int MODE>
+__global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs args) {
+  constexpr bool FP8 = (MODE == FP8_SWIGLU || MODE == FP8_PLAIN);
+  constexpr bool SWIGLU = (MODE == FP8_SWIGLU || MODE == BF16_SWIGLU);
+  constexpr int FEAT_PER_TILE = SWIGLU ? BN / 2 : BN;  // output features per block tile
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+
+  // ---- which tile --------------------------------------------------------------
+  const int nb = gridDim.x;  // multiple of 8
+  int L = (blockIdx.x % HDMOE_NUM_XCD) * (nb / HDMOE_NUM_XCD) + blockIdx.x / HDMOE_NUM_XCD;
+  int g = 0, rb = 0, re = 0, mtiles = 0, ntiles = 0;
+  for (; g < args.G; ++g) {
+    const GemmGroup& gg = args.g[g];
+    if (gg.row_begin >= 0) { rb = gg.row_begin; re = gg.row_end; }
+    else {
+      // loaded through the vector memory path; tell the compiler the values are wave-uniform
+      rb = __builtin_amdgcn_readfirstlane(args.offsets[gg.dyn]);
+      re = __builtin_amdgcn_readfirstlane(args.offsets[gg.dyn + 1]);
+    }
+    mtiles = (re - rb + BM - 1) / BM;
+    ntiles = gg.n_out / FEAT_PER_TILE;
+    const int tiles = mtiles * ntiles;
+    if (L < tiles) break;
+    L -= tiles;
+  }
+  if (g == args.G) return;
+  const GemmGroup& gg = args.g[g];
+  const int band = L / (GROUP_M * ntiles);
+  const int first_m = band * GROUP_M;
+  const int gm = min(mtiles - first_m, GROUP_M);
+  const int within = L - band * (GROUP_M * ntiles);
+  const int mt = first_m + within % gm;
+  const int nt = within / gm;
+  const int row0 = rb + mt * BM;            // first token row of the tile
+  const int rows_here = min(re - row0, BM); // valid rows in the tile
+  const int n0 = nt * FEAT_PER_TILE;        // first output feature of the tile
+  const int kbytes = gg.kbytes;
+  const int KT = kbytes / BK;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform by construction
+  const int wq = wave & 3, wt = wave >> 2;
+
+  // ---- global -> LDS addressing --------------------------------------------------
+  // One wave-level load moves 8 rows x 128 bytes. Lane i lands in LDS chunk (i&7) of
+  // row (i>>3) and therefore fetches logical chunk (i&7) ^ f(row).
+  // Rows past the segment end are outside the buffer range and read as zero.
+  const __amdgpu_buffer_rsrc_t rsrc_a = make_rsrc(gg.a + (size_t)row0 * kbytes, (uint32_t)rows_here * (uint32_t)kbytes);
+  const uint8_t* b_half0 = gg.b0 + (size_t)n0 * kbytes;
+  const uint8_t* b_half1 = SWIGLU ? gg.b1 + (size_t)n0 * kbytes : gg.b0 + (size_t)(n0 + BN / 2) * kbytes;
+  const __amdgpu_buffer_rsrc_t rsrc_b0 = make_rsrc(b_half0, (uint32_t)(BN / 2) * (uint32_t)kbytes);
+  const __amdgpu_buffer_rsrc_t rsrc_b1 = make_rsrc(b_half1, (uint32_t)(BN / 2) * (uint32_t)kbytes);
+  const int ld_row = wave * 8 + (lane >> 3);                 // row within a 64-row slab
+  const int ld_chunk = (lane & 7) ^ swz(ld_row);
+  // The row part must sit in the VGPR offset: only that offset is range-checked, the
+  // scalar offset (used for the K position) is not.
+  int ld_voff[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) ld_voff[j] = (j * 64 + ld_row) * kbytes + ld_chunk * 16;
+  const int ld_lds = wave * 8 * BK;                          // + slab*64*BK
+
+  auto issue_loads = [&](int stage, int kt) {
+    uint8_t* sa = smem + stage * STAGE_BYTES;
+    uint8_t* sb = sa + TILE_BYTES;
+    const int k0 = kt * BK;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_ptr_t)(sa + ld_lds + j * 64 * BK), 16, ld_voff[j], k0, 0, 0);
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b0, (lds_ptr_t)(sb + ld_lds + j * 64 * BK), 16, ld_voff[j], k0, 0, 0);
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b1, (lds_ptr_t)(sb + ld_lds + (j + 2) * 64 * BK), 16, ld_voff[j], k0, 0, 0);
+  };
+
+  // ---- LDS -> MFMA fragment addressing -------------------------------------------
+  // Operand tile of 32 rows: lane l reads row (l&31); its K sub-block is (l>>5).
+  const int fr_row = lane & 31;
+  const int fr_grp = lane >> 5;
+  const int fr_swz = swz(fr_row);  // tile origins are multiples of 32 rows, so f() only sees fr_row
+  const int a_base = (wt * 128 + fr_row) * BK;               // token operand, + tt*32*BK
+  const int b_base = TILE_BYTES + (wq * 32 + fr_row) * BK;   // weight operand, + ft*128*BK
+
+  v16f acc[2][4];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
+
+  auto compute = [&](int stage) {
+    const uint8_t* st = smem + stage * STAGE_BYTES;
+    if constexpr (FP8) {
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks) {
+        const int c0 = ((ks * 4 + fr_grp * 2) ^ fr_swz) * 16;
+        const int c1 = c0 ^ 16;
+        v8i fa[4], fb[2];
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt) {
+          const uint8_t* p = st + a_base + tt * 32 * BK;
+          const v4i lo = *reinterpret_cast<const v4i*>(p + c0);
+          const v4i hi = *reinterpret_cast<const v4i*>(p + c1);
+          fa[tt] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        }
+#pragma unroll
+        for (int ft = 0; ft < 2; ++ft) {
+          const uint8_t* p = st + b_base + ft * 128 * BK;
+          const v4i lo = *reinterpret_cast<const v4i*>(p + c0);
+          const v4i hi = *reinterpret_cast<const v4i*>(p + c1);
+          fb[ft] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        }
+#pragma unroll
+        for (int ft = 0; ft < 2; ++ft)
+#pragma unroll
+          for (int tt = 0; tt < 4; ++tt)
+            acc[ft][tt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[ft], fa[tt], acc[ft][tt], 0, 0, 0, 0, 0, 0);
+      }
+    } else {
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) {
+        const int c0 = ((ks * 2 + fr_grp) ^ fr_swz) * 16;
+        v8bf fa[4], fb[2];
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt)
+          fa[tt] = *reinterpret_cast<const v8bf*>(st + a_base + tt * 32 * BK + c0);
+#pragma unroll
+        for (int ft = 0; ft < 2; ++ft)
+          fb[ft] = *reinterpret_cast<const v8bf*>(st + b_base + ft * 128 * BK + c0);
+#pragma unroll
+        for (int ft = 0; ft < 2; ++ft)
+#pragma unroll
+          for (int tt = 0; tt < 4; ++tt)
+            acc[ft][tt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[ft], fa[tt], acc[ft][tt], 0, 0, 0);
+      }
+    }
+  };
+
+  // ---- main loop: one barrier per K step --------------------------------------------
+  issue_loads(0, 0);
+  for (int kt = 0; kt < KT; kt += 2) {
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's part of the stage has landed
+    __syncthreads();                      // everyone's part has; everyone is done reading the other stage
+    if (kt + 1 < KT) issue_loads(1, kt + 1);
+    compute(0);
+    if (kt + 1 < KT) {
+      __builtin_amdgcn_s_waitcnt(0x0f70);
+      __syncthreads();
+      if (kt + 2 < KT) issue_loads(0, kt + 2);
+      compute(1);
+    }
+  }
+
+  // ---- epilogue ----------------------------------------------------------------------
+  // acc[ft][tt][i]: feature = (i>>2)*8 + (lane>>5)*4 + (i&3) within the 32-row MFMA tile (ft = weight half),
+  // token = lane&31 within the 32-token MFMA tile.
+  float s_in = 1.0f;
+  if constexpr (FP8) s_in = gg.s_in ? *gg.s_in : 1.0f;
+  const int tok_lane = wt * 128 + (lane & 31);
+  const int feat_lane = wq * 32 + (lane >> 5) * 4;
+  if constexpr (SWIGLU) {
+    float sg = 1.0f, su = 1.0f, inv_next = 1.0f;
+    if constexpr (FP8) {
+      sg = s_in * *gg.sb0;
+      su = s_in * *gg.sb1;
+      inv_next = gg.s_next ? hdmoe_round_bf16(__fdiv_rn(1.0f, *gg.s_next)) : -1.0f;
+    }
+    const int ldo = gg.n_out * (FP8 ? 1 : 2);
+#pragma unroll
+    for (int tt = 0; tt < 4; ++tt) {
+      const int tok = tok_lane + tt * 32;
+      if (tok < rows_here) {
+        uint8_t* orow = gg.out + (size_t)(row0 + tok) * ldo;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          float m[4];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const float h1 = hdmoe_round_bf16(acc[0][tt][q * 4 + i] * sg);  // w1(x) as a bf16 tensor
+            const float h3 = hdmoe_round_bf16(acc[1][tt][q * 4 + i] * su);  // w3(x)
+            const float sl = hdmoe_round_bf16(h1 / (1.0f + __expf(-h1)));   // silu(.)
+            m[i] = hdmoe_round_bf16(sl * h3);                               // silu(.) * w3(x)
+          }
+          const int feat = n0 + feat_lane + q * 8;
+          if constexpr (FP8) {
+            // activation cast of the w2 Linear (ops.py:337-343)
+            uint32_t pk = 0;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              float y;
+              if (inv_next < 0.0f) y = m[i] < -448.0f ? -448.0f : (m[i] > 448.0f ? 448.0f : m[i]);
+              else y = hdmoe_round_bf16(m[i] * inv_next);
+              pk |= (uint32_t)hdmoe_f32_to_e4m3fn(y) << (8 * i);
+            }
+            *reinterpret_cast<uint32_t*>(orow + feat) = pk;
+          } else {
+            uint2 pk;
+            pk.x = (uint32_t)hdmoe_f32_to_bf16(m[0]) | ((uint32_t)hdmoe_f32_to_bf16(m[1]) << 16);
+            pk.y = (uint32_t)hdmoe_f32_to_bf16(m[2]) | ((uint32_t)hdmoe_f32_to_bf16(m[3]) << 16);
+            *reinterpret_cast<uint2*>(orow + (size_t)feat * 2) = pk;
+          }
+        }
+      }
+    }
+  } else {
+    float sc = 1.0f;
+    if constexpr (FP8) sc = s_in * *gg.sb0;
+    const int ldo = gg.n_out * 2;
+#pragma unroll
+    for (int tt = 0; tt < 4; ++tt) {
+      const int tok = tok_lane + tt * 32;
+      if (tok < rows_here) {
+        uint8_t* orow = gg.out + (size_t)(row0 + tok) * ldo;
+#pragma unroll
+        for (int ft = 0; ft < 2; ++ft) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const int feat = n0 + ft * 128 + feat_lane + q * 8;
+            uint2 pk;
+            pk.x = (uint32_t)hdmoe_f32_to_bf16(acc[ft][tt][q * 4 + 0] * sc) |
+                   ((uint32_t)hdmoe_f32_to_bf16(acc[ft][tt][q * 4 + 1] * sc) << 16);
+            pk.y = (uint32_t)hdmoe_f32_to_bf16(acc[ft][tt][q * 4 + 2] * sc) |
+                   ((uint32_t)hdmoe_f32_to_bf16(acc[ft][tt][q * 4 + 3] * sc) << 16);
+            *reinterpret_cast<uint2*>(orow + (size_t)feat * 2) = pk;
+          }
+        }
+      }
+    }
+  }
+}
+
+template <int MODE>
+int launch_grouped(const GemmArgs& args, int tile_bound, hipStream_t s, const char* what) {
+  static bool attr_set = false;  // per process and instantiation; setting it twice is harmless
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&grouped_gemm_kernel<MODE>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES);
+    if (e != hipSuccess) return hdmoe_fail(HDMOE_E_LAUNCH, "%s: hipFuncSetAttribute: %s", what, hipGetErrorString(e));
+    attr_set = true;
+  }
+  if (tile_bound <= 0) return HDMOE_OK;
+  const int grid = (tile_bound + HDMOE_NUM_XCD - 1) / HDMOE_NUM_XCD * HDMOE_NUM_XCD;
+  hipLaunchKernelGGL((grouped_gemm_kernel<MODE>), dim3(grid), dim3(NTHREADS), SMEM_BYTES, s, args);
+  return hdmoe_check_launch(what);
+}
+
+inline int elem_bytes(int weight_dtype) { return weight_dtype == HDMOE_W_E4M3FN ? 1 : 2; }
+
+int check_dtype(int weight_dtype, const char* what) {
+  if (weight_dtype != HDMOE_W_BF16 && weight_dtype != HDMOE_W_E4M3FN)
+    return hdmoe_fail(HDMOE_E_SHAPE, "%s: weight_dtype=%d is neither HDMOE_W_BF16 nor HDMOE_W_E4M3FN", what, weight_dtype);
+  return HDMOE_OK;
+}
+
+}  // namespace
+
+// Shared by hdmoe_grouped_swiglu / hdmoe_grouped_down / hdmoe_linear / hdmoe_moe_ffn.
+// groups: n_dyn experts with device-side segments, optionally one static group (the shared expert).
+int hdmoe_launch_ffn_gemm(bool swiglu, int weight_dtype, const uint8_t* a_dyn, const int32_t* offsets, int rows_dyn,
+                          int n_dyn, const hdmoe_ffn_weights* experts, uint8_t* out_dyn, const uint8_t* a_static,
+                          int rows_static, const hdmoe_ffn_weights* shared, uint8_t* out_static, int K_dyn, int N_dyn,
+                          int K_static, int N_static, hipStream_t s, const char* what) {
+  const int eb = elem_bytes(weight_dtype);
+  const bool fp8 = weight_dtype == HDMOE_W_E4M3FN;
+  const int feat_per_tile = swiglu ? BN / 2 : BN;
+  GemmArgs args;
+  memset(&args, 0, sizeof(args));
+  args.offsets = offsets;
+  int G = 0, tile_bound = 0;
+  for (int e = 0; e < n_dyn; ++e, ++G) {
+    GemmGroup& gg = args.g[G];
+    const hdmoe_ffn_weights& w = experts[e];
+    gg.a = a_dyn;
+    gg.out = out_dyn;
+    gg.row_begin = -1;
+    gg.dyn = e;
+    gg.n_out = N_dyn;
+    gg.kbytes = K_dyn * eb;
+    if (swiglu) {
+      gg.b0 = static_cast<const uint8_t*>(w.w1); gg.b1 = static_cast<const uint8_t*>(w.w3);
+      gg.sb0 = w.scale_w1; gg.sb1 = w.scale_w3; gg.s_in = w.scale_in1; gg.s_next = w.scale_in2;
+    } else {
+      gg.b0 = static_cast<const uint8_t*>(w.w2); gg.sb0 = w.scale_w2; gg.s_in = w.scale_in2;
+    }
+    if (!gg.b0 || (swiglu && !gg.b1)) return hdmoe_fail(HDMOE_E_NULL, "%s: expert %d has a NULL weight", what, e);
+    if (fp8 && (!gg.sb0 || (swiglu && !gg.sb1)))
+      return hdmoe_fail(HDMOE_E_NULL, "%s: expert %d has a NULL scale_weight", what, e);
+  }
+  if (n_dyn > 0) tile_bound += (rows_dyn / BM + n_dyn) * (N_dyn / feat_per_tile);
+  if (shared != nullptr && rows_static > 0) {
+    GemmGroup& gg = args.g[G];
+    const hdmoe_ffn_weights& w = *shared;
+    gg.a = a_static;
+    gg.out = out_static;
+    gg.row_begin = 0;
+    gg.row_end = rows_static;
+    gg.n_out = N_static;
+    gg.kbytes = K_static * eb;
+    if (swiglu) {
+      gg.b0 = static_cast<const uint8_t*>(w.w1); gg.b1 = static_cast<const uint8_t*>(w.w3);
+      gg.sb0 = w.scale_w1; gg.sb1 = w.scale_w3; gg.s_in = w.scale_in1; gg.s_next = w.scale_in2;
+    } else {
+      gg.b0 = static_cast<const uint8_t*>(w.w2); gg.sb0 = w.scale_w2; gg.s_in = w.scale_in2;
+    }
+    if (!gg.b0 || (swiglu && !gg.b1)) return hdmoe_fail(HDMOE_E_NULL, "%s: static group has a NULL weight", what);
+    if (fp8 && (!gg.sb0 || (swiglu && !gg.sb1)))
+      return hdmoe_fail(HDMOE_E_NULL, "%s: static group has a NULL scale_weight", what);
+    tile_bound += ((rows_static + BM - 1) / BM) * (N_static / feat_per_tile);
+    ++G;
+  }
+  args.G = G;
+  if (fp8) return swiglu ? launch_grouped<FP8_SWIGLU>(args, tile_bound, s, what)
+                         : launch_grouped<FP8_PLAIN>(args, tile_bound, s, what);
+  return swiglu ? launch_grouped<BF16_SWIGLU>(args, tile_bound, s, what)
+                : launch_grouped<BF16_PLAIN>(args, tile_bound, s, what);
+}
+
+// Size rules shared by the entry points: K bytes per row must be a multiple of the
+// 128-byte K step; total bytes of each operand must fit the 32-bit buffer range.
+int hdmoe_check_gemm_shape(const char* what, int weight_dtype, long rows, int K, int N, int feat_per_tile) {
+  if (int rc = check_dtype(weight_dtype, what)) return rc;
+  const int eb = elem_bytes(weight_dtype);
+  if (rows < 0 || K <= 0 || N <= 0 || (K * eb) % BK != 0 || N % feat_per_tile != 0)
+    return hdmoe_fail(HDMOE_E_SHAPE, "%s: rows=%ld K=%d N=%d (K*%d must be a multiple of %d, N of %d)", what, rows, K,
+                      N, eb, BK, feat_per_tile);
+  if ((unsigned long long)rows * K * eb >= (1ull << 32) || (unsigned long long)rows * N * 2 >= (1ull << 40))
+    return hdmoe_fail(HDMOE_E_SHAPE, "%s: rows=%ld K=%d exceeds the 4 GiB buffer range", what, rows, K);
+  return HDMOE_OK;
+}
+
+extern "C" int hdmoe_grouped_swiglu(int weight_dtype, const void* a, const int32_t* offsets, int rows_total, int E,
+                                    int D, int H, const hdmoe_ffn_weights* experts, void* h, hdmoe_stream_t stream) {
+  HDMOE_REQUIRE_PTR(a);
+  HDMOE_REQUIRE_PTR(offsets);
+  HDMOE_REQUIRE_PTR(experts);
+  HDMOE_REQUIRE_PTR(h);
+  if (E < 1 || E > HDMOE_MAX_EXPERTS) return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_grouped_swiglu: E=%d", E);
+  if (int rc = hdmoe_check_gemm_shape("hdmoe_grouped_swiglu", weight_dtype, rows_total, D, H, BN / 2)) return rc;
+  if (rows_total == 0) return HDMOE_OK;
+  return hdmoe_launch_ffn_gemm(true, weight_dtype, static_cast<const uint8_t*>(a), offsets, rows_total, E, experts,
+                               static_cast<uint8_t*>(h), nullptr, 0, nullptr, nullptr, D, H, 0, 0,
+                               static_cast<hipStream_t>(stream), "hdmoe_grouped_swiglu");
+}
+
+extern "C" int hdmoe_grouped_down(int weight_dtype, const void* h, const int32_t* offsets, int rows_total, int E, int H,
+                                  int D, const hdmoe_ffn_weights* experts, void* y_bf16, hdmoe_stream_t stream) {
+  HDMOE_REQUIRE_PTR(h);
+  HDMOE_REQUIRE_PTR(offsets);
+  HDMOE_REQUIRE_PTR(experts);
+  HDMOE_REQUIRE_PTR(y_bf16);
+  if (E < 1 || E > HDMOE_MAX_EXPERTS) return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_grouped_down: E=%d", E);
+  if (int rc = hdmoe_check_gemm_shape("hdmoe_grouped_down", weight_dtype, rows_total, H, D, BN)) return rc;
+  if (rows_total == 0) return HDMOE_OK;
+  return hdmoe_launch_ffn_gemm(false, weight_dtype, static_cast<const uint8_t*>(h), offsets, rows_total, E, experts,
+                               static_cast<uint8_t*>(y_bf16), nullptr, 0, nullptr, nullptr, H, D, 0, 0,
+                               static_cast<hipStream_t>(stream), "hdmoe_grouped_down");
+}
+
+extern "C" int hdmoe_linear(int weight_dtype, const void* a, int rows, int K, int N, const void* w,
+                            const float* scale_w_dev, const float* scale_in_dev, void* out_bf16,
+                            hdmoe_stream_t stream) {
+  HDMOE_REQUIRE_PTR(a);
+  HDMOE_REQUIRE_PTR(w);
+  HDMOE_REQUIRE_PTR(out_bf16);
+  if (int rc = hdmoe_check_gemm_shape("hdmoe_linear", weight_dtype, rows, K, N, BN)) return rc;
+  if (weight_dtype == HDMOE_W_E4M3FN) HDMOE_REQUIRE_PTR(scale_w_dev);
+  if (rows == 0) return HDMOE_OK;
+  hdmoe_ffn_weights fw;
+  memset(&fw, 0, sizeof(fw));
+  fw.w2 = w;
+  fw.scale_w2 = scale_w_dev;
+  fw.scale_in2 = scale_in_dev;
+  return hdmoe_launch_ffn_gemm(false, weight_dtype, nullptr, nullptr, 0, 0, nullptr, nullptr,
+                               static_cast<const uint8_t*>(a), rows, &fw, static_cast<uint8_t*>(out_bf16), 0, 0, K, N,
+                               static_cast<hipStream_t>(stream), "hdmoe_linear");
+}

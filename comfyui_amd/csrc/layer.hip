@@ -1,0 +1,130 @@
+// Whole-layer entry point: enqueues every stage of MOEFeedForwardSwiGLU.forward
+// (/root/reference/comfy/ldm/hidream/model.py:307-325) on one stream, with all
+// intermediates in a caller-provided workspace. Also hosts the library-wide pieces
+// (version, thread-local error text).
+#include "common.h"
+
+int hdmoe_launch_ffn_gemm(bool swiglu, int weight_dtype, const uint8_t* a_dyn, const int32_t* offsets, int rows_dyn,
+                          int n_dyn, const hdmoe_ffn_weights* experts, uint8_t* out_dyn, const uint8_t* a_static,
+                          int rows_static, const hdmoe_ffn_weights* shared, uint8_t* out_static, int K_dyn, int N_dyn,
+                          int K_static, int N_static, hipStream_t s, const char* what);
+int hdmoe_check_gemm_shape(const char* what, int weight_dtype, long rows, int K, int N, int feat_per_tile);
+
+char* hdmoe_error_buffer() {
+  static thread_local char buf[HDMOE_ERRBUF] = {0};
+  return buf;
+}
+
+extern "C" int hdmoe_version(void) { return HDMOE_VERSION; }
+extern "C" const char* hdmoe_last_error(void) { return hdmoe_error_buffer(); }
+
+extern "C" int hdmoe_layer_layout_get(int T, int D, int H, int Hs, int E, int weight_dtype,
+                                      hdmoe_layer_layout* out) {
+  HDMOE_REQUIRE_PTR(out);
+  if (T < 0 || D <= 0 || H <= 0 || Hs < 0 || E < 1 || E > HDMOE_MAX_EXPERTS ||
+      (weight_dtype != HDMOE_W_BF16 && weight_dtype != HDMOE_W_E4M3FN))
+    return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_layer_layout_get: T=%d D=%d H=%d Hs=%d E=%d dtype=%d", T, D, H, Hs, E,
+                      weight_dtype);
+  const size_t eb = weight_dtype == HDMOE_W_E4M3FN ? 1 : 2;
+  const size_t n = (size_t)T * HDMOE_TOPK;
+  const bool fp8 = weight_dtype == HDMOE_W_E4M3FN;
+  size_t off = 0;
+  auto take = [&](size_t bytes) { size_t o = off; off = hdmoe_align_up(off + bytes, 256); return o; };
+  out->topk_idx = take(n * 4);
+  out->topk_weight = take(n * 2);
+  out->counts = take((size_t)E * 4);
+  out->offsets = take((size_t)(E + 1) * 4);
+  out->perm = take(n * 4);
+  out->inv_perm = take(n * 4);
+  out->dispatch_ws = take(hdmoe_dispatch_workspace_bytes(T, E));
+  // a: routed rows sorted by expert [2T,D], then (fp8 only) the token-order copy for the shared expert [T,D]
+  out->a = take((n + ((fp8 && Hs > 0) ? (size_t)T : 0)) * D * eb);
+  // h: routed [2T,H] then shared [T,Hs]
+  out->h = take((n * H + (size_t)T * Hs) * eb);
+  // y: routed [2T,D] then shared [T,D], bf16
+  out->y = take((n + (Hs > 0 ? (size_t)T : 0)) * D * 2);
+  out->total = off;
+  return HDMOE_OK;
+}
+
+extern "C" size_t hdmoe_layer_workspace_bytes(int T, int D, int H, int Hs, int E, int weight_dtype) {
+  hdmoe_layer_layout l;
+  if (hdmoe_layer_layout_get(T, D, H, Hs, E, weight_dtype, &l) != HDMOE_OK) return 0;
+  return l.total;
+}
+
+extern "C" int hdmoe_moe_ffn(const hdmoe_layer_args* p, hdmoe_stream_t stream) {
+  HDMOE_REQUIRE_PTR(p);
+  HDMOE_REQUIRE_PTR(p->x);
+  HDMOE_REQUIRE_PTR(p->gate_w);
+  HDMOE_REQUIRE_PTR(p->experts);
+  HDMOE_REQUIRE_PTR(p->out);
+  HDMOE_REQUIRE_PTR(p->workspace);
+  const int T = p->T, D = p->D, H = p->H, Hs = p->Hs, E = p->E, wd = p->weight_dtype;
+  hdmoe_layer_layout l;
+  if (int rc = hdmoe_layer_layout_get(T, D, H, Hs, E, wd, &l)) return rc;
+  if (Hs > 0) HDMOE_REQUIRE_PTR(p->shared);
+  if (p->workspace_bytes < l.total || (reinterpret_cast<uintptr_t>(p->workspace) & 255))
+    return hdmoe_fail(HDMOE_E_WORKSPACE, "hdmoe_moe_ffn: workspace %zu bytes, need %zu (256-byte aligned)",
+                      p->workspace_bytes, l.total);
+  const long n = (long)T * HDMOE_TOPK;
+  if (int rc = hdmoe_check_gemm_shape("hdmoe_moe_ffn (gate/up)", wd, n + T, D, H, 128)) return rc;
+  if (int rc = hdmoe_check_gemm_shape("hdmoe_moe_ffn (down)", wd, n, H, D, 256)) return rc;
+  if (Hs > 0) {
+    if (int rc = hdmoe_check_gemm_shape("hdmoe_moe_ffn (shared gate/up)", wd, T, D, Hs, 128)) return rc;
+    if (int rc = hdmoe_check_gemm_shape("hdmoe_moe_ffn (shared down)", wd, T, Hs, D, 256)) return rc;
+  }
+  if (T == 0) return HDMOE_OK;
+
+  const bool fp8 = wd == HDMOE_W_E4M3FN;
+  const size_t eb = fp8 ? 1 : 2;
+  uint8_t* ws = static_cast<uint8_t*>(p->workspace);
+  int32_t* idx = p->topk_idx ? p->topk_idx : reinterpret_cast<int32_t*>(ws + l.topk_idx);
+  void* tw = p->topk_weight ? p->topk_weight : static_cast<void*>(ws + l.topk_weight);
+  int32_t* counts = reinterpret_cast<int32_t*>(ws + l.counts);
+  int32_t* offsets = reinterpret_cast<int32_t*>(ws + l.offsets);
+  int32_t* perm = reinterpret_cast<int32_t*>(ws + l.perm);
+  int32_t* inv_perm = reinterpret_cast<int32_t*>(ws + l.inv_perm);
+  uint8_t* a_routed = ws + l.a;
+  uint8_t* a_shared = a_routed + (size_t)n * D * eb;  // fp8 only
+  uint8_t* h_routed = ws + l.h;
+  uint8_t* h_shared = h_routed + (size_t)n * H * eb;
+  uint8_t* y_routed = ws + l.y;
+  uint8_t* y_shared = y_routed + (size_t)n * D * 2;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+
+  for (int e = 0; e < E; ++e) {
+    const hdmoe_ffn_weights& w = p->experts[e];
+    if (fp8 && w.scale_in1 != w.scale_in3 && (w.scale_in1 == nullptr || w.scale_in3 == nullptr))
+      return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_moe_ffn: expert %d: w1 and w3 disagree on having a scale_input", e);
+  }
+
+  if (int rc = hdmoe_gate_top2(p->x, p->gate_w, T, D, E, idx, tw, stream)) return rc;
+  if (int rc = hdmoe_dispatch(idx, T, E, counts, offsets, perm, inv_perm, ws + l.dispatch_ws,
+                              hdmoe_dispatch_workspace_bytes(T, E), stream))
+    return rc;
+
+  const uint8_t* a_static = nullptr;
+  if (fp8) {
+    const float* sin[HDMOE_MAX_EXPERTS];
+    for (int e = 0; e < E; ++e) sin[e] = p->experts[e].scale_in1;
+    if (int rc = hdmoe_quant_permute_fp8(p->x, perm, offsets, T, D, E, sin, a_routed, stream)) return rc;
+    if (Hs > 0) {
+      if (int rc = hdmoe_quant_fp8(p->x, T, D, p->shared->scale_in1, a_shared, stream)) return rc;
+      a_static = a_shared;
+    }
+  } else {
+    if (int rc = hdmoe_permute_bf16(p->x, perm, T, D, a_routed, stream)) return rc;
+    a_static = static_cast<const uint8_t*>(p->x);
+  }
+
+  // gate/up projections + SiLU*mul, routed experts and shared expert in one launch
+  if (int rc = hdmoe_launch_ffn_gemm(true, wd, a_routed, offsets, (int)n, E, p->experts, h_routed, a_static,
+                                     Hs > 0 ? T : 0, p->shared, h_shared, D, H, D, Hs, s, "hdmoe_moe_ffn (gate/up)"))
+    return rc;
+  // down projections, both in one launch
+  if (int rc = hdmoe_launch_ffn_gemm(false, wd, h_routed, offsets, (int)n, E, p->experts, y_routed, h_shared,
+                                     Hs > 0 ? T : 0, p->shared, y_shared, H, D, Hs, D, s, "hdmoe_moe_ffn (down)"))
+    return rc;
+  return hdmoe_combine(y_routed, inv_perm, tw, Hs > 0 ? y_shared : nullptr, T, D, p->out, stream);
+}

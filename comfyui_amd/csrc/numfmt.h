@@ -1,0 +1,82 @@
+// Bit-level bf16 and float8_e4m3fn conversions shared by the HIP kernels (device)
+// and the host-side self checks. Plain integer arithmetic on IEEE-754 fp32 bit
+// patterns, so host and device produce identical bytes.
+//
+// float8_e4m3fn: 1 sign, 4 exponent (bias 7), 3 mantissa bits; no infinities;
+// 0x7F / 0xFF are NaN; largest finite value 448. The encode below is
+// round-to-nearest-even WITHOUT saturation: |v| > 464 (the midpoint between 448
+// and the would-be 480) becomes NaN, exactly what `tensor.to(torch.float8_e4m3fn)`
+// produces and therefore what the reference's fp8_linear feeds torch._scaled_mm
+// (/root/reference/comfy/ops.py:337-343).
+#pragma once
+#include <stdint.h>
+#include <string.h>
+
+#if defined(__HIPCC__) || defined(__CUDACC__)
+#define HDMOE_HD __host__ __device__ __forceinline__
+#else
+#define HDMOE_HD static inline
+#endif
+
+HDMOE_HD uint32_t hdmoe_f32_bits(float f) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  return __float_as_uint(f);
+#else
+  uint32_t u;
+  memcpy(&u, &f, 4);
+  return u;
+#endif
+}
+
+HDMOE_HD float hdmoe_bits_f32(uint32_t u) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  return __uint_as_float(u);
+#else
+  float f;
+  memcpy(&f, &u, 4);
+  return f;
+#endif
+}
+
+// bf16 <-> fp32. Encode is round-to-nearest-even; NaN stays NaN (quiet bit forced).
+HDMOE_HD float hdmoe_bf16_to_f32(uint16_t h) { return hdmoe_bits_f32((uint32_t)h << 16); }
+
+HDMOE_HD uint16_t hdmoe_f32_to_bf16(float f) {
+  uint32_t u = hdmoe_f32_bits(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+// fp32 value rounded to the nearest bf16 and returned as fp32.
+HDMOE_HD float hdmoe_round_bf16(float f) { return hdmoe_bf16_to_f32(hdmoe_f32_to_bf16(f)); }
+
+HDMOE_HD float hdmoe_e4m3fn_to_f32(uint8_t b) {
+  uint32_t sign = (uint32_t)(b & 0x80u) << 24;
+  uint32_t e = (b >> 3) & 0xfu;
+  uint32_t m = b & 7u;
+  if (e == 0xfu && m == 7u) return hdmoe_bits_f32(sign | 0x7fc00000u);
+  if (e == 0u) {
+    // subnormal: m * 2^-9, exact in fp32
+    float v = (float)m * 0.001953125f;
+    return hdmoe_bits_f32(hdmoe_f32_bits(v) | sign);
+  }
+  return hdmoe_bits_f32(sign | ((e + 120u) << 23) | (m << 20));
+}
+
+HDMOE_HD uint8_t hdmoe_f32_to_e4m3fn(float f) {
+  uint32_t u = hdmoe_f32_bits(f);
+  uint8_t sign = (uint8_t)((u >> 24) & 0x80u);
+  uint32_t a = u & 0x7fffffffu;
+  if (a >= 0x43f00000u) return (uint8_t)(sign | 0x7fu);  // >= 480, inf, NaN
+  if (a < 0x3c800000u) {
+    // below the smallest normal 2^-6: align the ulp to 2^-9 by adding 2^14
+    // (fp32 ulp at 2^14 is 2^-9); the hardware add performs the RNE.
+    float t = hdmoe_bits_f32(a) + 16384.0f;
+    return (uint8_t)(sign | (uint8_t)(hdmoe_f32_bits(t) - 0x46800000u));
+  }
+  a += 0x7ffffu + ((a >> 20) & 1u);  // RNE on the 20 dropped mantissa bits
+  // exponent field rebias 127 -> 7; a carry out of the mantissa bumps the exponent,
+  // and 0x7F (would-be 480) is the NaN pattern, which is the no-saturation rule.
+  return (uint8_t)(sign | (uint8_t)((a >> 20) - 0x3c0u));
+}

@@ -1,0 +1,230 @@
+"""Tensor-level wrappers over the C ABI: they check devices/dtypes/shapes, allocate
+outputs with torch (device memory and stream plumbing only) and enqueue the HIP
+kernels on torch's current stream. Nothing here computes with torch.
+"""
+import ctypes
+
+import torch
+
+from . import _lib
+from ._lib import FfnWeights, LayerArgs, LayerLayout, W_BF16, W_E4M3FN, check, lib, ptr
+
+FP8 = torch.float8_e4m3fn
+BF16 = torch.bfloat16
+
+
+def _stream(t):
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _need_hip(t, what, dtype=None):
+    if not t.is_cuda:
+        raise RuntimeError(f"{what}: tensor is on {t.device}; comfyui_amd only computes on a HIP device "
+                           "(there is no CPU path)")
+    if dtype is not None and t.dtype != dtype:
+        raise TypeError(f"{what}: expected {dtype}, got {t.dtype}")
+    if not t.is_contiguous():
+        raise ValueError(f"{what}: tensor must be contiguous")
+
+
+def weight_dtype_code(dtype):
+    if dtype == BF16:
+        return W_BF16
+    if dtype == FP8:
+        return W_E4M3FN
+    raise TypeError(f"unsupported weight dtype {dtype}: the HIP path takes bfloat16 or float8_e4m3fn weights")
+
+
+def gate_top2(x2d, gate_w):
+    """MoEGate scoring + top-2 on the device. x2d [T,D] bf16, gate_w [E,D] bf16
+    -> topk_idx int32 [T,2], topk_weight bf16 [T,2]."""
+    _need_hip(x2d, "gate_top2 x", BF16)
+    _need_hip(gate_w, "gate_top2 gate weight", BF16)
+    T, D = x2d.shape
+    E = gate_w.shape[0]
+    if gate_w.shape[1] != D:
+        raise ValueError(f"gate weight {tuple(gate_w.shape)} does not match hidden size {D}")
+    idx = torch.empty((T, 2), dtype=torch.int32, device=x2d.device)
+    w = torch.empty((T, 2), dtype=BF16, device=x2d.device)
+    check(lib.hdmoe_gate_top2(ptr(x2d), ptr(gate_w), T, D, E, ptr(idx), ptr(w), _stream(x2d)))
+    return idx, w
+
+
+def dispatch(topk_idx, E):
+    """Stable permutation of the flat slots by expert.
+    -> counts [E], offsets [E+1], perm [2T], inv_perm [2T] (int32, device)."""
+    _need_hip(topk_idx, "dispatch topk_idx", torch.int32)
+    T = topk_idx.shape[0]
+    dev = topk_idx.device
+    counts = torch.empty(E, dtype=torch.int32, device=dev)
+    offsets = torch.empty(E + 1, dtype=torch.int32, device=dev)
+    perm = torch.empty(2 * T, dtype=torch.int32, device=dev)
+    inv = torch.empty(2 * T, dtype=torch.int32, device=dev)
+    nbytes = lib.hdmoe_dispatch_workspace_bytes(T, E)
+    ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=dev)
+    check(lib.hdmoe_dispatch(ptr(topk_idx), T, E, ptr(counts), ptr(offsets), ptr(perm), ptr(inv), ptr(ws), nbytes,
+                             _stream(topk_idx)))
+    return counts, offsets, perm, inv
+
+
+def _scale_ptr(s, device, what):
+    if s is None:
+        return None
+    if s.device != device or s.dtype != torch.float32 or s.numel() != 1:
+        raise ValueError(f"{what} must be an fp32 scalar tensor on {device}")
+    return s.data_ptr()
+
+
+def quant_fp8(x, scale_input):
+    """fp8_linear's activation cast: x bf16 [..., D] -> float8_e4m3fn, same shape."""
+    _need_hip(x, "quant_fp8 x", BF16)
+    D = x.shape[-1]
+    out = torch.empty(x.shape, dtype=FP8, device=x.device)
+    check(lib.hdmoe_quant_fp8(ptr(x), x.numel() // D, D, _scale_ptr(scale_input, x.device, "scale_input"), ptr(out),
+                              _stream(x)))
+    return out
+
+
+def quant_permute_fp8(x2d, perm, offsets, scale_inputs):
+    """Gather rows by perm and quantise each with its expert's scale_input. -> [2T,D] fp8."""
+    _need_hip(x2d, "quant_permute_fp8 x", BF16)
+    T, D = x2d.shape
+    E = len(scale_inputs)
+    arr = (ctypes.c_void_p * E)(*[_scale_ptr(s, x2d.device, "scale_input") for s in scale_inputs])
+    out = torch.empty((2 * T, D), dtype=FP8, device=x2d.device)
+    check(lib.hdmoe_quant_permute_fp8(ptr(x2d), ptr(perm), ptr(offsets), T, D, E, arr, ptr(out), _stream(x2d)))
+    return out
+
+
+def permute_bf16(x2d, perm):
+    _need_hip(x2d, "permute_bf16 x", BF16)
+    T, D = x2d.shape
+    out = torch.empty((2 * T, D), dtype=BF16, device=x2d.device)
+    check(lib.hdmoe_permute_bf16(ptr(x2d), ptr(perm), T, D, ptr(out), _stream(x2d)))
+    return out
+
+
+def linear(a2d, weight, scale_weight=None, scale_input=None):
+    """a2d [rows,K] (fp8 for fp8 weights, bf16 for bf16 weights) x weight [N,K]^T -> bf16 [rows,N]."""
+    code = weight_dtype_code(weight.dtype)
+    _need_hip(a2d, "linear activations", weight.dtype)
+    _need_hip(weight, "linear weight")
+    rows, K = a2d.shape
+    N = weight.shape[0]
+    if weight.shape[1] != K:
+        raise ValueError(f"linear: activations [{rows},{K}] do not match weight {tuple(weight.shape)}")
+    out = torch.empty((rows, N), dtype=BF16, device=a2d.device)
+    check(lib.hdmoe_linear(code, ptr(a2d), rows, K, N, ptr(weight),
+                           _scale_ptr(scale_weight, a2d.device, "scale_weight"),
+                           _scale_ptr(scale_input, a2d.device, "scale_input"), ptr(out), _stream(a2d)))
+    return out
+
+
+def silu_mul(a, b):
+    _need_hip(a, "silu_mul a", BF16)
+    _need_hip(b, "silu_mul b", BF16)
+    if a.shape != b.shape:
+        raise ValueError("silu_mul: shape mismatch")
+    out = torch.empty_like(a)
+    check(lib.hdmoe_silu_mul_bf16(ptr(a), ptr(b), a.numel(), ptr(out), _stream(a)))
+    return out
+
+
+def scale_to_bf16(src, scale):
+    """bf16(bf16(src) * bf16(scale)) for src in fp8 or bf16."""
+    code = weight_dtype_code(src.dtype)
+    _need_hip(src, "scale_to_bf16 src")
+    out = torch.empty(src.shape, dtype=BF16, device=src.device)
+    check(lib.hdmoe_scale_to_bf16(code, ptr(src), src.numel(), _scale_ptr(scale, src.device, "scale"), ptr(out),
+                                  _stream(src)))
+    return out
+
+
+def combine(y_sorted, inv_perm, topk_weight, shared):
+    _need_hip(y_sorted, "combine y", BF16)
+    _need_hip(topk_weight, "combine topk_weight", BF16)
+    T = topk_weight.shape[0]
+    D = y_sorted.shape[1]
+    out = torch.empty((T, D), dtype=BF16, device=y_sorted.device)
+    check(lib.hdmoe_combine(ptr(y_sorted), ptr(inv_perm), ptr(topk_weight), ptr(shared), T, D, ptr(out),
+                            _stream(y_sorted)))
+    return out
+
+
+def make_ffn_weights(w1, w2, w3, scales=None):
+    """Fill an hdmoe_ffn_weights. scales: dict with optional fp32 scalar tensors
+    scale_w1/2/3 and scale_in1/2/3 (fp8 only)."""
+    fw = FfnWeights()
+    fw.w1, fw.w2, fw.w3 = ptr(w1), ptr(w2), ptr(w3)
+    if scales:
+        for k, v in scales.items():
+            setattr(fw, k, ptr(v))
+    return fw
+
+
+def grouped_swiglu(a, offsets, experts, H):
+    """experts: list of FfnWeights. a [2T,D] -> h [2T,H] (same element type as a)."""
+    code = weight_dtype_code(a.dtype)
+    _need_hip(a, "grouped_swiglu a")
+    rows, D = a.shape
+    E = len(experts)
+    arr = (FfnWeights * E)(*experts)
+    h = torch.empty((rows, H), dtype=a.dtype, device=a.device)
+    check(lib.hdmoe_grouped_swiglu(code, ptr(a), ptr(offsets), rows, E, D, H, arr, ptr(h), _stream(a)))
+    return h
+
+
+def grouped_down(h, offsets, experts, D):
+    code = weight_dtype_code(h.dtype)
+    _need_hip(h, "grouped_down h")
+    rows, H = h.shape
+    E = len(experts)
+    arr = (FfnWeights * E)(*experts)
+    y = torch.empty((rows, D), dtype=BF16, device=h.device)
+    check(lib.hdmoe_grouped_down(code, ptr(h), ptr(offsets), rows, E, H, D, arr, ptr(y), _stream(h)))
+    return y
+
+
+def layer_layout(T, D, H, Hs, E, code):
+    lay = LayerLayout()
+    check(lib.hdmoe_layer_layout_get(T, D, H, Hs, E, code, ctypes.byref(lay)))
+    return lay
+
+
+def moe_ffn(x2d, gate_w, experts, shared, H, Hs, weight_dtype, out=None, workspace=None, want_routing=False):
+    """The whole layer as one enqueue. experts: list of FfnWeights, shared: FfnWeights or None.
+    Returns out [T,D] bf16 (and topk_idx int32, topk_weight bf16 when want_routing)."""
+    _need_hip(x2d, "moe_ffn x", BF16)
+    _need_hip(gate_w, "moe_ffn gate weight", BF16)
+    T, D = x2d.shape
+    E = len(experts)
+    code = weight_dtype_code(weight_dtype)
+    nbytes = lib.hdmoe_layer_workspace_bytes(T, D, H, Hs if shared is not None else 0, E, code)
+    if nbytes == 0 and T > 0:
+        raise _lib.HdmoeError(_lib.lib.hdmoe_layer_layout_get(T, D, H, Hs, E, code, ctypes.byref(LayerLayout())),
+                              lib.hdmoe_last_error().decode())
+    if workspace is None or workspace.numel() < nbytes:
+        workspace = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=x2d.device)
+    if out is None:
+        out = torch.empty((T, D), dtype=BF16, device=x2d.device)
+    args = LayerArgs()
+    args.T, args.D, args.H, args.Hs, args.E, args.weight_dtype = T, D, H, (Hs if shared is not None else 0), E, code
+    args.x, args.gate_w = ptr(x2d), ptr(gate_w)
+    arr = (FfnWeights * E)(*experts)
+    args.experts = arr
+    sh = None
+    if shared is not None:
+        sh = FfnWeights.from_buffer_copy(shared)
+        args.shared = ctypes.pointer(sh)
+    args.out, args.workspace, args.workspace_bytes = ptr(out), ptr(workspace), workspace.numel()
+    idx = tw = None
+    if want_routing:
+        idx = torch.empty((T, 2), dtype=torch.int32, device=x2d.device)
+        tw = torch.empty((T, 2), dtype=BF16, device=x2d.device)
+        args.topk_idx, args.topk_weight = ptr(idx), ptr(tw)
+    check(lib.hdmoe_moe_ffn(ctypes.byref(args), _stream(x2d)))
+    # the workspace must outlive the enqueued kernels: torch's caching allocator keeps a freed block
+    # tied to the stream it was allocated on, so releasing it here is safe for work on that stream
+    if want_routing:
+        return out, idx, tw
+    return out

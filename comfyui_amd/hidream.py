@@ -1,0 +1,200 @@
+"""HiDream mixture-of-experts SwiGLU feed-forward modules with the constructor and
+forward signatures, attribute names and state-dict keys of the reference
+(/root/reference/comfy/ldm/hidream/model.py:215-325), computing on the MI355X.
+
+  FeedForwardSwiGLU      model.py:215-238   w2(silu(w1 x) * w3 x)
+  MoEGate                model.py:242-283   softmax scores, top-2 of E, not renormalised
+  MOEFeedForwardSwiGLU   model.py:287-325   gate -> dispatch -> experts -> weighted sum -> + shared
+
+State-dict keys per layer: shared_experts.{w1,w2,w3}.weight, experts.{i}.{w1,w2,w3}.weight,
+gate.weight (+ .scale_weight / .scale_input under scaled-fp8 operations) -- the names LoRA
+key maps and checkpoints address.
+
+MOEFeedForwardSwiGLU.forward enqueues the whole layer through ONE library call when all
+Linears share a supported storage dtype (bf16, or float8_e4m3fn with fp8 matrix multiply);
+otherwise it composes the same HIP stages per expert through the Linear modules, which
+needs the per-expert row counts on the host (one sync, as the reference's mask indexing).
+Inputs must be bf16 HIP tensors: there is no CPU path.
+"""
+from typing import Optional
+
+import torch
+import torch.nn as nn
+
+from . import functional as HF
+from . import ops as amd_ops
+
+FP8 = torch.float8_e4m3fn
+BF16 = torch.bfloat16
+
+
+class FeedForwardSwiGLU(nn.Module):
+    def __init__(self, dim: int, hidden_dim: int, multiple_of: int = 256,
+                 ffn_dim_multiplier: Optional[float] = None, dtype=None, device=None, operations=None):
+        super().__init__()
+        hidden_dim = int(2 * hidden_dim / 3)
+        if ffn_dim_multiplier is not None:
+            hidden_dim = int(ffn_dim_multiplier * hidden_dim)
+        hidden_dim = multiple_of * ((hidden_dim + multiple_of - 1) // multiple_of)
+        operations = operations if operations is not None else amd_ops.disable_weight_init
+        self.w1 = operations.Linear(dim, hidden_dim, bias=False, dtype=dtype, device=device)
+        self.w2 = operations.Linear(hidden_dim, dim, bias=False, dtype=dtype, device=device)
+        self.w3 = operations.Linear(dim, hidden_dim, bias=False, dtype=dtype, device=device)
+
+    def forward(self, x):
+        return self.w2(HF.silu_mul(self.w1(x), self.w3(x)))
+
+
+class MoEGate(nn.Module):
+    def __init__(self, embed_dim, num_routed_experts=4, num_activated_experts=2, aux_loss_alpha=0.01,
+                 dtype=None, device=None, operations=None):
+        super().__init__()
+        self.top_k = num_activated_experts
+        self.n_routed_experts = num_routed_experts
+        self.scoring_func = 'softmax'
+        self.alpha = aux_loss_alpha
+        self.seq_aux = False
+        self.norm_topk_prob = False
+        self.gating_dim = embed_dim
+        self.weight = nn.Parameter(torch.empty((self.n_routed_experts, self.gating_dim), dtype=dtype, device=device))
+        self.reset_parameters()
+
+    def reset_parameters(self) -> None:
+        pass
+
+    def _check(self):
+        if self.scoring_func != 'softmax':
+            raise NotImplementedError(f'insupportable scoring function for MoE gating: {self.scoring_func}')
+        if self.top_k != 2 or self.norm_topk_prob:
+            raise NotImplementedError("the HIP gate kernel selects the top 2 experts without renormalisation")
+
+    def device_weight(self, hidden_states):
+        """The gate weight in the activations' dtype on their device (model.py:268 routes it through
+        cast_to because a bare Parameter may have been left on the offload device)."""
+        return amd_ops.cast_to(self.weight, dtype=hidden_states.dtype, device=hidden_states.device).contiguous()
+
+    def forward(self, hidden_states):
+        self._check()
+        bsz, seq_len, h = hidden_states.shape
+        x2 = hidden_states.reshape(-1, h).contiguous()
+        idx, w = HF.gate_top2(x2, self.device_weight(x2))
+        return idx.to(torch.int64), w, None
+
+
+def _plain(lin):
+    return len(lin.weight_function) == 0 and len(lin.bias_function) == 0 and lin.bias is None
+
+
+class MOEFeedForwardSwiGLU(nn.Module):
+    def __init__(self, dim: int, hidden_dim: int, num_routed_experts: int, num_activated_experts: int,
+                 dtype=None, device=None, operations=None):
+        super().__init__()
+        self.shared_experts = FeedForwardSwiGLU(dim, hidden_dim // 2, dtype=dtype, device=device, operations=operations)
+        self.experts = nn.ModuleList([FeedForwardSwiGLU(dim, hidden_dim, dtype=dtype, device=device, operations=operations)
+                                      for i in range(num_routed_experts)])
+        self.gate = MoEGate(embed_dim=dim, num_routed_experts=num_routed_experts,
+                            num_activated_experts=num_activated_experts, dtype=dtype, device=device,
+                            operations=operations)
+        self.num_activated_experts = num_activated_experts
+        self._scale_cache = {}
+
+    # ---- fused path ----------------------------------------------------------------
+
+    def _scale_value(self, p):
+        """Host copy of an fp32 scalar Parameter, cached on (identity, version): read once per
+        parameter object, so steady-state forwards do not synchronise."""
+        key = (id(p), p._version, p.data_ptr())
+        v = self._scale_cache.get(key)
+        if v is None:
+            if len(self._scale_cache) > 256:
+                self._scale_cache.clear()
+            v = float(p.detach().float().cpu())
+            self._scale_cache[key] = v
+        return v
+
+    def _collect(self, x):
+        """Device pointers of all 15 Linears for the one-call path, or None when the layer
+        needs the per-Linear composition. Returned tensors are kept alive by the caller."""
+        ffns = list(self.experts) + [self.shared_experts]
+        lins = [l for f in ffns for l in (f.w1, f.w2, f.w3)]
+        for l in lins:
+            if not isinstance(l, amd_ops.disable_weight_init.Linear) or l.bias is not None or len(l.bias_function) > 0:
+                return None
+        wdt = lins[0].weight.dtype
+        if wdt not in (BF16, FP8) or any(l.weight.dtype != wdt for l in lins):
+            return None
+        fp8 = wdt == FP8
+        if fp8 and not all(getattr(l, "hdmoe_fp8_matrix_mult", isinstance(l, amd_ops.fp8_ops.Linear)) for l in lins):
+            return None  # scaled fp8 without fp8 matrix multiply: dequantising Linear path
+        dev = x.device
+        keep = []
+        packed = []
+        one = None
+        for f in ffns:
+            scales = {}
+            ws = []
+            for name, l in (("1", f.w1), ("2", f.w2), ("3", f.w3)):
+                if _plain(l) and l.weight.device == dev:
+                    w = l.weight
+                else:
+                    w, _ = amd_ops.cast_bias_weight(l, x, dtype=wdt)
+                w = w.contiguous()
+                keep.append(w)
+                ws.append(w)
+                if fp8:
+                    sw = getattr(l, "scale_weight", None)
+                    if sw is None:
+                        one = one if one is not None else amd_ops._one(dev)
+                        sw = one
+                    sw = sw.to(dev)
+                    si = getattr(l, "scale_input", None)
+                    if si is not None:
+                        si = si.to(dev)
+                        keep.append(si)
+                    keep.append(sw)
+                    scales["scale_w" + name] = sw
+                    scales["scale_in" + name] = si
+            if fp8:
+                s1, s3 = scales["scale_in1"], scales["scale_in3"]
+                if (s1 is None) != (s3 is None):
+                    return None
+                if s1 is not None and s1.data_ptr() != s3.data_ptr() and self._scale_value(s1) != self._scale_value(s3):
+                    return None  # w1 and w3 quantise the same input differently: cannot share one fp8 copy
+            packed.append(HF.make_ffn_weights(ws[0], ws[1], ws[2], scales))
+        return wdt, packed[:-1], packed[-1], keep
+
+    def forward(self, x):
+        if x.dtype != BF16 or not x.is_cuda:
+            raise RuntimeError(f"MOEFeedForwardSwiGLU: expected a bfloat16 HIP tensor, got {x.dtype} on {x.device}; "
+                               "comfyui_amd has no CPU path")
+        self.gate._check()
+        orig_shape = x.shape
+        x2 = x.reshape(-1, orig_shape[-1]).contiguous()
+        gate_w = self.gate.device_weight(x2)
+        got = self._collect(x2)
+        if got is not None:
+            wdt, experts, shared, keep = got
+            H = self.experts[0].w1.weight.shape[0]
+            Hs = self.shared_experts.w1.weight.shape[0]
+            y = HF.moe_ffn(x2, gate_w, experts, shared, H, Hs, wdt)
+            del keep
+            return y.view(*orig_shape)
+        return self._forward_composed(x2, gate_w).view(*orig_shape)
+
+    # ---- composed path -----------------------------------------------------------------
+
+    def _forward_composed(self, x2, gate_w):
+        """Same stages, one expert at a time through the Linear modules (weight functions,
+        offloaded or mixed-dtype weights, dequantising scaled-fp8 Linears)."""
+        E = len(self.experts)
+        idx, w = HF.gate_top2(x2, gate_w)
+        counts, offsets, perm, inv_perm = HF.dispatch(idx, E)
+        xs = HF.permute_bf16(x2, perm)
+        y = torch.empty_like(xs)
+        bounds = offsets.tolist()  # host sync: segment sizes steer the per-expert calls
+        for i, expert in enumerate(self.experts):
+            lo, hi = bounds[i], bounds[i + 1]
+            if hi > lo:
+                y[lo:hi] = expert(xs[lo:hi])
+        shared = self.shared_experts(x2)
+        return HF.combine(y, inv_perm, w, shared)

@@ -1,0 +1,193 @@
+/*
+ * libhdmoe -- C ABI of the MI355X (gfx950) implementation of the HiDream
+ * mixture-of-experts SwiGLU feed-forward.
+ *
+ * The reference (ComfyUI v0.3.64, all Python) has no FFI for this path; what each
+ * entry point replaces is the torch call sequence at the cited reference lines
+ * (paths relative to the reference root).
+ *
+ * Conventions
+ *   - every pointer named *_dev / documented "device" is HIP device memory owned by
+ *     the caller; "host array" means an ordinary host pointer to E entries that is
+ *     only read during the call;
+ *   - all matrices are row-major and contiguous; weights are [out_features, in_features]
+ *     exactly as torch.nn.Linear stores them;
+ *   - `stream` is a hipStream_t passed as void*; kernels are enqueued on it and the
+ *     call returns without synchronising; nothing is allocated and no global state
+ *     is mutated, so calls on different streams may overlap;
+ *   - return value 0 = enqueued; negative = HDMOE_E_* and nothing was enqueued;
+ *     hdmoe_last_error() gives a thread-local message for the last failure;
+ *   - scale pointers (float*, device) address the fp32 scalar Parameters
+ *     `scale_weight` / `scale_input` of a scaled-fp8 Linear (comfy/ops.py:388-397);
+ *     a NULL scale_input means "Parameter is None": the input is clamped to +-448
+ *     and cast, with scale 1 (comfy/ops.py:337-340). The caller's input is never
+ *     modified (the reference clamps it in place).
+ */
+#ifndef HDMOE_H
+#define HDMOE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define HDMOE_VERSION 100
+
+#define HDMOE_OK 0
+#define HDMOE_E_NULL (-1)      /* required pointer is NULL */
+#define HDMOE_E_SHAPE (-2)     /* unsupported or inconsistent sizes */
+#define HDMOE_E_WORKSPACE (-3) /* workspace too small or misaligned */
+#define HDMOE_E_LAUNCH (-4)    /* HIP reported a launch error */
+
+#define HDMOE_MAX_EXPERTS 16
+#define HDMOE_TOPK 2
+
+/* weight storage of the Linear layers */
+#define HDMOE_W_BF16 0
+#define HDMOE_W_E4M3FN 1
+
+typedef void* hdmoe_stream_t;
+
+int hdmoe_version(void);
+const char* hdmoe_last_error(void);
+
+/* ---- stage entry points ------------------------------------------------------ */
+
+/* MoEGate.forward, comfy/ldm/hidream/model.py:263-283 (F.linear :268, softmax :270,
+ * topk k=2 :275, no renormalisation :253). x [T,D] bf16, gate_w [E,D] bf16.
+ * Writes topk_idx [T,2] int32 and topk_weight [T,2] bf16; slot 0 holds the larger
+ * score, equal scores go to the lower expert index. Logits and scores are rounded
+ * to bf16 between the three steps as the three torch kernels do.
+ * D % 8 == 0, E in {2,4,8,16}. */
+int hdmoe_gate_top2(const void* x_bf16, const void* gate_w_bf16, int T, int D, int E,
+                    int32_t* topk_idx, void* topk_weight_bf16, hdmoe_stream_t stream);
+
+/* Token dispatch, comfy/ldm/hidream/model.py:313-318: the boolean-mask gathers
+ * `x[flat_topk_idx == i]` for i = 0..E-1 select flat slots p = 2t+s in ascending p,
+ * i.e. a stable sort of the flat expert ids. Writes counts [E], offsets [E+1]
+ * (exclusive scan), perm [2T] (sorted row -> flat slot) and inv_perm [2T]
+ * (flat slot -> sorted row), all int32 device arrays.
+ * workspace: hdmoe_dispatch_workspace_bytes(T, E) bytes, 256-byte aligned. */
+size_t hdmoe_dispatch_workspace_bytes(int T, int E);
+int hdmoe_dispatch(const int32_t* topk_idx, int T, int E, int32_t* counts, int32_t* offsets,
+                   int32_t* perm, int32_t* inv_perm, void* workspace, size_t workspace_bytes,
+                   hdmoe_stream_t stream);
+
+/* Activation quantisation of fp8_linear, comfy/ops.py:337-343:
+ * out = e4m3fn( bf16( x * bf16(1/scale_input) ) ), no saturation (|v| > 464 -> NaN);
+ * scale_input == NULL: out = e4m3fn(clamp(x, -448, 448)).
+ * x [rows,D] bf16 -> out [rows,D] bytes. D % 8 == 0. */
+int hdmoe_quant_fp8(const void* x_bf16, int64_t rows, int D, const float* scale_input_dev,
+                    void* out_fp8, hdmoe_stream_t stream);
+
+/* Same quantisation fused with the gather of model.py:315,318: sorted row r takes
+ * token perm[r] / 2 and the scale_input of the expert whose segment
+ * [offsets[e], offsets[e+1]) holds r. scale_input: host array of E device pointers
+ * (entries may be NULL). a_fp8 [2T,D]. */
+int hdmoe_quant_permute_fp8(const void* x_bf16, const int32_t* perm, const int32_t* offsets,
+                            int T, int D, int E, const float* const* scale_input,
+                            void* a_fp8, hdmoe_stream_t stream);
+
+/* bf16 gather of model.py:315,318 for bf16 weights: a[r] = x[perm[r] / 2]. */
+int hdmoe_permute_bf16(const void* x_bf16, const int32_t* perm, int T, int D, void* a_bf16,
+                       hdmoe_stream_t stream);
+
+/* One group of rows of a grouped GEMM: an expert (or the shared expert). */
+typedef struct hdmoe_ffn_weights {
+  const void* w1; /* [H,D] */
+  const void* w2; /* [D,H] */
+  const void* w3; /* [H,D] */
+  /* fp8 only (ignored for bf16 weights): device fp32 scalars */
+  const float* scale_w1;
+  const float* scale_w2;
+  const float* scale_w3;
+  const float* scale_in1; /* scale_input of w1; must describe the same value as scale_in3 */
+  const float* scale_in2; /* scale_input of w2 */
+  const float* scale_in3;
+} hdmoe_ffn_weights;
+
+/* First half of FeedForwardSwiGLU.forward (model.py:238) for every expert at once:
+ *   h[r] = quant2( bf16(silu(bf16(w1 a[r]))) * bf16(w3 a[r]) )       r in expert e's segment
+ * with each Linear evaluated as fp8_linear (ops.py:345-348: fp32 accumulation of
+ * fp8 x fp8 products, times scale_in*scale_w, rounded to bf16), and quant2 the
+ * activation quantisation of the following w2 Linear (scale_in2), so h is e4m3fn.
+ * For bf16 weights every Linear is bf16 x bf16 with fp32 accumulation and h is bf16.
+ * a [rows_total,D] (e4m3fn or bf16, rows sorted by expert), offsets [E+1] device,
+ * h [rows_total,H]. D % 128 == 0 (fp8) or D % 64 == 0 (bf16); H % 128 == 0. */
+int hdmoe_grouped_swiglu(int weight_dtype, const void* a, const int32_t* offsets, int rows_total,
+                         int E, int D, int H, const hdmoe_ffn_weights* experts, void* h,
+                         hdmoe_stream_t stream);
+
+/* Second half: y[r] = bf16(w2 h[r]) per expert segment. h [rows_total,H], y [rows_total,D] bf16.
+ * H % 128 == 0 (fp8) or H % 64 == 0 (bf16); D % 256 == 0. */
+int hdmoe_grouped_down(int weight_dtype, const void* h, const int32_t* offsets, int rows_total,
+                       int E, int H, int D, const hdmoe_ffn_weights* experts, void* y_bf16,
+                       hdmoe_stream_t stream);
+
+/* One Linear without bias on already-prepared activations:
+ *   fp8:  out = bf16( (a_fp8 . w_fp8^T) * scale_in * scale_w )   (fp8_linear, ops.py:345-348;
+ *         scale_in NULL = 1)
+ *   bf16: out = bf16( a_bf16 . w_bf16^T )                        (Linear, ops.py:107-115)
+ * a [rows,K], w [N,K], out [rows,N] bf16. K % 128 == 0 (fp8) / K % 64 == 0 (bf16); N % 256 == 0. */
+int hdmoe_linear(int weight_dtype, const void* a, int rows, int K, int N, const void* w,
+                 const float* scale_w_dev, const float* scale_in_dev, void* out_bf16,
+                 hdmoe_stream_t stream);
+
+/* Elementwise middle of model.py:238 for the unfused path: out = bf16(bf16(silu(a)) * b). */
+int hdmoe_silu_mul_bf16(const void* a_bf16, const void* b_bf16, int64_t n, void* out_bf16,
+                        hdmoe_stream_t stream);
+
+/* `weight * scale_weight` or `input * scale_weight` of the scaled-fp8 Linear WITHOUT fp8
+ * matmul (comfy/ops.py:407-410), after the operand was cast to bf16:
+ *   out = bf16( bf16(src) * bf16(scale) ).   src: n elements of e4m3fn or bf16, n % 8 == 0. */
+int hdmoe_scale_to_bf16(int src_dtype, const void* src, int64_t n, const float* scale_dev,
+                        void* out_bf16, hdmoe_stream_t stream);
+
+/* Weighted combine, model.py:319-324:
+ *   out[t] = bf16( bf16( bf16(y[r0]*w[t,0]) + bf16(y[r1]*w[t,1]) ) + shared[t] ),  r_s = inv_perm[2t+s]
+ * y_sorted [2T,D] bf16, topk_weight [T,2] bf16, shared [T,D] bf16 or NULL, out [T,D] bf16.
+ * Deterministic (a gather, no atomics). D % 8 == 0. */
+int hdmoe_combine(const void* y_sorted_bf16, const int32_t* inv_perm, const void* topk_weight_bf16,
+                  const void* shared_bf16, int T, int D, void* out_bf16, hdmoe_stream_t stream);
+
+/* ---- whole layer -------------------------------------------------------------- */
+
+/* MOEFeedForwardSwiGLU.forward, model.py:307-325, as one call that enqueues
+ * gate -> dispatch -> quantise/permute -> grouped gate/up GEMM with SiLU*mul ->
+ * grouped down GEMM -> combine (+ shared expert through the same GEMMs). */
+typedef struct hdmoe_layer_args {
+  int T;            /* tokens (batch * sequence) */
+  int D;            /* model width, 2560 for HiDream */
+  int H;            /* routed expert hidden width */
+  int Hs;           /* shared expert hidden width (0 = no shared expert) */
+  int E;            /* routed experts */
+  int weight_dtype; /* HDMOE_W_BF16 or HDMOE_W_E4M3FN */
+  const void* x;            /* [T,D] bf16 device */
+  const void* gate_w;       /* [E,D] bf16 device */
+  const hdmoe_ffn_weights* experts; /* host array [E] */
+  const hdmoe_ffn_weights* shared;  /* host pointer or NULL */
+  void* out;                /* [T,D] bf16 device */
+  void* workspace;          /* hdmoe_layer_workspace_bytes(...) bytes, 256-byte aligned, device */
+  size_t workspace_bytes;
+  /* optional device outputs (may be NULL): routing decision and permutation */
+  int32_t* topk_idx;  /* [T,2] */
+  void* topk_weight;  /* [T,2] bf16 */
+} hdmoe_layer_args;
+
+size_t hdmoe_layer_workspace_bytes(int T, int D, int H, int Hs, int E, int weight_dtype);
+int hdmoe_moe_ffn(const hdmoe_layer_args* args, hdmoe_stream_t stream);
+
+/* Where the pieces of the workspace live, for tests that inspect intermediates. */
+typedef struct hdmoe_layer_layout {
+  size_t topk_idx, topk_weight, counts, offsets, perm, inv_perm, dispatch_ws;
+  size_t a, h, y, total;
+} hdmoe_layer_layout;
+int hdmoe_layer_layout_get(int T, int D, int H, int Hs, int E, int weight_dtype,
+                           hdmoe_layer_layout* out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HDMOE_H */

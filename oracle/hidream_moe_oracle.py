@@ -1,0 +1,252 @@
+"""TEST INFRASTRUCTURE ONLY -- CPU oracle for the HiDream MoE SwiGLU feed-forward.
+
+Only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg may import
+this module; nothing under comfyui_amd/ does.
+
+It restates, with torch CPU tensors as the array library (the reference itself is
+torch code; torch 2.10.0 is what this image carries, requirements.txt:4 leaves it
+unpinned), the dataflow of these reference functions (paths under /root/reference):
+
+  comfy/ldm/hidream/model.py:237-238   FeedForwardSwiGLU.forward      -> ffn_swiglu
+  comfy/ldm/hidream/model.py:263-283   MoEGate.forward                -> gate_torch / gate_fixed_order
+  comfy/ldm/hidream/model.py:307-325   MOEFeedForwardSwiGLU.forward   -> moe_forward
+  comfy/ops.py:103-115, 283-284        (manual_cast) Linear           -> Linear mode "plain"
+  comfy/ops.py:399-410                 scaled_fp8 Linear, upcast path -> Linear mode "upcast"
+  comfy/ops.py:314-358                 fp8_linear                     -> Linear mode "fp8mm"
+
+The reference has no golden vectors, known-answer tests or fixtures for any of
+these (its tests never touch comfy.ops or hidream), so every function is pinned by
+tests/test_oracle_*.py against closed forms, brute force on tiny inputs, dense
+(every expert on every token) evaluation, invariants, and torch library routines.
+
+Top-2 selection: the reference calls torch.topk(sorted=False), whose tie choice is
+an implementation detail of torch; the contract here is "larger score first, ties
+to the lower expert index", i.e. the first two entries of a stable descending sort.
+"""
+import ctypes
+import os
+
+import numpy as np
+import torch
+import torch.nn.functional as F
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB = None
+
+
+def _lib():
+    """The C part of the oracle (moe_ref.c), built by `make -C oracle`."""
+    global _LIB
+    if _LIB is None:
+        path = os.path.join(_HERE, "libhdmoe_oracle.so")
+        if not os.path.exists(path):
+            raise RuntimeError(f"{path} missing: run `make -C oracle` (or __graft_entry__.build())")
+        lib = ctypes.CDLL(path)
+        lib.ref_gate_top2.restype = ctypes.c_int
+        lib.ref_dispatch.restype = ctypes.c_int
+        lib.ref_combine.restype = None
+        lib.ref_e4m3fn_encode.restype = None
+        lib.ref_e4m3fn_decode_table.restype = None
+        _LIB = lib
+    return _LIB
+
+
+def _p(t):
+    return ctypes.c_void_p(t.data_ptr())
+
+
+# --------------------------------------------------------------------------- fp8
+
+def e4m3fn_decode_table():
+    out = torch.empty(256, dtype=torch.float32)
+    _lib().ref_e4m3fn_decode_table(_p(out))
+    return out
+
+
+def e4m3fn_encode(x_f32):
+    """fp32 -> e4m3fn bytes (uint8): RNE, |v|>464 -> NaN (ops.py:340,343 `.to(dtype)`)."""
+    x = x_f32.detach().to(torch.float32).contiguous()
+    out = torch.empty(x.shape, dtype=torch.uint8)
+    _lib().ref_e4m3fn_encode(_p(x), _p(out), ctypes.c_int64(x.numel()))
+    return out
+
+
+def e4m3fn_decode(b_u8):
+    return e4m3fn_decode_table()[b_u8.long()]
+
+
+def quantize_weight_per_tensor(w_f32):
+    """BASELINE.json configs[1]: scale_weight = amax/448, W8 = (W/scale_weight) -> e4m3fn.
+    Returns (W8 as torch.float8_e4m3fn, scale_weight fp32 scalar tensor)."""
+    w = w_f32.to(torch.float32)
+    s = (w.abs().amax() / 448.0).to(torch.float32)
+    w8 = (w / s).to(torch.float8_e4m3fn)
+    return w8, s
+
+
+# -------------------------------------------------------------------------- gate
+
+def top2_lowest_index(scores):
+    """First two columns of a stable descending sort: larger score first, ties -> lower index."""
+    order = torch.sort(scores.float(), dim=-1, descending=True, stable=True).indices
+    idx = order[:, :2].contiguous()
+    return idx, torch.gather(scores, 1, idx)
+
+
+def gate_torch(x2d, wg):
+    """model.py:267-275 with torch's own kernels at x's dtype (bf16 or fp32):
+    F.linear -> softmax -> top-2. Returns idx int64 [T,2], weight [T,2], logits, scores."""
+    logits = F.linear(x2d, wg.to(x2d.dtype), None)
+    scores = logits.softmax(dim=-1)
+    idx, w = top2_lowest_index(scores)
+    return idx, w, logits, scores
+
+
+def gate_fixed_order(x2d_bf16, wg_bf16):
+    """Same computation with the one fixed fp32 summation order and exp() of moe_ref.c
+    (what the HIP gate kernel is compared with bit for bit).
+    Returns idx int32 [T,2], weight bf16 [T,2], logits bf16 [T,E], scores bf16 [T,E]."""
+    x = x2d_bf16.contiguous()
+    wg = wg_bf16.contiguous()
+    assert x.dtype == torch.bfloat16 and wg.dtype == torch.bfloat16
+    T, D = x.shape
+    E = wg.shape[0]
+    idx = torch.empty((T, 2), dtype=torch.int32)
+    w = torch.empty((T, 2), dtype=torch.bfloat16)
+    logits = torch.empty((T, E), dtype=torch.bfloat16)
+    scores = torch.empty((T, E), dtype=torch.bfloat16)
+    rc = _lib().ref_gate_top2(_p(x), _p(wg), T, D, E, _p(idx), _p(w), _p(logits), _p(scores))
+    if rc != 0:
+        raise ValueError("ref_gate_top2: bad arguments")
+    return idx, w, logits, scores
+
+
+# ---------------------------------------------------------------------- dispatch
+
+def dispatch(topk_idx, E):
+    """Stable counting sort of the flat expert ids (model.py:313-318).
+    Returns counts[E], offsets[E+1], perm[2T], inv_perm[2T] (int32)."""
+    flat = topk_idx.reshape(-1).to(torch.int32).contiguous()
+    n = flat.numel()
+    counts = torch.empty(E, dtype=torch.int32)
+    offsets = torch.empty(E + 1, dtype=torch.int32)
+    perm = torch.empty(n, dtype=torch.int32)
+    inv = torch.empty(n, dtype=torch.int32)
+    rc = _lib().ref_dispatch(_p(flat), ctypes.c_int64(n), E, _p(counts), _p(offsets), _p(perm), _p(inv))
+    if rc != 0:
+        raise ValueError("ref_dispatch: expert id out of range")
+    return counts, offsets, perm, inv
+
+
+def combine_c(y_sorted_bf16, inv_perm, w_bf16, shared_bf16):
+    """C restatement of model.py:319,324 at bf16 (see moe_ref.c ref_combine)."""
+    T = w_bf16.shape[0]
+    D = y_sorted_bf16.shape[1]
+    out = torch.empty((T, D), dtype=torch.bfloat16)
+    _lib().ref_combine(_p(y_sorted_bf16.contiguous()), _p(inv_perm.contiguous()), _p(w_bf16.contiguous()),
+                       _p(shared_bf16.contiguous()) if shared_bf16 is not None else None, T, D, _p(out))
+    return out
+
+
+# ------------------------------------------------------------------------ linear
+
+class LinearParams:
+    """One reference Linear without bias: weight [out,in] (bf16/fp32, or float8_e4m3fn with
+    scale_weight and optional scale_input fp32 scalars, ops.py:388-397)."""
+
+    def __init__(self, weight, scale_weight=None, scale_input=None):
+        self.weight = weight
+        self.scale_weight = scale_weight
+        self.scale_input = scale_input
+
+
+def linear(x, p, mode):
+    """mode "plain":  F.linear at x.dtype with the weight cast to x.dtype (ops.py:107-109).
+    mode "upcast": scaled-fp8 Linear without fp8 matmul (ops.py:405-410).
+    mode "fp8mm":  fp8_linear (ops.py:314-358): quantise x (x * (1/scale_input).to(x.dtype) -> e4m3fn,
+                   or clamp +-448 when scale_input is None), fp8 x fp8 products accumulated in fp32,
+                   times scale_input*scale_weight, rounded to x.dtype. Products of two e4m3 values are
+                   exact in fp32, so an fp32 matmul of the decoded operands is the same contraction."""
+    if mode == "plain":
+        return F.linear(x, p.weight.to(x.dtype), None)
+    if mode == "upcast":
+        w = p.weight.to(x.dtype)
+        s = p.scale_weight.to(x.dtype)
+        if w.numel() < x.numel():
+            return F.linear(x, w * s, None)
+        return F.linear(x * s, w, None)
+    if mode == "fp8mm":
+        assert p.weight.dtype == torch.float8_e4m3fn
+        if p.scale_input is None:
+            s_in = torch.ones((), dtype=torch.float32)
+            xq = torch.clamp(x, min=-448, max=448).to(torch.float8_e4m3fn)
+        else:
+            s_in = p.scale_input.to(torch.float32)
+            xq = (x * (1.0 / s_in).to(x.dtype)).to(torch.float8_e4m3fn)
+        acc = xq.to(torch.float32) @ p.weight.to(torch.float32).t()
+        return (acc * (s_in * p.scale_weight.to(torch.float32))).to(x.dtype)
+    raise ValueError(mode)
+
+
+def ffn_swiglu(x, ffn, mode):
+    """model.py:238: w2(silu(w1 x) * w3 x); every op rounds to x.dtype as torch does."""
+    w1, w2, w3 = ffn
+    return linear(F.silu(linear(x, w1, mode)) * linear(x, w3, mode), w2, mode)
+
+
+# ------------------------------------------------------------------------- layer
+
+def moe_forward(x, params, mode, gate_result=None):
+    """model.py:307-325, literally: gate, repeat_interleave, boolean-mask gather per expert,
+    weighted sum over the K slots, plus the shared expert.
+    params: dict(gate=Wg [E,D], experts=[(w1,w2,w3)]*E, shared=(w1,w2,w3)) of LinearParams.
+    gate_result: optional (topk_idx, topk_weight) to reuse a routing decision (e.g. the GPU's)."""
+    wtype = x.dtype
+    orig_shape = x.shape
+    x2 = x.reshape(-1, x.shape[-1])
+    if gate_result is None:
+        topk_idx, topk_weight, _, _ = gate_torch(x2, params["gate"])
+    else:
+        topk_idx, topk_weight = gate_result
+        topk_idx = topk_idx.long()
+        topk_weight = topk_weight.to(wtype)
+    K = topk_idx.shape[1]
+    flat = topk_idx.reshape(-1)
+    xr = x2.repeat_interleave(K, dim=0)
+    y = torch.zeros_like(xr)
+    for i, ffn in enumerate(params["experts"]):
+        m = flat == i
+        if bool(m.any()):
+            y[m] = ffn_swiglu(xr[m], ffn, mode).to(wtype)
+    y = (y.view(*topk_weight.shape, -1) * topk_weight.unsqueeze(-1)).sum(dim=1)
+    y = y.view(*orig_shape).to(wtype)
+    return y + ffn_swiglu(x, params["shared"], mode)
+
+
+def moe_forward_dense(x, params, mode, topk_idx, topk_weight):
+    """Brute force used to pin moe_forward: run EVERY expert on EVERY token and pick by mask.
+    Same rounding points as moe_forward (slot products rounded, then summed)."""
+    x2 = x.reshape(-1, x.shape[-1])
+    outs = torch.stack([ffn_swiglu(x2, ffn, mode) for ffn in params["experts"]], dim=0)  # [E,T,D]
+    T = x2.shape[0]
+    sel = outs[topk_idx.long().t(), torch.arange(T).unsqueeze(0)]  # [K,T,D]
+    y = (sel.permute(1, 0, 2) * topk_weight.to(x.dtype).unsqueeze(-1)).sum(dim=1)
+    y = y.view(x.shape).to(x.dtype)
+    return y + ffn_swiglu(x, params["shared"], mode)
+
+
+def error_metrics(got, ref):
+    """rms(err)/rms(ref), max|err|/rms(ref), max|err|/max|ref| in fp64."""
+    g = got.double().reshape(-1)
+    r = ref.double().reshape(-1)
+    err = (g - r).abs()
+    rms_ref = float(r.pow(2).mean().sqrt())
+    return {
+        "rel_rms": float(err.pow(2).mean().sqrt()) / rms_ref,
+        "max_over_rms": float(err.max()) / rms_ref,
+        "max_over_max": float(err.max()) / float(r.abs().max()),
+    }
+
+
+def to_numpy_u16(t_bf16):
+    return t_bf16.view(torch.int16).numpy().view(np.uint16)

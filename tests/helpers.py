@@ -1,0 +1,30 @@
+"""Shared by the parity tests: small synthetic layers and oracle parameter packing."""
+import torch
+
+from comfyui_amd import synth
+from oracle import hidream_moe_oracle as O
+
+
+def oracle_params(state_dict, num_experts):
+    """state dict (bf16 or scaled fp8) -> oracle params dict of LinearParams."""
+    def lin(prefix):
+        return O.LinearParams(state_dict[prefix + ".weight"], state_dict.get(prefix + ".scale_weight"),
+                              state_dict.get(prefix + ".scale_input"))
+
+    def ffn(prefix):
+        return (lin(prefix + "w1"), lin(prefix + "w2"), lin(prefix + "w3"))
+
+    return dict(gate=state_dict["gate.weight"], experts=[ffn(f"experts.{e}.") for e in range(num_experts)],
+                shared=ffn("shared_experts."))
+
+
+def small_layer(seed, dim, tokens, weights, num_experts=4, hidden_arg=None, scale_in=None, batch=1):
+    """A small layer: returns (state_dict on CPU, x bf16 [batch, tokens/batch, dim])."""
+    master, g = synth.make_weights(seed, dim=dim, hidden_arg=hidden_arg, num_experts=num_experts)
+    sd = synth.to_state_dict(master, weights)
+    if scale_in is not None:
+        for k in list(sd):
+            if k.endswith("scale_input"):
+                sd[k] = torch.tensor(float(scale_in[k] if isinstance(scale_in, dict) else scale_in), dtype=torch.float32)
+    x = synth.make_input(g, tokens, dim=dim, batch=batch)
+    return sd, x

@@ -1,0 +1,134 @@
+"""GPU parity of the whole MoE feed-forward (module forward -> hdmoe_moe_ffn) against the CPU oracle.
+
+Gates (fp8 weights tolerance 3e-2, bf16 weights 1e-2, from the task statement):
+  * routing (top-2 indices, bf16 weights) and permutation: bit-exact against the fixed-order oracle;
+  * output vs the oracle that follows the reference's bf16 dataflow with the same quantisation points:
+    rms(err)/rms(ref) <= TOL_RMS and max|err|/max|ref| <= tol;
+  * output vs the same dataflow evaluated with fp32 intermediates (no bf16 rounding between ops):
+    rms(err)/rms(ref) <= tol.
+max|err|/rms(ref) is reported, not gated: rounding the output itself to bf16 already costs up to
+2^-8 * |y|, i.e. 1.6e-2 * rms at |y| = 4 rms.
+"""
+import pytest
+import torch
+
+from comfyui_amd import synth
+from oracle import hidream_moe_oracle as O
+from tests.helpers import oracle_params, small_layer
+
+pytestmark = pytest.mark.gpu
+BF16 = torch.bfloat16
+TOL = {"fp8": 3e-2, "bf16": 1e-2}
+TOL_RMS_SAME_DATAFLOW = {"fp8": 1e-2, "bf16": 4e-3}
+
+
+def run_gpu(sd, x, weights, dev, dim, hidden_arg=None, num_experts=4, **kw):
+    from comfyui_amd import functional as HF
+    m = synth.build_module({k: v.to(dev) for k, v in sd.items()}, weights, dev, dim=dim, hidden_arg=hidden_arg,
+                           num_experts=num_experts, **kw)
+    xd = x.to(dev)
+    y = m(xd)
+    idx, w = HF.gate_top2(xd.reshape(-1, dim), m.gate.weight.to(BF16))
+    torch.cuda.synchronize()
+    return y.cpu(), idx.cpu(), w.cpu(), m
+
+
+def check_layer(sd, x, weights, y, idx, w, num_experts, token_subset=None):
+    dim = x.shape[-1]
+    x2 = x.reshape(-1, dim)
+    # routing: bit-exact
+    idx_ref, w_ref, _, _ = O.gate_fixed_order(x2, sd["gate.weight"])
+    assert torch.equal(idx, idx_ref), "routing indices differ"
+    assert torch.equal(w.view(torch.int16), w_ref.view(torch.int16)), "routing weights differ"
+    params = oracle_params(sd, num_experts)
+    mode = "fp8mm" if weights == "fp8" else "plain"
+    sel = torch.arange(x2.shape[0]) if token_subset is None else token_subset
+    xs = x2[sel].unsqueeze(0)
+    got = y.reshape(-1, dim)[sel].unsqueeze(0)
+    ref_same = O.moe_forward(xs, params, mode, gate_result=(idx[sel], w[sel]))
+    ref_f32 = O.moe_forward(xs.float(), params, mode, gate_result=(idx[sel], w[sel].float()))
+    m_same = O.error_metrics(got, ref_same)
+    m_f32 = O.error_metrics(got, ref_f32)
+    print(f"\n[{weights}] T={x2.shape[0]} vs bf16-dataflow oracle {m_same}\n        vs fp32-intermediate oracle {m_f32}")
+    assert not bool(got.float().isnan().any())
+    assert m_same["rel_rms"] <= TOL_RMS_SAME_DATAFLOW[weights], m_same
+    assert m_same["max_over_max"] <= TOL[weights], m_same
+    assert m_f32["rel_rms"] <= TOL[weights], m_f32
+    assert m_f32["max_over_max"] <= TOL[weights], m_f32
+    return m_same, m_f32
+
+
+@pytest.mark.parametrize("weights", ["fp8", "bf16"])
+@pytest.mark.parametrize("dim,tokens,batch", [(256, 64, 1), (512, 700, 2), (256, 1, 1), (1024, 513, 1)])
+def test_small_layers(dev, weights, dim, tokens, batch):
+    sd, x = small_layer(seed=dim + tokens, dim=dim, tokens=tokens, weights=weights, batch=batch)
+    y, idx, w, _ = run_gpu(sd, x, weights, dev, dim)
+    assert y.shape == x.shape and y.dtype == BF16
+    check_layer(sd, x, weights, y, idx, w, 4)
+
+
+def test_fp8_nontrivial_scale_inputs(dev):
+    # per-Linear scale_input values: w1/w3 of an expert share one, experts differ
+    dim = 512
+    sd, x = small_layer(seed=9, dim=dim, tokens=300, weights="fp8")
+    vals = {}
+    for k in sd:
+        if k.endswith("scale_input"):
+            ffn = k.rsplit(".", 2)[0]
+            lin = k.split(".")[-2]
+            h = sum(ord(c) for c in ffn)
+            base = 0.05 + 0.01 * (h % 7)
+            vals[k] = base if lin in ("w1", "w3") else 0.002 * (1 + h % 3)
+    for k, v in vals.items():
+        sd[k] = torch.tensor(v, dtype=torch.float32)
+    y, idx, w, _ = run_gpu(sd, x, "fp8", dev, dim)
+    check_layer(sd, x, "fp8", y, idx, w, 4)
+
+
+def test_fp8_no_scale_input_uses_clamp_rule(dev):
+    dim = 256
+    sd, x = small_layer(seed=4, dim=dim, tokens=200, weights="fp8")
+    sd = {k: v for k, v in sd.items() if not k.endswith("scale_input")}
+    y, idx, w, m = run_gpu(sd, x, "fp8", dev, dim, scale_input=False)
+    assert m.experts[0].w1.scale_input is None
+    check_layer(sd, x, "fp8", y, idx, w, 4)
+
+
+def test_composed_path_matches_fused(dev):
+    # a weight_function on one Linear forces nothing special in the fused path (it goes through
+    # cast_bias_weight); mixed dtypes force the per-expert composition
+    dim = 256
+    sd, x = small_layer(seed=21, dim=dim, tokens=150, weights="fp8")
+    y, idx, w, m = run_gpu(sd, x, "fp8", dev, dim)
+    xd = x.to(dev)
+    gate_w = m.gate.device_weight(xd.reshape(-1, dim))
+    y2 = m._forward_composed(xd.reshape(-1, dim).contiguous(), gate_w).view(x.shape).cpu()
+    diff = O.error_metrics(y2, y)
+    print("composed vs fused", diff)
+    assert diff["rel_rms"] < 2e-3
+
+
+@pytest.mark.parametrize("name,subset", [("cfg1", 256), ("cfg2", 192), ("cfg3", 192), ("cfg5-256", 256), ("cfg5-4096", 192)])
+def test_benchmark_configs(dev, name, subset):
+    cfg = synth.make_config(name)
+    weights = cfg["weights"]
+    sd = synth.to_state_dict(cfg["master"], weights)
+    x = cfg["x"]
+    y, idx, w, _ = run_gpu(sd, x, weights, dev, synth.DIM)
+    T = x.shape[0] * x.shape[1]
+    g = torch.Generator().manual_seed(1)
+    sel = torch.randperm(T, generator=g)[:subset].sort().values
+    if name.startswith("cfg5"):
+        sel = torch.unique(torch.cat([sel, torch.arange(0, T, 64)[:32]]))  # include exact-tie tokens
+        counts = torch.bincount(idx.reshape(-1).long(), minlength=4).float() / T
+        print("expert share of tokens", counts.tolist())
+        assert counts[0] > 0.6 and counts[3] < 0.02
+        ties = idx[::64]
+        assert bool(((ties[:, 0] == 0) & (ties[:, 1] == 1)).all()), "exact tie must go to the lower index"
+    check_layer(sd, x, weights, y, idx, w, 4, token_subset=sel)
+    # permutation invariants at full size
+    counts_r, offs_r, perm_r, inv_r = O.dispatch(idx, 4)
+    from comfyui_amd import functional as HF
+    got = HF.dispatch(idx.to(dev), 4)
+    for a, b in zip(got, (counts_r, offs_r, perm_r, inv_r)):
+        assert torch.equal(a.cpu(), b)
