@@ -1,0 +1,224 @@
+#!/usr/bin/env python3
+"""Benchmark of the HiDream MoE SwiGLU feed-forward layer on one MI355X.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg3|cfg2|cfg1] [--no-cpu-baseline]
+
+A step is one forward of comfyui_amd.hidream.MOEFeedForwardSwiGLU (gate, dispatch, quantise,
+grouped fp8 GEMMs, combine, shared expert) over one synthetic batch that is already resident in
+HBM. The default workload is the headline configuration: 8192 tokens (2 x 4096), fp8 e4m3fn
+weights with per-tensor scales, activations N(0,1) with 1 % of the channels scaled by 20.
+
+Prints ONE JSON line. `value` is tokens/s over the K timed steps. `roofline` describes the
+dominant kernel (the grouped gate/up GEMM with the SiLU*mul epilogue): its algorithmic FLOP per
+launch divided by its average duration, measured with HIP events recorded on the launch stream
+around that kernel inside the timed steps. `cpu_baseline` is the CPU oracle's restatement of the
+reference's `--cpu` dataflow (fp32 compute, fp8 weights dequantised per call) timed on this
+host's cores over a bounded sample of the same batch.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_FP8_TFLOPS = 5000.0    # MI355X dense fp8 MFMA
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
+PEAK_HBM_GBPS = 8000.0      # MI355X HBM3E
+
+
+class HipEvents:
+    """hipEvent_t handles through the HIP runtime that torch already loaded; they can be recorded
+    from inside the library on the stream the kernels are launched on."""
+
+    def __init__(self):
+        self.hip = ctypes.CDLL("libamdhip64.so")
+        self.hip.hipEventCreate.argtypes = [ctypes.POINTER(ctypes.c_void_p)]
+        self.hip.hipEventElapsedTime.argtypes = [ctypes.POINTER(ctypes.c_float), ctypes.c_void_p, ctypes.c_void_p]
+        self.hip.hipEventSynchronize.argtypes = [ctypes.c_void_p]
+        self.hip.hipEventDestroy.argtypes = [ctypes.c_void_p]
+
+    def create(self, n):
+        out = []
+        for _ in range(n):
+            e = ctypes.c_void_p()
+            rc = self.hip.hipEventCreate(ctypes.byref(e))
+            if rc != 0:
+                raise RuntimeError(f"hipEventCreate failed: {rc}")
+            out.append(e.value)
+        return out
+
+    def elapsed_ms(self, a, b):
+        ms = ctypes.c_float()
+        self.hip.hipEventSynchronize(b)
+        rc = self.hip.hipEventElapsedTime(ctypes.byref(ms), a, b)
+        if rc != 0:
+            raise RuntimeError(f"hipEventElapsedTime failed: {rc}")
+        return ms.value
+
+    def destroy(self, evs):
+        for e in evs:
+            self.hip.hipEventDestroy(e)
+
+
+def flops_per_token(D, H, Hs, E, K=2):
+    gate_up = K * 2 * 2 * D * H + 2 * 2 * D * Hs
+    down = K * 2 * D * H + 2 * D * Hs
+    return dict(gate=2 * D * E, gate_up=gate_up, down=down, total=gate_up + down + 2 * D * E)
+
+
+def cpu_baseline(cfg, sd, sample_tokens):
+    """The oracle's restatement of the reference's --cpu path on a bounded sample."""
+    from oracle import hidream_moe_oracle as O
+    params = O.oracle_params(sd, 4)
+    mode = "upcast" if cfg["weights"] == "fp8" else "plain"
+    x2 = cfg["x"].reshape(-1, cfg["x"].shape[-1]).float()  # --cpu computes in fp32
+    gate = params["gate"].float()
+    params = dict(params, gate=gate)
+    if mode == "plain":
+        for ffn in params["experts"] + [params["shared"]]:
+            for lp in ffn:
+                lp.weight = lp.weight.float()   # --cpu upcasts bf16 checkpoints once at load
+    xs = x2[:sample_tokens].unsqueeze(0).contiguous()
+    O.moe_forward(x2[:32].unsqueeze(0).contiguous(), params, mode)  # warm caches / thread pool
+    reps, dt = 0, 0.0
+    t0 = time.perf_counter()
+    while reps < 10 and dt < 10.0:   # about 10 s of CPU work, at most 10 forwards
+        O.moe_forward(xs, params, mode)
+        reps += 1
+        dt = time.perf_counter() - t0
+    return dict(value=reps * sample_tokens / dt, unit="tokens/s", cores=torch.get_num_threads(), kind="port",
+                sample=f"{reps} forward(s) over the first {sample_tokens} tokens of the same batch through the oracle's "
+                       f"restatement of the reference --cpu dataflow (fp32 compute, mode={mode}, fp8 weights dequantised "
+                       f"per call), {dt:.2f} s, torch CPU threads={torch.get_num_threads()}, os.cpu_count()={os.cpu_count()}")
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="cfg3", choices=["cfg1", "cfg2", "cfg3"])
+    ap.add_argument("--cpu-sample-tokens", type=int, default=8192)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on exactly one GPU (one MI355X holds the whole layer; tokens are "
+              "independent, so more GPUs would only replicate it). Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no HIP device visible", file=sys.stderr)
+        sys.exit(1)
+
+    from comfyui_amd import synth
+    from comfyui_amd._lib import STAGE_NAMES
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    cfg = synth.make_config(args.workload)
+    sd = synth.to_state_dict(cfg["master"], cfg["weights"])
+    cfg["master"] = None
+    module = synth.build_module({k: v.to(dev) for k, v in sd.items()}, cfg["weights"], dev)
+    x = cfg["x"].to(dev)
+    B, S, D = x.shape
+    T = B * S
+    H, Hs, E = synth.H_ROUTED, synth.H_SHARED, synth.NUM_EXPERTS
+    fl = flops_per_token(D, H, Hs, E)
+
+    hip = HipEvents()
+    with torch.no_grad():
+        for _ in range(args.warmup):
+            y = module(x)
+        torch.cuda.synchronize()
+        # K timed steps; every step also records the per-stage events on the launch stream
+        ev_sets = [hip.create(len(STAGE_NAMES) + 1) for _ in range(args.steps)]
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for k in range(args.steps):
+            y = module(x, stage_events=ev_sets[k])
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+    if bool(torch.isnan(y.float()).any()):
+        print("bench.py: output contains NaN", file=sys.stderr)
+        sys.exit(1)
+
+    sec = (t1 - t0) / args.steps
+    stage_ms = {n: 0.0 for n in STAGE_NAMES}
+    for evs in ev_sets:
+        for i, n in enumerate(STAGE_NAMES):
+            stage_ms[n] += hip.elapsed_ms(evs[i], evs[i + 1])
+    for n in stage_ms:
+        stage_ms[n] /= args.steps
+    for evs in ev_sets:
+        hip.destroy(evs)
+
+    fp8 = cfg["weights"] == "fp8"
+    peak = PEAK_FP8_TFLOPS if fp8 else PEAK_BF16_TFLOPS
+    tokens_per_s = T / sec
+    tflops = tokens_per_s * fl["total"] / 1e12
+    gemm1_tflops = T * fl["gate_up"] / (stage_ms["gemm_gate_up"] * 1e-3) / 1e12
+    gemm2_tflops = T * fl["down"] / (stage_ms["gemm_down"] * 1e-3) / 1e12
+    eb = 1 if fp8 else 2
+    gate_bytes = T * D * 2 + E * D * 2 + T * 2 * (4 + 2)
+    # dispatch as built: index sort (read 2T ids twice, write perm + inv_perm) plus the materialised permuted
+    # activation copy for the routed experts and the token-order copy for the shared expert
+    dispatch_bytes = 2 * (2 * T * 4) + 2 * (2 * T * 4) + (2 * T * D * 2 + 2 * T * D * eb) + (T * D * 2 + T * D * eb if fp8 else 0)
+    gd_ms = stage_ms["gate"] + stage_ms["dispatch"] + stage_ms["quant_permute"]
+    combine_bytes = 2 * T * D * 2 + T * D * 2 + T * D * 2 + T * 2 * 2 + 2 * T * 4
+
+    out = {
+        "metric": "MoE-FFN tokens/sec at 8192 tok fp8" if args.workload == "cfg3" else f"MoE-FFN tokens/sec ({args.workload})",
+        "value": tokens_per_s,
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": sec * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "fp8" if fp8 else "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": {"cfg1": "cfg1: 1x1024 tokens, bf16 weights",
+                         "cfg2": "cfg2: 1x4096 tokens, scaled fp8 e4m3fn weights, scale_input 1.0",
+                         "cfg3": "cfg3 (headline): 2x4096 = 8192 tokens x 2560, scaled fp8 e4m3fn weights "
+                                 "(scale_weight = amax/448, scale_input = 1.0), bf16 gate, x ~ N(0,1) with 1% "
+                                 "outlier channels x20, 4 routed experts (hidden 6912) top-2 + shared expert (hidden 3584)"}[args.workload],
+            "tokens": T, "dim": D, "hidden_routed": H, "hidden_shared": Hs, "experts": E, "top_k": 2,
+        },
+        "tflops": tflops,
+        "pct_of_mfma_peak": 100.0 * tflops / peak,
+        "flop_per_token": fl["total"],
+        "gate_dispatch_GBps": (gate_bytes + dispatch_bytes) / (gd_ms * 1e-3) / 1e9,
+        "gate_dispatch_bytes": gate_bytes + dispatch_bytes,
+        "combine_GBps": combine_bytes / (stage_ms["combine"] * 1e-3) / 1e9,
+        "stage_ms": stage_ms,
+        "gemm_down_tflops": gemm2_tflops,
+        "roofline": {
+            "kernel": "grouped_gemm_kernel<FP8_SWIGLU>" if fp8 else "grouped_gemm_kernel<BF16_SWIGLU>",
+            "bound": "mfma",
+            "achieved": gemm1_tflops,
+            "peak": peak,
+            "unit": "TFLOP/s",
+            "frac": gemm1_tflops / peak,
+            "traffic": None,
+            "flop_per_launch": T * fl["gate_up"],
+            "avg_launch_ms": stage_ms["gemm_gate_up"],
+        },
+    }
+    if not args.no_cpu_baseline:
+        del module
+        torch.cuda.empty_cache()
+        out["cpu_baseline"] = cpu_baseline(cfg, sd, min(args.cpu_sample_tokens, T))
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

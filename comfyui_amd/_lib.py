@@ -6,6 +6,10 @@ of this module raises, there is no fallback.
 import ctypes
 import os
 
+# torch must be imported before the library is loaded: libhdmoe.so depends on libamdhip64 by soname,
+# and the process must end up with the ONE HIP runtime torch brings, not a second copy.
+import torch  # noqa: F401
+
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libhdmoe.so")
 
@@ -14,6 +18,8 @@ W_E4M3FN = 1
 MAX_EXPERTS = 16
 E_NULL, E_SHAPE, E_WORKSPACE, E_LAUNCH = -1, -2, -3, -4
 TOPK = 2
+NUM_STAGES = 6
+STAGE_NAMES = ("gate", "dispatch", "quant_permute", "gemm_gate_up", "gemm_down", "combine")
 
 c_void_p = ctypes.c_void_p
 c_int = ctypes.c_int
@@ -38,6 +44,7 @@ class LayerArgs(ctypes.Structure):
         ("experts", ctypes.POINTER(FfnWeights)), ("shared", ctypes.POINTER(FfnWeights)),
         ("out", c_void_p), ("workspace", c_void_p), ("workspace_bytes", c_size_t),
         ("topk_idx", c_void_p), ("topk_weight", c_void_p),
+        ("stage_events", ctypes.POINTER(c_void_p)),
     ]
 
 

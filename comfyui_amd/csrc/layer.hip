@@ -99,10 +99,18 @@ extern "C" int hdmoe_moe_ffn(const hdmoe_layer_args* p, hdmoe_stream_t stream) {
       return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_moe_ffn: expert %d: w1 and w3 disagree on having a scale_input", e);
   }
 
+  int ev = 0;
+  auto mark = [&]() {
+    if (p->stage_events) hipEventRecord(static_cast<hipEvent_t>(p->stage_events[ev]), s);
+    ++ev;
+  };
+  mark();
   if (int rc = hdmoe_gate_top2(p->x, p->gate_w, T, D, E, idx, tw, stream)) return rc;
+  mark();
   if (int rc = hdmoe_dispatch(idx, T, E, counts, offsets, perm, inv_perm, ws + l.dispatch_ws,
                               hdmoe_dispatch_workspace_bytes(T, E), stream))
     return rc;
+  mark();
 
   const uint8_t* a_static = nullptr;
   if (fp8) {
@@ -118,13 +126,18 @@ extern "C" int hdmoe_moe_ffn(const hdmoe_layer_args* p, hdmoe_stream_t stream) {
     a_static = static_cast<const uint8_t*>(p->x);
   }
 
+  mark();
   // gate/up projections + SiLU*mul, routed experts and shared expert in one launch
   if (int rc = hdmoe_launch_ffn_gemm(true, wd, a_routed, offsets, (int)n, E, p->experts, h_routed, a_static,
                                      Hs > 0 ? T : 0, p->shared, h_shared, D, H, D, Hs, s, "hdmoe_moe_ffn (gate/up)"))
     return rc;
+  mark();
   // down projections, both in one launch
   if (int rc = hdmoe_launch_ffn_gemm(false, wd, h_routed, offsets, (int)n, E, p->experts, y_routed, h_shared,
                                      Hs > 0 ? T : 0, p->shared, y_shared, H, D, Hs, D, s, "hdmoe_moe_ffn (down)"))
     return rc;
-  return hdmoe_combine(y_routed, inv_perm, tw, Hs > 0 ? y_shared : nullptr, T, D, p->out, stream);
+  mark();
+  const int rc = hdmoe_combine(y_routed, inv_perm, tw, Hs > 0 ? y_shared : nullptr, T, D, p->out, stream);
+  mark();
+  return rc;
 }

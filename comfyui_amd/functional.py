@@ -191,7 +191,8 @@ def layer_layout(T, D, H, Hs, E, code):
     return lay
 
 
-def moe_ffn(x2d, gate_w, experts, shared, H, Hs, weight_dtype, out=None, workspace=None, want_routing=False):
+def moe_ffn(x2d, gate_w, experts, shared, H, Hs, weight_dtype, out=None, workspace=None, want_routing=False,
+            stage_events=None):
     """The whole layer as one enqueue. experts: list of FfnWeights, shared: FfnWeights or None.
     Returns out [T,D] bf16 (and topk_idx int32, topk_weight bf16 when want_routing)."""
     _need_hip(x2d, "moe_ffn x", BF16)
@@ -222,6 +223,10 @@ def moe_ffn(x2d, gate_w, experts, shared, H, Hs, weight_dtype, out=None, workspa
         idx = torch.empty((T, 2), dtype=torch.int32, device=x2d.device)
         tw = torch.empty((T, 2), dtype=BF16, device=x2d.device)
         args.topk_idx, args.topk_weight = ptr(idx), ptr(tw)
+    if stage_events is not None:
+        # sequence of NUM_STAGES + 1 hipEvent_t handles (ints) created by the caller
+        ev = (ctypes.c_void_p * (_lib.NUM_STAGES + 1))(*stage_events)
+        args.stage_events = ev
     check(lib.hdmoe_moe_ffn(ctypes.byref(args), _stream(x2d)))
     # the workspace must outlive the enqueued kernels: torch's caching allocator keeps a freed block
     # tied to the stream it was allocated on, so releasing it here is safe for work on that stream

@@ -163,7 +163,9 @@ class MOEFeedForwardSwiGLU(nn.Module):
             packed.append(HF.make_ffn_weights(ws[0], ws[1], ws[2], scales))
         return wdt, packed[:-1], packed[-1], keep
 
-    def forward(self, x):
+    def forward(self, x, stage_events=None):
+        """x [B,S,dim] -> [B,S,dim]. `stage_events` (optional, not in the reference signature) is a
+        sequence of 7 hipEvent_t handles recorded around the six stages of the one-call path."""
         if x.dtype != BF16 or not x.is_cuda:
             raise RuntimeError(f"MOEFeedForwardSwiGLU: expected a bfloat16 HIP tensor, got {x.dtype} on {x.device}; "
                                "comfyui_amd has no CPU path")
@@ -176,7 +178,7 @@ class MOEFeedForwardSwiGLU(nn.Module):
             wdt, experts, shared, keep = got
             H = self.experts[0].w1.weight.shape[0]
             Hs = self.shared_experts.w1.weight.shape[0]
-            y = HF.moe_ffn(x2, gate_w, experts, shared, H, Hs, wdt)
+            y = HF.moe_ffn(x2, gate_w, experts, shared, H, Hs, wdt, stage_events=stage_events)
             del keep
             return y.view(*orig_shape)
         return self._forward_composed(x2, gate_w).view(*orig_shape)

@@ -98,7 +98,7 @@ def make_config(name, seed=0):
     raise ValueError(name)
 
 
-def apply_routing_skew(master, x, bias=(2.2, 0.0, 0.0, -3.0), tie_every=64):
+def apply_routing_skew(master, x, bias=(0.1875, 0.0, 0.0, -3.0), tie_every=64):
     """Routing-skew stress: the reference gate has no bias (model.py:268), so a bias is realised
     through the existing signature -- channel 0 of x is the constant 1 and Wg[e,0] = bias[e].
     Every `tie_every`-th token is zero except channel 0, so its logits are exactly the biases and

@@ -171,10 +171,17 @@ typedef struct hdmoe_layer_args {
   void* out;                /* [T,D] bf16 device */
   void* workspace;          /* hdmoe_layer_workspace_bytes(...) bytes, 256-byte aligned, device */
   size_t workspace_bytes;
-  /* optional device outputs (may be NULL): routing decision and permutation */
+  /* optional device outputs (may be NULL): routing decision */
   int32_t* topk_idx;  /* [T,2] */
   void* topk_weight;  /* [T,2] bf16 */
+  /* optional timing hook (may be NULL): HDMOE_NUM_STAGE_EVENTS hipEvent_t created by the caller.
+   * Event i is recorded on `stream` before stage i and event i+1 after it; stages in order:
+   * gate, dispatch, quantise/permute, gate-up GEMM, down GEMM, combine. */
+  void** stage_events;
 } hdmoe_layer_args;
+
+#define HDMOE_NUM_STAGES 6
+#define HDMOE_NUM_STAGE_EVENTS (HDMOE_NUM_STAGES + 1)
 
 size_t hdmoe_layer_workspace_bytes(int T, int D, int H, int Hs, int E, int weight_dtype);
 int hdmoe_moe_ffn(const hdmoe_layer_args* args, hdmoe_stream_t stream);

@@ -160,6 +160,19 @@ class LinearParams:
         self.scale_input = scale_input
 
 
+def oracle_params(state_dict, num_experts):
+    """Module state dict (bf16, or scaled fp8 with .scale_weight/.scale_input) -> params for moe_forward."""
+    def lin(prefix):
+        return LinearParams(state_dict[prefix + ".weight"], state_dict.get(prefix + ".scale_weight"),
+                            state_dict.get(prefix + ".scale_input"))
+
+    def ffn(prefix):
+        return (lin(prefix + "w1"), lin(prefix + "w2"), lin(prefix + "w3"))
+
+    return dict(gate=state_dict["gate.weight"], experts=[ffn(f"experts.{e}.") for e in range(num_experts)],
+                shared=ffn("shared_experts."))
+
+
 def linear(x, p, mode):
     """mode "plain":  F.linear at x.dtype with the weight cast to x.dtype (ops.py:107-109).
     mode "upcast": scaled-fp8 Linear without fp8 matmul (ops.py:405-410).

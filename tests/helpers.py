@@ -5,17 +5,7 @@ from comfyui_amd import synth
 from oracle import hidream_moe_oracle as O
 
 
-def oracle_params(state_dict, num_experts):
-    """state dict (bf16 or scaled fp8) -> oracle params dict of LinearParams."""
-    def lin(prefix):
-        return O.LinearParams(state_dict[prefix + ".weight"], state_dict.get(prefix + ".scale_weight"),
-                              state_dict.get(prefix + ".scale_input"))
-
-    def ffn(prefix):
-        return (lin(prefix + "w1"), lin(prefix + "w2"), lin(prefix + "w3"))
-
-    return dict(gate=state_dict["gate.weight"], experts=[ffn(f"experts.{e}.") for e in range(num_experts)],
-                shared=ffn("shared_experts."))
+oracle_params = O.oracle_params
 
 
 def small_layer(seed, dim, tokens, weights, num_experts=4, hidden_arg=None, scale_in=None, batch=1):

