@@ -17,21 +17,18 @@ struct ScalePtrs {
 
 __device__ __forceinline__ float bf16_lo(uint32_t u) { return __uint_as_float(u << 16); }
 __device__ __forceinline__ float bf16_hi(uint32_t u) { return __uint_as_float(u & 0xffff0000u); }
-__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
-  return (uint32_t)hdmoe_f32_to_bf16(lo) | ((uint32_t)hdmoe_f32_to_bf16(hi) << 16);
-}
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) { return hdmoe_dev_pack_bf16(lo, hi); }
+__device__ __forceinline__ float round_bf16(float f) { return hdmoe_dev_round_bf16(f); }
 
 // fp8_linear's activation cast (/root/reference/comfy/ops.py:337-343).
 // inv < 0 selects the scale_input-is-None rule (clamp to +-448, scale 1).
-__device__ __forceinline__ uint32_t quant1(float v, float inv) {
-  float y;
-  if (inv < 0.0f) y = v < -448.0f ? -448.0f : (v > 448.0f ? 448.0f : v);
-  else y = hdmoe_round_bf16(v * inv);  // bf16 tensor times bf16 scalar, rounded to bf16
-  return hdmoe_f32_to_e4m3fn(y);
+__device__ __forceinline__ float quant_pre(float v, float inv) {
+  if (inv < 0.0f) return v < -448.0f ? -448.0f : (v > 448.0f ? 448.0f : v);
+  return round_bf16(v * inv);  // bf16 tensor times bf16 scalar, rounded to bf16
 }
 
 __device__ __forceinline__ uint32_t quant2x(uint32_t u, float inv) {
-  return quant1(bf16_lo(u), inv) | (quant1(bf16_hi(u), inv) << 8);
+  return hdmoe_dev_pack_e4m3fn(quant_pre(bf16_lo(u), inv), quant_pre(bf16_hi(u), inv));
 }
 
 __device__ __forceinline__ uint2 quant8(const uint4& v, float inv) {
@@ -44,7 +41,7 @@ __device__ __forceinline__ uint2 quant8(const uint4& v, float inv) {
 // (1.0 / scale_input).to(bfloat16) as fp32; NULL pointer -> clamp rule marker
 __device__ __forceinline__ float inv_scale(const float* s) {
   if (s == nullptr) return -1.0f;
-  return hdmoe_round_bf16(__fdiv_rn(1.0f, *s));
+  return round_bf16(__fdiv_rn(1.0f, *s));
 }
 
 __global__ __launch_bounds__(THREADS) void quant_rows_kernel(const uint4* __restrict__ x, long rows, int row16,
@@ -87,7 +84,7 @@ __global__ __launch_bounds__(THREADS) void permute_rows_kernel(const uint4* __re
 
 // bf16( bf16(silu(a)) * b ); silu evaluated in fp32 as a / (1 + exp(-a))
 __device__ __forceinline__ float silu_mul1(float a, float b) {
-  const float s = hdmoe_round_bf16(a / (1.0f + __expf(-a)));
+  const float s = round_bf16(a * __builtin_amdgcn_rcpf(1.0f + __expf(-a)));
   return s * b;
 }
 
@@ -110,7 +107,7 @@ __global__ __launch_bounds__(THREADS) void silu_mul_kernel(const uint4* __restri
 // bf16, the two-term sum is formed in fp32 and rounded, then the shared row is added
 // and the result rounded again.
 __device__ __forceinline__ float comb1(float y0, float y1, float w0, float w1, float sh, bool has_shared) {
-  float s = hdmoe_round_bf16(hdmoe_round_bf16(y0 * w0) + hdmoe_round_bf16(y1 * w1));
+  float s = round_bf16(round_bf16(y0 * w0) + round_bf16(y1 * w1));
   return has_shared ? s + sh : s;
 }
 
@@ -151,7 +148,7 @@ __global__ __launch_bounds__(THREADS) void combine_kernel(const uint4* __restric
 // whose operands have already been cast to the compute dtype.
 __global__ __launch_bounds__(THREADS) void scale_fp8_to_bf16_kernel(const uint2* __restrict__ src, long n8,
                                                                     const float* scale, uint4* __restrict__ out) {
-  const float sc = hdmoe_round_bf16(*scale);
+  const float sc = round_bf16(*scale);
   const long stride = (long)gridDim.x * THREADS;
   for (long i = (long)blockIdx.x * THREADS + threadIdx.x; i < n8; i += stride) {
     const uint2 v = src[i];
@@ -167,7 +164,7 @@ __global__ __launch_bounds__(THREADS) void scale_fp8_to_bf16_kernel(const uint2*
 
 __global__ __launch_bounds__(THREADS) void scale_bf16_kernel(const uint4* __restrict__ src, long n8, const float* scale,
                                                              uint4* __restrict__ out) {
-  const float sc = hdmoe_round_bf16(*scale);
+  const float sc = round_bf16(*scale);
   const long stride = (long)gridDim.x * THREADS;
   for (long i = (long)blockIdx.x * THREADS + threadIdx.x; i < n8; i += stride) {
     const uint4 v = src[i];

@@ -251,7 +251,7 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
     if constexpr (FP8) {
       sg = s_in * *gg.sb0;
       su = s_in * *gg.sb1;
-      inv_next = gg.s_next ? hdmoe_round_bf16(__fdiv_rn(1.0f, *gg.s_next)) : -1.0f;
+      inv_next = gg.s_next ? hdmoe_dev_round_bf16(__fdiv_rn(1.0f, *gg.s_next)) : -1.0f;
     }
     const int ldo = gg.n_out * (FP8 ? 1 : 2);
 #pragma unroll
@@ -264,27 +264,25 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
           float m[4];
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            const float h1 = hdmoe_round_bf16(acc[0][tt][q * 4 + i] * sg);  // w1(x) as a bf16 tensor
-            const float h3 = hdmoe_round_bf16(acc[1][tt][q * 4 + i] * su);  // w3(x)
-            const float sl = hdmoe_round_bf16(h1 / (1.0f + __expf(-h1)));   // silu(.)
-            m[i] = hdmoe_round_bf16(sl * h3);                               // silu(.) * w3(x)
+            const float h1 = hdmoe_dev_round_bf16(acc[0][tt][q * 4 + i] * sg);  // w1(x) as a bf16 tensor
+            const float h3 = hdmoe_dev_round_bf16(acc[1][tt][q * 4 + i] * su);  // w3(x)
+            const float sl = hdmoe_dev_round_bf16(h1 * __builtin_amdgcn_rcpf(1.0f + __expf(-h1)));  // silu(.)
+            m[i] = hdmoe_dev_round_bf16(sl * h3);                               // silu(.) * w3(x)
           }
           const int feat = n0 + feat_lane + q * 8;
           if constexpr (FP8) {
             // activation cast of the w2 Linear (ops.py:337-343)
-            uint32_t pk = 0;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-              float y;
-              if (inv_next < 0.0f) y = m[i] < -448.0f ? -448.0f : (m[i] > 448.0f ? 448.0f : m[i]);
-              else y = hdmoe_round_bf16(m[i] * inv_next);
-              pk |= (uint32_t)hdmoe_f32_to_e4m3fn(y) << (8 * i);
+              if (inv_next < 0.0f) m[i] = m[i] < -448.0f ? -448.0f : (m[i] > 448.0f ? 448.0f : m[i]);
+              else m[i] = hdmoe_dev_round_bf16(m[i] * inv_next);
             }
+            const uint32_t pk = hdmoe_dev_pack_e4m3fn(m[0], m[1]) | (hdmoe_dev_pack_e4m3fn(m[2], m[3]) << 16);
             *reinterpret_cast<uint32_t*>(orow + feat) = pk;
           } else {
             uint2 pk;
-            pk.x = (uint32_t)hdmoe_f32_to_bf16(m[0]) | ((uint32_t)hdmoe_f32_to_bf16(m[1]) << 16);
-            pk.y = (uint32_t)hdmoe_f32_to_bf16(m[2]) | ((uint32_t)hdmoe_f32_to_bf16(m[3]) << 16);
+            pk.x = hdmoe_dev_pack_bf16(m[0], m[1]);
+            pk.y = hdmoe_dev_pack_bf16(m[2], m[3]);
             *reinterpret_cast<uint2*>(orow + (size_t)feat * 2) = pk;
           }
         }
@@ -305,10 +303,8 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
           for (int q = 0; q < 4; ++q) {
             const int feat = n0 + ft * 128 + feat_lane + q * 8;
             uint2 pk;
-            pk.x = (uint32_t)hdmoe_f32_to_bf16(acc[ft][tt][q * 4 + 0] * sc) |
-                   ((uint32_t)hdmoe_f32_to_bf16(acc[ft][tt][q * 4 + 1] * sc) << 16);
-            pk.y = (uint32_t)hdmoe_f32_to_bf16(acc[ft][tt][q * 4 + 2] * sc) |
-                   ((uint32_t)hdmoe_f32_to_bf16(acc[ft][tt][q * 4 + 3] * sc) << 16);
+            pk.x = hdmoe_dev_pack_bf16(acc[ft][tt][q * 4 + 0] * sc, acc[ft][tt][q * 4 + 1] * sc);
+            pk.y = hdmoe_dev_pack_bf16(acc[ft][tt][q * 4 + 2] * sc, acc[ft][tt][q * 4 + 3] * sc);
             *reinterpret_cast<uint2*>(orow + (size_t)feat * 2) = pk;
           }
         }

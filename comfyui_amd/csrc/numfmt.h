@@ -80,3 +80,33 @@ HDMOE_HD uint8_t hdmoe_f32_to_e4m3fn(float f) {
   // and 0x7F (would-be 480) is the NaN pattern, which is the no-saturation rule.
   return (uint8_t)(sign | (uint8_t)((a >> 20) - 0x3c0u));
 }
+
+#if defined(__HIPCC__)
+// ---- device-only fast paths on the gfx950 conversion instructions --------------------
+// v_cvt_pk_bf16_f32 rounds to nearest even; v_cvt_pk_fp8_f32 converts two fp32 values to
+// OCP e4m3fn. Both are checked bit for bit against the integer versions above by the GPU
+// tests (every bf16 input pattern for the fp8 cast, torch's own bf16 arithmetic for the
+// bf16 rounding).
+typedef __bf16 hdmoe_bf16x2 __attribute__((ext_vector_type(2)));
+typedef float hdmoe_f32x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ uint32_t hdmoe_dev_pack_bf16(float lo, float hi) {
+  hdmoe_f32x2 v = {lo, hi};
+  hdmoe_bf16x2 b = __builtin_convertvector(v, hdmoe_bf16x2);
+  return *reinterpret_cast<uint32_t*>(&b);
+}
+
+__device__ __forceinline__ float hdmoe_dev_round_bf16(float f) {
+  return __uint_as_float(hdmoe_dev_pack_bf16(f, 0.0f) << 16);
+}
+
+// e4m3fn bytes of (a, b) in the low 16 bits. Values past the rounding midpoint above 448
+// must become NaN (0x7F); the explicit compare makes that rule independent of the wave's
+// overflow-clamp mode bit.
+__device__ __forceinline__ uint32_t hdmoe_dev_pack_e4m3fn(float a, float b) {
+  uint32_t p = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false) & 0xffffu;
+  if (__builtin_fabsf(a) > 464.0f) p = (p & 0xff80u) | 0x7fu;
+  if (__builtin_fabsf(b) > 464.0f) p = (p & 0x80ffu) | 0x7f00u;
+  return p;
+}
+#endif

@@ -175,6 +175,8 @@ def test_silu_mul(dev):
     b = torch.randn((64, 1024), generator=g).to(BF16)
     got = _hf().silu_mul(a.to(dev), b.to(dev)).cpu()
     want = torch.nn.functional.silu(a) * b
+    # silu uses the hardware reciprocal (1 ulp of fp32), so the bf16 rounding of silu(a) can land on the
+    # neighbouring value when it sits on a rounding boundary; after the product that is at most 2 bf16 ulps
     diff = (got.float() - want.float()).abs()
-    assert bool((diff <= want.float().abs() * 2 ** -7 + 1e-30).all())
+    assert bool((diff <= want.float().abs() * 2 ** -6 + 1e-30).all())
     assert float((got.view(torch.int16) != want.view(torch.int16)).float().mean()) < 0.01
