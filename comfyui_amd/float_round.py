@@ -18,16 +18,21 @@ _FORMATS = {
 
 def _round_slice(x, dtype, generator):
     mant_bits, bias = _FORMATS[dtype]
+    exp_max = (1 << (8 - 1 - mant_bits)) - 1
     xh = x.half()
     mag = xh.abs()
-    # exponent of the fp8 binade that holds |x| (subnormals share the lowest one)
-    expo = torch.floor(torch.log2(mag)).clamp(min=1 - bias, max=(1 << (8 - 1 - mant_bits)) - 1 - bias)
-    expo = torch.where(mag == 0, torch.full_like(expo, 1 - bias), expo)
-    ulp = torch.exp2(expo - mant_bits)
-    steps = mag / ulp
-    steps = torch.floor(steps + torch.rand(steps.size(), dtype=steps.dtype, layout=steps.layout,
-                                           device=steps.device, generator=generator))
-    out = torch.sign(xh) * steps * ulp
+    # biased exponent of the fp8 binade holding |x|; 0 marks the subnormal binade
+    biased = (torch.floor(torch.log2(mag)) + bias).clamp(min=0, max=exp_max)
+    normal = biased != 0
+    # position inside the binade in units of one fp8 step, in [0, 2^mant_bits); the noise is added at this
+    # scale, in float16, as the reference does
+    pos = torch.where(normal,
+                      (mag / torch.exp2(biased - bias) - 1.0) * (1 << mant_bits),
+                      mag / (2.0 ** (1 - bias - mant_bits)))
+    pos = pos + torch.rand(pos.size(), dtype=pos.dtype, layout=pos.layout, device=pos.device, generator=generator)
+    frac = pos.floor() / (1 << mant_bits)
+    out = torch.where(normal, torch.exp2(biased - bias) * (1.0 + frac), (2.0 ** (1 - bias)) * frac)
+    out = torch.where(mag == 0, torch.zeros_like(out), out) * torch.sign(xh)
     lim = torch.finfo(dtype)
     return out.clamp(min=lim.min, max=lim.max)
 

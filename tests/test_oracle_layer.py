@@ -1,0 +1,117 @@
+"""Pins the Linear / SwiGLU / whole-layer restatements of the oracle
+(/root/reference/comfy/ops.py:314-358, 399-410; comfy/ldm/hidream/model.py:237-238, 307-325)."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from comfyui_amd import synth
+from oracle import hidream_moe_oracle as O
+from tests.helpers import oracle_params, small_layer
+
+BF16 = torch.bfloat16
+FP8 = torch.float8_e4m3fn
+
+
+def test_fp8mm_linear_equals_torch_scaled_mm():
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn((48, 256), generator=g).to(BF16)
+    w8, sw = O.quantize_weight_per_tensor(torch.randn((128, 256), generator=g) * 0.02)
+    for s_in in (1.0, 0.25):
+        si = torch.tensor(s_in, dtype=torch.float32)
+        got = O.linear(x, O.LinearParams(w8, sw, si), "fp8mm")
+        xq = (x * (1.0 / si).to(BF16)).to(FP8)
+        try:
+            ref = torch._scaled_mm(xq, w8.t(), out_dtype=BF16, scale_a=si, scale_b=sw)
+        except Exception as e:                      # not every torch build has the CPU kernel
+            pytest.skip(f"torch._scaled_mm unavailable on CPU: {e}")
+        assert torch.equal(got.view(torch.int16), ref.view(torch.int16))
+    # closed form on a case small enough to do by hand: one row, K = 2 (padded), values exactly representable
+    x1 = torch.zeros((1, 16), dtype=BF16); x1[0, 0], x1[0, 1] = 1.5, -2.0
+    w1 = torch.zeros((16, 16)); w1[0, 0], w1[0, 1] = 0.5, 0.25
+    p = O.LinearParams(w1.to(FP8), torch.tensor(2.0), torch.tensor(1.0))
+    assert float(O.linear(x1, p, "fp8mm")[0, 0]) == (1.5 * 0.5 - 2.0 * 0.25) * 2.0
+
+
+def test_fp8mm_without_scale_input_clamps():
+    x = torch.tensor([[1000.0, -1000.0, 3.0, 0.0] + [0.0] * 12], dtype=BF16)
+    w = torch.zeros((16, 16)); w[0, 0] = w[0, 1] = w[0, 2] = 1.0
+    p = O.LinearParams(w.to(FP8), torch.tensor(1.0), None)
+    assert float(O.linear(x, p, "fp8mm")[0, 0]) == 448.0 - 448.0 + 3.0
+
+
+def test_upcast_linear_is_dequantised_matmul():
+    g = torch.Generator().manual_seed(1)
+    w8, sw = O.quantize_weight_per_tensor(torch.randn((96, 64), generator=g) * 0.02)
+    for rows in (4, 300):                                   # scale on the input / on the weight (ops.py:407-410)
+        x = torch.randn((rows, 64), generator=g)
+        got = O.linear(x, O.LinearParams(w8, sw), "upcast")
+        ref = x.double() @ (w8.double() * sw.double()).t()
+        assert float((got.double() - ref).abs().max()) <= 1e-5 * float(ref.abs().max())
+
+
+def test_swiglu_closed_form_fp64():
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn((10, 32), generator=g, dtype=torch.float64)
+    w1, w2, w3 = (torch.randn(s, generator=g, dtype=torch.float64) for s in ((48, 32), (32, 48), (48, 32)))
+    got = O.ffn_swiglu(x, (O.LinearParams(w1), O.LinearParams(w2), O.LinearParams(w3)), "plain")
+    a = x @ w1.t()
+    ref = ((a / (1 + torch.exp(-a))) * (x @ w3.t())) @ w2.t()
+    assert float((got - ref).abs().max()) < 1e-12
+
+
+@pytest.mark.parametrize("weights,mode,dtype,tol", [("bf16", "plain", torch.float32, 2e-6), ("fp8", "upcast", torch.float32, 2e-6),
+                                                    ("fp8", "fp8mm", torch.float32, 2e-6), ("fp8", "fp8mm", BF16, 3e-3),
+                                                    ("bf16", "plain", BF16, 3e-3)])
+def test_layer_equals_dense_brute_force(weights, mode, dtype, tol):
+    sd, x = small_layer(seed=5, dim=128, tokens=96, weights=weights, hidden_arg=384)
+    params = oracle_params(sd, 4)
+    xx = x.to(dtype)
+    idx, w, _, _ = O.gate_torch(xx.reshape(-1, 128), sd["gate.weight"])
+    got = O.moe_forward(xx, params, mode)
+    ref = O.moe_forward_dense(xx, params, mode, idx, w)
+    m = O.error_metrics(got, ref)
+    assert m["rel_rms"] <= tol, m       # row subsets change torch's summation order, nothing else
+
+
+def test_layer_special_cases():
+    sd, x = small_layer(seed=6, dim=128, tokens=64, weights="bf16", hidden_arg=384)
+    # all routed experts identical => y = (w0 + w1) * FFN(x) + shared(x)   (fp32 so the algebra holds to rounding)
+    for e in range(1, 4):
+        for l in ("w1", "w2", "w3"):
+            sd[f"experts.{e}.{l}.weight"] = sd[f"experts.0.{l}.weight"]
+    params = oracle_params(sd, 4)
+    xf = x.float()
+    idx, w, _, _ = O.gate_torch(xf.reshape(-1, 128), sd["gate.weight"])
+    got = O.moe_forward(xf, params, "plain")
+    ffn = O.ffn_swiglu(xf, params["experts"][0], "plain")
+    ref = ffn * w.sum(dim=1).view(1, -1, 1) + O.ffn_swiglu(xf, params["shared"], "plain")
+    assert O.error_metrics(got, ref)["rel_rms"] < 1e-6
+    # reusing a routing decision reproduces the self-routed result
+    again = O.moe_forward(xf, params, "plain", gate_result=(idx, w))
+    assert torch.equal(got, again)
+
+
+def test_bf16_rounding_points_match_torch_kernels():
+    # the statements the HIP kernels rely on: bf16 softmax / silu / products are fp32 math rounded once
+    g = torch.Generator().manual_seed(7)
+    a = (torch.randn(4096, generator=g) * 3).to(BF16)
+    b = torch.randn(4096, generator=g).to(BF16)
+    silu = (a.float() / (1 + torch.exp(-a.float()))).to(BF16)
+    assert float((F.silu(a).view(torch.int16) != silu.view(torch.int16)).float().mean()) < 2e-3
+    assert torch.equal((a * b).view(torch.int16), (a.float() * b.float()).to(BF16).view(torch.int16))
+    lg = torch.randn((1024, 4), generator=g).to(BF16)
+    sm = torch.softmax(lg.float(), dim=-1).to(BF16)
+    assert float((lg.softmax(-1).view(torch.int16) != sm.view(torch.int16)).float().mean()) < 2e-3
+
+
+def test_synth_configs_shapes():
+    assert synth.H_ROUTED == 6912 and synth.H_SHARED == 3584
+    master, g = synth.make_weights(0, dim=128, hidden_arg=384)
+    keys = list(master.keys())
+    assert keys[:3] == ["shared_experts.w1.weight", "shared_experts.w2.weight", "shared_experts.w3.weight"]
+    assert keys[3] == "experts.0.w1.weight" and keys[-1] == "gate.weight"
+    sd = synth.to_state_dict(master, "fp8")
+    assert sd["experts.1.w2.weight"].dtype == FP8 and sd["gate.weight"].dtype == BF16
+    assert float(sd["experts.1.w2.weight"].float().abs().max()) == 448.0
+    x = synth.make_input(g, 64, dim=128, outlier_frac=0.05)
+    assert x.shape == (1, 64, 128) and x.dtype == BF16
