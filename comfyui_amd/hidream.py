@@ -82,7 +82,8 @@ class MoEGate(nn.Module):
 
 
 def _plain(lin):
-    return len(lin.weight_function) == 0 and len(lin.bias_function) == 0 and lin.bias is None
+    return (len(getattr(lin, "weight_function", ())) == 0 and len(getattr(lin, "bias_function", ())) == 0
+            and lin.bias is None)
 
 
 class MOEFeedForwardSwiGLU(nn.Module):
@@ -118,7 +119,8 @@ class MOEFeedForwardSwiGLU(nn.Module):
         ffns = list(self.experts) + [self.shared_experts]
         lins = [l for f in ffns for l in (f.w1, f.w2, f.w3)]
         for l in lins:
-            if not isinstance(l, amd_ops.disable_weight_init.Linear) or l.bias is not None or len(l.bias_function) > 0:
+            # any Linear that follows the operations contract (this package's or ComfyUI's own classes)
+            if not isinstance(l, torch.nn.Linear) or l.bias is not None or len(getattr(l, "bias_function", ())) > 0:
                 return None
         wdt = lins[0].weight.dtype
         if wdt not in (BF16, FP8) or any(l.weight.dtype != wdt for l in lins):

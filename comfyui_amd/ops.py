@@ -84,14 +84,14 @@ def cast_bias_weight(s, input=None, dtype=None, device=None, bias_dtype=None):
 
     bias = None
     if s.bias is not None:
-        has_fn = len(s.bias_function) > 0
+        has_fn = len(getattr(s, "bias_function", ())) > 0
         bias = cast_to(s.bias, bias_dtype, device, non_blocking=non_blocking, copy=has_fn, stream=offload_stream)
         if has_fn:
             with fn_ctx:
                 for f in s.bias_function:
                     bias = f(bias)
 
-    has_fn = len(s.weight_function) > 0
+    has_fn = len(getattr(s, "weight_function", ())) > 0
     weight = cast_to(s.weight, dtype, device, non_blocking=non_blocking, copy=has_fn, stream=offload_stream)
     if has_fn:
         with fn_ctx:
