@@ -33,6 +33,8 @@
 #include "common.h"
 #include "numfmt.h"
 
+#include <type_traits>
+
 namespace {
 
 typedef int v8i __attribute__((ext_vector_type(8)));
@@ -89,6 +91,9 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
   constexpr bool SWIGLU = (MODE == FP8_SWIGLU || MODE == BF16_SWIGLU);
   constexpr int FEAT_PER_TILE = SWIGLU ? BN / 2 : BN;  // output features per block tile
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+#ifdef HDMOE_DBG_CLOCK
+  const long long dbg_start = clock64();
+#endif
 
   // ---- which tile --------------------------------------------------------------
   const int nb = gridDim.x;  // multiple of 8
@@ -116,9 +121,18 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
   const int within = L - band * (GROUP_M * ntiles);
   const int mt = first_m + within % gm;
   const int nt = within / gm;
+#ifdef HDMOE_DBG_SAME_TILE
+  // experiment: every block reads (and rewrites) tile (0,0) of its group, so all operand traffic hits L2
+  const int row0 = rb; (void)mt;
+#else
   const int row0 = rb + mt * BM;            // first token row of the tile
+#endif
   const int rows_here = min(re - row0, BM); // valid rows in the tile
+#ifdef HDMOE_DBG_SAME_TILE
+  const int n0 = 0; (void)nt;
+#else
   const int n0 = nt * FEAT_PER_TILE;        // first output feature of the tile
+#endif
   const int kbytes = gg.kbytes;
   const int KT = kbytes / BK;
 
@@ -176,66 +190,85 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
 
-  auto compute = [&](int stage) {
+  // Fragments of one K sub-step: 4 token tiles and 2 weight tiles of 32 rows.
+  using Frag = typename std::conditional<FP8, v8i, v8bf>::type;
+  constexpr int NSUB = FP8 ? 2 : 4;  // sub-steps (one MFMA K extent each) per 128-byte K step
+  struct FragSet { Frag a[4]; Frag b[2]; };
+
+  auto load_frags = [&](int stage, int ks, FragSet& f) {
     const uint8_t* st = smem + stage * STAGE_BYTES;
     if constexpr (FP8) {
+      const int c0 = ((ks * 4 + fr_grp * 2) ^ fr_swz) * 16;
+      const int c1 = c0 ^ 16;
 #pragma unroll
-      for (int ks = 0; ks < 2; ++ks) {
-        const int c0 = ((ks * 4 + fr_grp * 2) ^ fr_swz) * 16;
-        const int c1 = c0 ^ 16;
-        v8i fa[4], fb[2];
+      for (int tt = 0; tt < 4; ++tt) {
+        const uint8_t* p = st + a_base + tt * 32 * BK;
+        const v4i lo = *reinterpret_cast<const v4i*>(p + c0);
+        const v4i hi = *reinterpret_cast<const v4i*>(p + c1);
+        f.a[tt] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+      }
 #pragma unroll
-        for (int tt = 0; tt < 4; ++tt) {
-          const uint8_t* p = st + a_base + tt * 32 * BK;
-          const v4i lo = *reinterpret_cast<const v4i*>(p + c0);
-          const v4i hi = *reinterpret_cast<const v4i*>(p + c1);
-          fa[tt] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-        }
-#pragma unroll
-        for (int ft = 0; ft < 2; ++ft) {
-          const uint8_t* p = st + b_base + ft * 128 * BK;
-          const v4i lo = *reinterpret_cast<const v4i*>(p + c0);
-          const v4i hi = *reinterpret_cast<const v4i*>(p + c1);
-          fb[ft] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-        }
-#pragma unroll
-        for (int ft = 0; ft < 2; ++ft)
-#pragma unroll
-          for (int tt = 0; tt < 4; ++tt)
-            acc[ft][tt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[ft], fa[tt], acc[ft][tt], 0, 0, 0, 0, 0, 0);
+      for (int ft = 0; ft < 2; ++ft) {
+        const uint8_t* p = st + b_base + ft * 128 * BK;
+        const v4i lo = *reinterpret_cast<const v4i*>(p + c0);
+        const v4i hi = *reinterpret_cast<const v4i*>(p + c1);
+        f.b[ft] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
       }
     } else {
+      const int c0 = ((ks * 2 + fr_grp) ^ fr_swz) * 16;
 #pragma unroll
-      for (int ks = 0; ks < 4; ++ks) {
-        const int c0 = ((ks * 2 + fr_grp) ^ fr_swz) * 16;
-        v8bf fa[4], fb[2];
+      for (int tt = 0; tt < 4; ++tt) f.a[tt] = *reinterpret_cast<const v8bf*>(st + a_base + tt * 32 * BK + c0);
 #pragma unroll
-        for (int tt = 0; tt < 4; ++tt)
-          fa[tt] = *reinterpret_cast<const v8bf*>(st + a_base + tt * 32 * BK + c0);
-#pragma unroll
-        for (int ft = 0; ft < 2; ++ft)
-          fb[ft] = *reinterpret_cast<const v8bf*>(st + b_base + ft * 128 * BK + c0);
-#pragma unroll
-        for (int ft = 0; ft < 2; ++ft)
-#pragma unroll
-          for (int tt = 0; tt < 4; ++tt)
-            acc[ft][tt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[ft], fa[tt], acc[ft][tt], 0, 0, 0);
-      }
+      for (int ft = 0; ft < 2; ++ft) f.b[ft] = *reinterpret_cast<const v8bf*>(st + b_base + ft * 128 * BK + c0);
     }
   };
 
-  // ---- main loop: one barrier per K step --------------------------------------------
+  auto mfma_set = [&](const FragSet& f) {
+#pragma unroll
+    for (int ft = 0; ft < 2; ++ft)
+#pragma unroll
+      for (int tt = 0; tt < 4; ++tt) {
+        if constexpr (FP8)
+          acc[ft][tt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.b[ft], f.a[tt], acc[ft][tt], 0, 0, 0, 0, 0, 0);
+        else
+          acc[ft][tt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.b[ft], f.a[tt], acc[ft][tt], 0, 0, 0);
+      }
+  };
+
+#ifdef HDMOE_DBG_CLOCK
+  const long long dbg_c0 = clock64(), dbg_w0 = wall_clock64();
+#endif
+  // ---- main loop -------------------------------------------------------------------------
+  // Software pipeline: the fragments of sub-step s+1 are read from LDS while the MFMAs of
+  // sub-step s run, so a wave never waits on LDS with an idle matrix pipe. One barrier per
+  // K step, placed before the last sub-step: by then this wave has issued (and, at the
+  // barrier, completed) all its reads of the current stage, so the stage can be refilled
+  // with K step kt+2 right after the barrier, while K step kt+1 (issued one step earlier)
+  // has landed for everybody.
+  FragSet f0, f1;
   issue_loads(0, 0);
-  for (int kt = 0; kt < KT; kt += 2) {
-    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's part of the stage has landed
-    __syncthreads();                      // everyone's part has; everyone is done reading the other stage
-    if (kt + 1 < KT) issue_loads(1, kt + 1);
-    compute(0);
-    if (kt + 1 < KT) {
-      __builtin_amdgcn_s_waitcnt(0x0f70);
-      __syncthreads();
-      if (kt + 2 < KT) issue_loads(0, kt + 2);
-      compute(1);
+  if (KT > 1) {
+    issue_loads(1, 1);
+    __builtin_amdgcn_s_waitcnt(0x0f78);  // vmcnt(8): the 8 loads of stage 0 have landed, stage 1 may be in flight
+  } else {
+    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
+  }
+  __builtin_amdgcn_s_barrier();
+  load_frags(0, 0, f0);
+  for (int kt = 0; kt < KT; ++kt) {
+    const int st = kt & 1;
+#pragma unroll
+    for (int s2 = 0; s2 < NSUB; ++s2) {
+      FragSet& cur = (s2 & 1) ? f1 : f0;
+      FragSet& nxt = (s2 & 1) ? f0 : f1;
+      if (s2 + 1 < NSUB) {
+        load_frags(st, s2 + 1, nxt);
+      } else if (kt + 1 < KT) {
+        __syncthreads();  // waits for this wave's LDS reads and its loads of K step kt+1, then for the block
+        if (kt + 2 < KT) issue_loads(st, kt + 2);
+        load_frags(st ^ 1, 0, nxt);
+      }
+      mfma_set(cur);
     }
   }
 
@@ -311,6 +344,11 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
       }
     }
   }
+#ifdef HDMOE_DBG_CLOCK
+  __builtin_amdgcn_s_waitcnt(0);
+  if (threadIdx.x == 0 && (blockIdx.x == 0 || blockIdx.x == 1001))
+    printf("block %d: epilogue %lld shader clocks (stores drained)\n", (int)blockIdx.x, clock64() - dbg_c1);
+#endif
 }
 
 template <int MODE>
