@@ -53,6 +53,8 @@ def build(verbose=True, extra_flags=()):
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.check_call(cmd)
+    # an unresolved symbol (e.g. a kernel stub the host pass dropped) must fail the build, not the first call
+    subprocess.check_call([sys.executable, "-c", f"import ctypes; ctypes.CDLL({LIB!r})"])
     return LIB
 
 

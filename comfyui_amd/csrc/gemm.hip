@@ -33,8 +33,6 @@
 #include "common.h"
 #include "numfmt.h"
 
-#include <type_traits>
-
 namespace {
 
 typedef int v8i __attribute__((ext_vector_type(8)));
@@ -73,7 +71,8 @@ struct GemmGroup {
 
 struct GemmArgs {
   GemmGroup g[MAX_GROUPS];
-  const int32_t* offsets;
+  const int32_t* offsets;  // segment bounds of the dynamic groups, n_offsets + 1 entries
+  int n_offsets;
   int G;
 };
 
@@ -85,93 +84,104 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint3
 
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+
 template <int MODE>
 __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs args) {
   constexpr bool FP8 = (MODE == FP8_SWIGLU || MODE == FP8_PLAIN);
   constexpr bool SWIGLU = (MODE == FP8_SWIGLU || MODE == BF16_SWIGLU);
   constexpr int FEAT_PER_TILE = SWIGLU ? BN / 2 : BN;  // output features per block tile
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
-#ifdef HDMOE_DBG_CLOCK
-  const long long dbg_start = clock64();
-#endif
-
-  // ---- which tile --------------------------------------------------------------
-  const int nb = gridDim.x;  // multiple of 8
-  int L = (blockIdx.x % HDMOE_NUM_XCD) * (nb / HDMOE_NUM_XCD) + blockIdx.x / HDMOE_NUM_XCD;
-  int g = 0, rb = 0, re = 0, mtiles = 0, ntiles = 0;
-  for (; g < args.G; ++g) {
-    const GemmGroup& gg = args.g[g];
-    if (gg.row_begin >= 0) { rb = gg.row_begin; re = gg.row_end; }
-    else {
-      // loaded through the vector memory path; tell the compiler the values are wave-uniform
-      rb = __builtin_amdgcn_readfirstlane(args.offsets[gg.dyn]);
-      re = __builtin_amdgcn_readfirstlane(args.offsets[gg.dyn + 1]);
-    }
-    mtiles = (re - rb + BM - 1) / BM;
-    ntiles = gg.n_out / FEAT_PER_TILE;
-    const int tiles = mtiles * ntiles;
-    if (L < tiles) break;
-    L -= tiles;
-  }
-  if (g == args.G) return;
-  const GemmGroup& gg = args.g[g];
-  const int band = L / (GROUP_M * ntiles);
-  const int first_m = band * GROUP_M;
-  const int gm = min(mtiles - first_m, GROUP_M);
-  const int within = L - band * (GROUP_M * ntiles);
-  const int mt = first_m + within % gm;
-  const int nt = within / gm;
-#ifdef HDMOE_DBG_SAME_TILE
-  // experiment: every block reads (and rewrites) tile (0,0) of its group, so all operand traffic hits L2
-  const int row0 = rb; (void)mt;
-#else
-  const int row0 = rb + mt * BM;            // first token row of the tile
-#endif
-  const int rows_here = min(re - row0, BM); // valid rows in the tile
-#ifdef HDMOE_DBG_SAME_TILE
-  const int n0 = 0; (void)nt;
-#else
-  const int n0 = nt * FEAT_PER_TILE;        // first output feature of the tile
-#endif
-  const int kbytes = gg.kbytes;
-  const int KT = kbytes / BK;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform by construction
   const int wq = wave & 3, wt = wave >> 2;
 
+  // ---- tile enumeration (persistent blocks) ----------------------------------------------
+  // Segment bounds of the dynamic groups: one vector load, then lane reads.
+  int off_lane = 0;
+  if (args.offsets != nullptr && lane <= args.n_offsets) off_lane = args.offsets[lane];
+  auto seg = [&](const GemmGroup& gg, int& rb, int& re) {
+    if (gg.row_begin >= 0) { rb = gg.row_begin; re = gg.row_end; }
+    else { rb = __builtin_amdgcn_readlane(off_lane, gg.dyn); re = __builtin_amdgcn_readlane(off_lane, gg.dyn + 1); }
+  };
+  int total = 0;
+  for (int g = 0; g < args.G; ++g) {
+    int rb, re;
+    seg(args.g[g], rb, re);
+    total += ((re - rb + BM - 1) / BM) * (args.g[g].n_out / FEAT_PER_TILE);
+  }
+  // Each XCD (block ids congruent mod 8) walks one contiguous eighth of the tile list and its blocks take
+  // consecutive tiles, so the CUs of an XCD share operand tiles in their L2.
+  const int per_xcd = (total + HDMOE_NUM_XCD - 1) / HDMOE_NUM_XCD;
+  const int xcd = blockIdx.x % HDMOE_NUM_XCD, slot = blockIdx.x / HDMOE_NUM_XCD;
+  const int nslots = gridDim.x / HDMOE_NUM_XCD;
+
+  struct Tile { int g, row0, rows_here, n0, kbytes; };
+  auto decode = [&](int i) -> Tile {
+    Tile d = {-1, 0, 0, 0, 0};
+    const int in_xcd = slot + i * nslots;
+    int L = xcd * per_xcd + in_xcd;
+    if (in_xcd >= per_xcd || L >= total) return d;
+    int g = 0, rb = 0, re = 0, mtiles = 0, ntiles = 0;
+    for (; g < args.G; ++g) {
+      seg(args.g[g], rb, re);
+      mtiles = (re - rb + BM - 1) / BM;
+      ntiles = args.g[g].n_out / FEAT_PER_TILE;
+      const int tiles = mtiles * ntiles;
+      if (L < tiles) break;
+      L -= tiles;
+    }
+    if (g >= args.G) return d;
+    const int band = L / (GROUP_M * ntiles);
+    const int first_m = band * GROUP_M;
+    const int gm = min(mtiles - first_m, GROUP_M);
+    const int within = L - band * (GROUP_M * ntiles);
+    d.g = g;
+    d.row0 = rb + (first_m + within % gm) * BM;
+    d.rows_here = min(re - d.row0, BM);
+    d.n0 = (within / gm) * FEAT_PER_TILE;
+    d.kbytes = args.g[g].kbytes;
+    return d;
+  };
+
   // ---- global -> LDS addressing --------------------------------------------------
-  // One wave-level load moves 8 rows x 128 bytes. Lane i lands in LDS chunk (i&7) of
-  // row (i>>3) and therefore fetches logical chunk (i&7) ^ f(row).
-  // Rows past the segment end are outside the buffer range and read as zero.
-  const __amdgpu_buffer_rsrc_t rsrc_a = make_rsrc(gg.a + (size_t)row0 * kbytes, (uint32_t)rows_here * (uint32_t)kbytes);
-  const uint8_t* b_half0 = gg.b0 + (size_t)n0 * kbytes;
-  const uint8_t* b_half1 = SWIGLU ? gg.b1 + (size_t)n0 * kbytes : gg.b0 + (size_t)(n0 + BN / 2) * kbytes;
-  const __amdgpu_buffer_rsrc_t rsrc_b0 = make_rsrc(b_half0, (uint32_t)(BN / 2) * (uint32_t)kbytes);
-  const __amdgpu_buffer_rsrc_t rsrc_b1 = make_rsrc(b_half1, (uint32_t)(BN / 2) * (uint32_t)kbytes);
+  // One wave-level load moves 8 rows x 128 bytes. Lane i lands in LDS chunk (i&7) of row (i>>3) and therefore
+  // fetches logical chunk (i&7) ^ f(row). Rows past the segment end are outside the buffer range and read as
+  // zero: the row part of the address sits in the VGPR offset, the only one that is range-checked; the K
+  // position goes through the scalar offset.
   const int ld_row = wave * 8 + (lane >> 3);                 // row within a 64-row slab
   const int ld_chunk = (lane & 7) ^ swz(ld_row);
-  // The row part must sit in the VGPR offset: only that offset is range-checked, the
-  // scalar offset (used for the K position) is not.
-  int ld_voff[4];
-#pragma unroll
-  for (int j = 0; j < 4; ++j) ld_voff[j] = (j * 64 + ld_row) * kbytes + ld_chunk * 16;
   const int ld_lds = wave * 8 * BK;                          // + slab*64*BK
 
+  // source of the tile being loaded (buffer resources are kept as plain locals: the opaque resource type
+  // cannot be a struct member)
+  __amdgpu_buffer_rsrc_t src_a = make_rsrc(nullptr, 0), src_b0 = src_a, src_b1 = src_a;
+  int src_voff[4] = {0, 0, 0, 0};
+  auto set_src = [&](const Tile& d) {
+    const GemmGroup& gg = args.g[d.g];
+    src_a = make_rsrc(gg.a + (size_t)d.row0 * d.kbytes, (uint32_t)d.rows_here * (uint32_t)d.kbytes);
+    const uint8_t* b_half0 = gg.b0 + (size_t)d.n0 * d.kbytes;
+    const uint8_t* b_half1 = SWIGLU ? gg.b1 + (size_t)d.n0 * d.kbytes : gg.b0 + (size_t)(d.n0 + BN / 2) * d.kbytes;
+    src_b0 = make_rsrc(b_half0, (uint32_t)(BN / 2) * (uint32_t)d.kbytes);
+    src_b1 = make_rsrc(b_half1, (uint32_t)(BN / 2) * (uint32_t)d.kbytes);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) src_voff[j] = (j * 64 + ld_row) * d.kbytes + ld_chunk * 16;
+  };
   auto issue_loads = [&](int stage, int kt) {
     uint8_t* sa = smem + stage * STAGE_BYTES;
     uint8_t* sb = sa + TILE_BYTES;
     const int k0 = kt * BK;
 #pragma unroll
     for (int j = 0; j < 4; ++j)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_ptr_t)(sa + ld_lds + j * 64 * BK), 16, ld_voff[j], k0, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(src_a, (lds_ptr_t)(sa + ld_lds + j * 64 * BK), 16, src_voff[j], k0, 0, 0);
 #pragma unroll
     for (int j = 0; j < 2; ++j)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b0, (lds_ptr_t)(sb + ld_lds + j * 64 * BK), 16, ld_voff[j], k0, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(src_b0, (lds_ptr_t)(sb + ld_lds + j * 64 * BK), 16, src_voff[j], k0, 0, 0);
 #pragma unroll
     for (int j = 0; j < 2; ++j)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_b1, (lds_ptr_t)(sb + ld_lds + (j + 2) * 64 * BK), 16, ld_voff[j], k0, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(src_b1, (lds_ptr_t)(sb + ld_lds + (j + 2) * 64 * BK), 16, src_voff[j], k0, 0, 0);
   };
 
   // ---- LDS -> MFMA fragment addressing -------------------------------------------
@@ -183,115 +193,76 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
   const int b_base = TILE_BYTES + (wq * 32 + fr_row) * BK;   // weight operand, + ft*128*BK
 
   v16f acc[2][4];
-#pragma unroll
-  for (int i = 0; i < 2; ++i)
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.0f;
-
-  // Fragments of one K sub-step: 4 token tiles and 2 weight tiles of 32 rows.
-  using Frag = typename std::conditional<FP8, v8i, v8bf>::type;
-  constexpr int NSUB = FP8 ? 2 : 4;  // sub-steps (one MFMA K extent each) per 128-byte K step
-  struct FragSet { Frag a[4]; Frag b[2]; };
-
-  auto load_frags = [&](int stage, int ks, FragSet& f) {
+  auto compute = [&](int stage) {
     const uint8_t* st = smem + stage * STAGE_BYTES;
     if constexpr (FP8) {
-      const int c0 = ((ks * 4 + fr_grp * 2) ^ fr_swz) * 16;
-      const int c1 = c0 ^ 16;
 #pragma unroll
-      for (int tt = 0; tt < 4; ++tt) {
-        const uint8_t* p = st + a_base + tt * 32 * BK;
-        const v4i lo = *reinterpret_cast<const v4i*>(p + c0);
-        const v4i hi = *reinterpret_cast<const v4i*>(p + c1);
-        f.a[tt] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-      }
+      for (int ks = 0; ks < 2; ++ks) {
+        const int c0 = ((ks * 4 + fr_grp * 2) ^ fr_swz) * 16;
+        const int c1 = c0 ^ 16;
+        v8i fa[4], fb[2];
 #pragma unroll
-      for (int ft = 0; ft < 2; ++ft) {
-        const uint8_t* p = st + b_base + ft * 128 * BK;
-        const v4i lo = *reinterpret_cast<const v4i*>(p + c0);
-        const v4i hi = *reinterpret_cast<const v4i*>(p + c1);
-        f.b[ft] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        for (int tt = 0; tt < 4; ++tt) {
+          const uint8_t* p = st + a_base + tt * 32 * BK;
+          const v4i lo = *reinterpret_cast<const v4i*>(p + c0);
+          const v4i hi = *reinterpret_cast<const v4i*>(p + c1);
+          fa[tt] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        }
+#pragma unroll
+        for (int ft = 0; ft < 2; ++ft) {
+          const uint8_t* p = st + b_base + ft * 128 * BK;
+          const v4i lo = *reinterpret_cast<const v4i*>(p + c0);
+          const v4i hi = *reinterpret_cast<const v4i*>(p + c1);
+          fb[ft] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        }
+#pragma unroll
+        for (int ft = 0; ft < 2; ++ft)
+#pragma unroll
+          for (int tt = 0; tt < 4; ++tt)
+            acc[ft][tt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[ft], fa[tt], acc[ft][tt], 0, 0, 0, 0, 0, 0);
       }
     } else {
-      const int c0 = ((ks * 2 + fr_grp) ^ fr_swz) * 16;
 #pragma unroll
-      for (int tt = 0; tt < 4; ++tt) f.a[tt] = *reinterpret_cast<const v8bf*>(st + a_base + tt * 32 * BK + c0);
+      for (int ks = 0; ks < 4; ++ks) {
+        const int c0 = ((ks * 2 + fr_grp) ^ fr_swz) * 16;
+        v8bf fa[4], fb[2];
 #pragma unroll
-      for (int ft = 0; ft < 2; ++ft) f.b[ft] = *reinterpret_cast<const v8bf*>(st + b_base + ft * 128 * BK + c0);
+        for (int tt = 0; tt < 4; ++tt)
+          fa[tt] = *reinterpret_cast<const v8bf*>(st + a_base + tt * 32 * BK + c0);
+#pragma unroll
+        for (int ft = 0; ft < 2; ++ft)
+          fb[ft] = *reinterpret_cast<const v8bf*>(st + b_base + ft * 128 * BK + c0);
+#pragma unroll
+        for (int ft = 0; ft < 2; ++ft)
+#pragma unroll
+          for (int tt = 0; tt < 4; ++tt)
+            acc[ft][tt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[ft], fa[tt], acc[ft][tt], 0, 0, 0);
+      }
     }
   };
-
-  auto mfma_set = [&](const FragSet& f) {
-#pragma unroll
-    for (int ft = 0; ft < 2; ++ft)
-#pragma unroll
-      for (int tt = 0; tt < 4; ++tt) {
-        if constexpr (FP8)
-          acc[ft][tt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(f.b[ft], f.a[tt], acc[ft][tt], 0, 0, 0, 0, 0, 0);
-        else
-          acc[ft][tt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.b[ft], f.a[tt], acc[ft][tt], 0, 0, 0);
-      }
-  };
-
-#ifdef HDMOE_DBG_CLOCK
-  const long long dbg_c0 = clock64(), dbg_w0 = wall_clock64();
-#endif
-  // ---- main loop -------------------------------------------------------------------------
-  // Software pipeline: the fragments of sub-step s+1 are read from LDS while the MFMAs of
-  // sub-step s run, so a wave never waits on LDS with an idle matrix pipe. One barrier per
-  // K step, placed before the last sub-step: by then this wave has issued (and, at the
-  // barrier, completed) all its reads of the current stage, so the stage can be refilled
-  // with K step kt+2 right after the barrier, while K step kt+1 (issued one step earlier)
-  // has landed for everybody.
-  FragSet f0, f1;
-  issue_loads(0, 0);
-  if (KT > 1) {
-    issue_loads(1, 1);
-    __builtin_amdgcn_s_waitcnt(0x0f78);  // vmcnt(8): the 8 loads of stage 0 have landed, stage 1 may be in flight
-  } else {
-    __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0)
-  }
-  __builtin_amdgcn_s_barrier();
-  load_frags(0, 0, f0);
-  for (int kt = 0; kt < KT; ++kt) {
-    const int st = kt & 1;
-#pragma unroll
-    for (int s2 = 0; s2 < NSUB; ++s2) {
-      FragSet& cur = (s2 & 1) ? f1 : f0;
-      FragSet& nxt = (s2 & 1) ? f0 : f1;
-      if (s2 + 1 < NSUB) {
-        load_frags(st, s2 + 1, nxt);
-      } else if (kt + 1 < KT) {
-        __syncthreads();  // waits for this wave's LDS reads and its loads of K step kt+1, then for the block
-        if (kt + 2 < KT) issue_loads(st, kt + 2);
-        load_frags(st ^ 1, 0, nxt);
-      }
-      mfma_set(cur);
-    }
-  }
 
   // ---- epilogue ----------------------------------------------------------------------
   // acc[ft][tt][i]: feature = (i>>2)*8 + (lane>>5)*4 + (i&3) within the 32-row MFMA tile (ft = weight half),
-  // token = lane&31 within the 32-token MFMA tile.
-  float s_in = 1.0f;
-  if constexpr (FP8) s_in = gg.s_in ? *gg.s_in : 1.0f;
+  // token = lane&31 within the 32-token MFMA tile. Stores go through a buffer resource covering exactly the
+  // valid rows of the tile: rows past the segment end are dropped by the range check.
   const int tok_lane = wt * 128 + (lane & 31);
   const int feat_lane = wq * 32 + (lane >> 5) * 4;
-  if constexpr (SWIGLU) {
-    float sg = 1.0f, su = 1.0f, inv_next = 1.0f;
-    if constexpr (FP8) {
-      sg = s_in * *gg.sb0;
-      su = s_in * *gg.sb1;
-      inv_next = gg.s_next ? hdmoe_dev_round_bf16(__fdiv_rn(1.0f, *gg.s_next)) : -1.0f;
-    }
-    const int ldo = gg.n_out * (FP8 ? 1 : 2);
+  auto epilogue = [&](const Tile& d) {
+    const GemmGroup& gg = args.g[d.g];
+    float s_in = 1.0f;
+    if constexpr (FP8) s_in = gg.s_in ? *gg.s_in : 1.0f;
+    if constexpr (SWIGLU) {
+      float sg = 1.0f, su = 1.0f, inv_next = 1.0f;
+      if constexpr (FP8) {
+        sg = s_in * *gg.sb0;
+        su = s_in * *gg.sb1;
+        inv_next = gg.s_next ? hdmoe_dev_round_bf16(__fdiv_rn(1.0f, *gg.s_next)) : -1.0f;
+      }
+      const int ldo = gg.n_out * (FP8 ? 1 : 2);
+      const __amdgpu_buffer_rsrc_t ro = make_rsrc(gg.out + (size_t)d.row0 * ldo, (uint32_t)d.rows_here * (uint32_t)ldo);
 #pragma unroll
-    for (int tt = 0; tt < 4; ++tt) {
-      const int tok = tok_lane + tt * 32;
-      if (tok < rows_here) {
-        uint8_t* orow = gg.out + (size_t)(row0 + tok) * ldo;
+      for (int tt = 0; tt < 4; ++tt) {
+        const int rowoff = (tok_lane + tt * 32) * ldo;
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           float m[4];
@@ -302,7 +273,7 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
             const float sl = hdmoe_dev_round_bf16(h1 * __builtin_amdgcn_rcpf(1.0f + __expf(-h1)));  // silu(.)
             m[i] = hdmoe_dev_round_bf16(sl * h3);                               // silu(.) * w3(x)
           }
-          const int feat = n0 + feat_lane + q * 8;
+          const int feat = d.n0 + feat_lane + q * 8;
           if constexpr (FP8) {
             // activation cast of the w2 Linear (ops.py:337-343)
 #pragma unroll
@@ -311,44 +282,76 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
               else m[i] = hdmoe_dev_round_bf16(m[i] * inv_next);
             }
             const uint32_t pk = hdmoe_dev_pack_e4m3fn(m[0], m[1]) | (hdmoe_dev_pack_e4m3fn(m[2], m[3]) << 16);
-            *reinterpret_cast<uint32_t*>(orow + feat) = pk;
+            __builtin_amdgcn_raw_buffer_store_b32(pk, ro, rowoff + feat, 0, 0);
           } else {
-            uint2 pk;
+            u32x2 pk;
             pk.x = hdmoe_dev_pack_bf16(m[0], m[1]);
             pk.y = hdmoe_dev_pack_bf16(m[2], m[3]);
-            *reinterpret_cast<uint2*>(orow + (size_t)feat * 2) = pk;
+            __builtin_amdgcn_raw_buffer_store_b64(pk, ro, rowoff + feat * 2, 0, 0);
           }
         }
       }
-    }
-  } else {
-    float sc = 1.0f;
-    if constexpr (FP8) sc = s_in * *gg.sb0;
-    const int ldo = gg.n_out * 2;
+    } else {
+      float sc = 1.0f;
+      if constexpr (FP8) sc = s_in * *gg.sb0;
+      const int ldo = gg.n_out * 2;
+      const __amdgpu_buffer_rsrc_t ro = make_rsrc(gg.out + (size_t)d.row0 * ldo, (uint32_t)d.rows_here * (uint32_t)ldo);
 #pragma unroll
-    for (int tt = 0; tt < 4; ++tt) {
-      const int tok = tok_lane + tt * 32;
-      if (tok < rows_here) {
-        uint8_t* orow = gg.out + (size_t)(row0 + tok) * ldo;
+      for (int tt = 0; tt < 4; ++tt) {
+        const int rowoff = (tok_lane + tt * 32) * ldo;
 #pragma unroll
         for (int ft = 0; ft < 2; ++ft) {
 #pragma unroll
           for (int q = 0; q < 4; ++q) {
-            const int feat = n0 + ft * 128 + feat_lane + q * 8;
-            uint2 pk;
+            const int feat = d.n0 + ft * 128 + feat_lane + q * 8;
+            u32x2 pk;
             pk.x = hdmoe_dev_pack_bf16(acc[ft][tt][q * 4 + 0] * sc, acc[ft][tt][q * 4 + 1] * sc);
             pk.y = hdmoe_dev_pack_bf16(acc[ft][tt][q * 4 + 2] * sc, acc[ft][tt][q * 4 + 3] * sc);
-            *reinterpret_cast<uint2*>(orow + (size_t)feat * 2) = pk;
+            __builtin_amdgcn_raw_buffer_store_b64(pk, ro, rowoff + feat * 2, 0, 0);
           }
         }
       }
     }
+  };
+
+  // ---- persistent loop over this block's tiles ------------------------------------------------------
+  // Per tile: K steps of 128 bytes through two LDS stages, one barrier per step (the loads of step kt+1 fly
+  // while step kt is multiplied). The first K step of the NEXT tile is requested before the epilogue of the
+  // current one, so its latency hides behind the stores.
+  Tile cur = decode(0);
+  if (cur.g < 0) return;
+  set_src(cur);
+  issue_loads(0, 0);
+  for (int i = 0; cur.g >= 0; ++i) {
+    const int KT = cur.kbytes / BK;
+#pragma unroll
+    for (int a2 = 0; a2 < 2; ++a2)
+#pragma unroll
+      for (int b2 = 0; b2 < 4; ++b2)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[a2][b2][r] = 0.0f;
+    for (int kt = 0; kt < KT; kt += 2) {
+      __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's part of the stage has landed
+      __syncthreads();                      // everyone's part has; everyone is done reading the other stage
+      if (kt + 1 < KT) issue_loads(1, kt + 1);
+      compute(0);
+      if (kt + 1 < KT) {
+        __builtin_amdgcn_s_waitcnt(0x0f70);
+        __syncthreads();
+        if (kt + 2 < KT) issue_loads(0, kt + 2);
+        compute(1);
+      }
+    }
+    const Tile nxt = decode(i + 1);
+    if (nxt.g >= 0) {
+      // stage 0 was last read in the second-to-last K step when KT is even; with an odd KT it was read just now
+      if (KT & 1) __syncthreads();
+      set_src(nxt);
+      issue_loads(0, 0);
+    }
+    epilogue(cur);
+    cur = nxt;
   }
-#ifdef HDMOE_DBG_CLOCK
-  __builtin_amdgcn_s_waitcnt(0);
-  if (threadIdx.x == 0 && (blockIdx.x == 0 || blockIdx.x == 1001))
-    printf("block %d: epilogue %lld shader clocks (stores drained)\n", (int)blockIdx.x, clock64() - dbg_c1);
-#endif
 }
 
 template <int MODE>
@@ -361,7 +364,9 @@ int launch_grouped(const GemmArgs& args, int tile_bound, hipStream_t s, const ch
     attr_set = true;
   }
   if (tile_bound <= 0) return HDMOE_OK;
-  const int grid = (tile_bound + HDMOE_NUM_XCD - 1) / HDMOE_NUM_XCD * HDMOE_NUM_XCD;
+  // persistent blocks: one per CU (128 KiB of LDS allow no second one), a multiple of the XCD count
+  int grid = (tile_bound + HDMOE_NUM_XCD - 1) / HDMOE_NUM_XCD * HDMOE_NUM_XCD;
+  if (grid > HDMOE_NUM_CU) grid = HDMOE_NUM_CU;
   hipLaunchKernelGGL((grouped_gemm_kernel<MODE>), dim3(grid), dim3(NTHREADS), SMEM_BYTES, s, args);
   return hdmoe_check_launch(what);
 }
@@ -388,6 +393,7 @@ int hdmoe_launch_ffn_gemm(bool swiglu, int weight_dtype, const uint8_t* a_dyn, c
   GemmArgs args;
   memset(&args, 0, sizeof(args));
   args.offsets = offsets;
+  args.n_offsets = n_dyn;
   int G = 0, tile_bound = 0;
   for (int e = 0; e < n_dyn; ++e, ++G) {
     GemmGroup& gg = args.g[G];
