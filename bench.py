@@ -32,6 +32,11 @@ PEAK_FP8_TFLOPS = 5000.0    # MI355X dense fp8 MFMA
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBPS = 8000.0      # MI355X HBM3E
 
+# L2-side traffic of the dominant kernel per launch (bytes fetched + written), from the two rocprofv3 --pmc runs
+# summarised in profiles/bench_cfg3_pmc.txt (FETCH_SIZE x 2.000 and WRITE_SIZE x 1.000 after calibration against a
+# plain 256 MiB copy). Only known for the workload that was profiled.
+MEASURED_TRAFFIC_BYTES = {"cfg3": 1269.6e6 + 142.6e6}
+
 
 class HipEvents:
     """hipEvent_t handles through the HIP runtime that torch already loaded; they can be recorded
@@ -107,6 +112,8 @@ def main():
     ap.add_argument("--workload", default="cfg3", choices=["cfg1", "cfg2", "cfg3"])
     ap.add_argument("--cpu-sample-tokens", type=int, default=8192)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--pmc-calibration", action="store_true",
+                    help="also run one plain 256 MiB device copy, whose FETCH_SIZE/WRITE_SIZE readings calibrate the counters")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on exactly one GPU (one MI355X holds the whole layer; tokens are "
@@ -130,6 +137,14 @@ def main():
     T = B * S
     H, Hs, E = synth.H_ROUTED, synth.H_SHARED, synth.NUM_EXPERTS
     fl = flops_per_token(D, H, Hs, E)
+
+    if args.pmc_calibration:
+        # known traffic: 256 MiB read + 256 MiB written by one elementwise copy kernel
+        src_cal = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst_cal = torch.empty_like(src_cal)
+        dst_cal.copy_(src_cal)
+        torch.cuda.synchronize()
+        del src_cal, dst_cal
 
     hip = HipEvents()
     with torch.no_grad():
@@ -208,7 +223,9 @@ def main():
             "peak": peak,
             "unit": "TFLOP/s",
             "frac": gemm1_tflops / peak,
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+            "traffic_note": "rocprofv3 FETCH_SIZE+WRITE_SIZE per launch, calibrated; see profiles/bench_cfg3_pmc.txt",
+            "algorithmic_bytes": T * (3 * D * eb + (2 * H + Hs) * eb) + (E * 2 * H + 2 * Hs) * D * eb,
             "flop_per_launch": T * fl["gate_up"],
             "avg_launch_ms": stage_ms["gemm_gate_up"],
         },
