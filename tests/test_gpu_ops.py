@@ -1,0 +1,198 @@
+"""GPU behaviour of the operation classes and of the paths ModelPatcher exercises: Linear forwards of every
+operations class, offloaded weights, weight functions (the LowVramPatch hook), replaced Parameters, and the
+per-expert composition the module falls back to. Each result is checked against the CPU oracle's Linear."""
+import pytest
+import torch
+
+from comfyui_amd import synth
+from oracle import hidream_moe_oracle as O
+from tests.helpers import oracle_params, small_layer
+
+pytestmark = pytest.mark.gpu
+BF16 = torch.bfloat16
+FP8 = torch.float8_e4m3fn
+
+
+def close(got, ref, rel):
+    m = O.error_metrics(got, ref)
+    assert m["rel_rms"] <= rel, m
+    return m
+
+
+def make_fp8_linear(cls, K, N, seed, dev, s_in=None):
+    g = torch.Generator().manual_seed(seed)
+    w8, sw = synth.quantize_per_tensor(torch.randn((N, K), generator=g) * 0.02)
+    lin = cls.Linear(K, N, bias=False, dtype=BF16, device=dev)
+    lin.weight = torch.nn.Parameter(w8.to(dev), requires_grad=False)
+    with torch.no_grad():
+        lin.scale_weight.copy_(sw)
+        if s_in is not None and lin.scale_input is not None:
+            lin.scale_input.fill_(s_in)
+    x = torch.randn((3, 50, K), generator=g).to(BF16)
+    return lin, x, w8, sw
+
+
+def test_plain_and_manual_cast_linear(dev):
+    from comfyui_amd import ops
+    g = torch.Generator().manual_seed(0)
+    w = (torch.randn((512, 256), generator=g) * 0.05)
+    x = torch.randn((2, 33, 256), generator=g).to(BF16)
+    ref = O.linear(x, O.LinearParams(w.to(BF16)), "plain")
+    lin = ops.disable_weight_init.Linear(256, 512, bias=False, dtype=BF16, device=dev)
+    with torch.no_grad():
+        lin.weight.copy_(w)
+    y = lin(x.to(dev))
+    assert y.shape == (2, 33, 512) and y.dtype == BF16
+    close(y.cpu(), ref, 3e-3)
+    # manual_cast: weight kept in fp32 on the CPU (offloaded), cast and copied per call
+    lin2 = ops.manual_cast.Linear(256, 512, bias=False, dtype=torch.float32, device="cpu")
+    with torch.no_grad():
+        lin2.weight.copy_(w)
+    close(lin2(x.to(dev)).cpu(), ref, 3e-3)
+    assert lin2.weight.device.type == "cpu"
+
+
+def test_scaled_fp8_linear_with_fp8_matmul(dev):
+    from comfyui_amd import ops
+    cls = ops.scaled_fp8_ops(fp8_matrix_mult=True, scale_input=True, override_dtype=FP8)
+    for s_in in (1.0, 0.5):
+        lin, x, w8, sw = make_fp8_linear(cls, 256, 512, 1, dev, s_in)
+        ref = O.linear(x, O.LinearParams(w8, sw, torch.tensor(s_in)), "fp8mm")
+        xd = x.to(dev)
+        before = xd.clone()
+        y = lin(xd)
+        close(y.cpu(), ref, 3e-3)
+        assert torch.equal(xd, before)          # the input is not modified
+    # 2-D input keeps its rank (ops.py:320-322, 353-354)
+    assert lin(x.to(dev)[0]).shape == (50, 512)
+    # scale_input None -> clamp rule
+    cls2 = ops.scaled_fp8_ops(fp8_matrix_mult=True, scale_input=False, override_dtype=FP8)
+    lin2, x2, w82, sw2 = make_fp8_linear(cls2, 256, 512, 2, dev)
+    x2 = x2 * 300
+    ref2 = O.linear(x2, O.LinearParams(w82, sw2, None), "fp8mm")
+    close(lin2(x2.to(dev)).cpu(), ref2, 3e-3)
+
+
+def test_scaled_fp8_linear_without_fp8_matmul(dev):
+    # the dequantising branch (ops.py:405-410): scale on the weight when it is the smaller operand, else on the input
+    from comfyui_amd import ops
+    cls = ops.scaled_fp8_ops(fp8_matrix_mult=False, scale_input=False, override_dtype=FP8)
+    lin, x, w8, sw = make_fp8_linear(cls, 256, 512, 3, dev)
+    for xx in (x, x[:1, :8]):                                    # 150 rows: weight smaller; 8 rows: input smaller
+        ref = O.linear(xx, O.LinearParams(w8, sw), "upcast")
+        close(lin(xx.contiguous().to(dev)).cpu(), ref, 3e-3)
+
+
+def test_fp8_ops_linear(dev):
+    from comfyui_amd import ops
+    g = torch.Generator().manual_seed(4)
+    w8 = (torch.randn((512, 256), generator=g)).to(FP8)
+    lin = ops.fp8_ops.Linear(256, 512, bias=False, dtype=FP8, device=dev)
+    lin.weight = torch.nn.Parameter(w8.to(dev), requires_grad=False)
+    lin.eval()
+    x = torch.randn((40, 256), generator=g).to(BF16)
+    ref = O.linear(x, O.LinearParams(w8, torch.ones(()), None), "fp8mm")
+    close(lin(x.to(dev)).cpu(), ref, 3e-3)
+
+
+def test_weight_function_and_offloaded_weights_in_the_layer(dev):
+    """What ModelPatcher's low-vram mode does to a module: weights stay on the offload device with
+    comfy_cast_weights=True and a weight_function (LowVramPatch) rewrites the weight at every forward."""
+    dim = 256
+    sd, x = small_layer(seed=31, dim=dim, tokens=120, weights="fp8")
+    m = synth.build_module({k: v.to(dev) for k, v in sd.items()}, "fp8", dev, dim=dim)
+    xd = x.to(dev)
+    base = m(xd).cpu()
+    # (a) offload two Linears and the gate to the CPU: results unchanged
+    m.experts[1].w2.to("cpu")
+    m.shared_experts.w1.to("cpu")
+    m.gate.to("cpu")
+    off = m(xd).cpu()
+    assert torch.equal(off, base)
+    # (b) a weight function that swaps in another weight (what a LoRA patch amounts to)
+    other = sd["experts.0.w1.weight"].to(dev)
+    lin = m.experts[2].w1
+    lin.weight_function = [lambda w: other.clone()]
+    patched = m(xd).cpu()
+    sd2 = dict(sd)
+    sd2["experts.2.w1.weight"] = sd["experts.0.w1.weight"]
+    idx, w, _, _ = O.gate_fixed_order(x.reshape(-1, dim), sd["gate.weight"])
+    ref = O.moe_forward(x, oracle_params(sd2, 4), "fp8mm", gate_result=(idx, w))
+    close(patched, ref, 1e-2)
+    assert not torch.equal(patched, base)
+    lin.weight_function = []
+    # (c) ModelPatcher replaces Parameter objects (utils.set_attr_param): the next forward must see the new one
+    m.experts[2].w1.weight = torch.nn.Parameter(other.clone(), requires_grad=False)
+    assert torch.equal(m(xd).cpu(), patched)
+
+
+def test_mixed_dtypes_use_the_composed_path(dev):
+    dim = 256
+    sd, x = small_layer(seed=32, dim=dim, tokens=90, weights="fp8")
+    m = synth.build_module({k: v.to(dev) for k, v in sd.items()}, "fp8", dev, dim=dim)
+    xd = x.to(dev)
+    fused = m(xd).cpu()
+    # w1 and w3 of one expert disagree on scale_input -> one quantised copy cannot serve both
+    with torch.no_grad():
+        m.experts[0].w3.scale_input.fill_(0.5)
+    assert m._collect(xd.reshape(-1, dim)) is None
+    got = m(xd).cpu()
+    sd2 = dict(sd)
+    sd2["experts.0.w3.scale_input"] = torch.tensor(0.5)
+    idx, w, _, _ = O.gate_fixed_order(x.reshape(-1, dim), sd["gate.weight"])
+    ref = O.moe_forward(x, oracle_params(sd2, 4), "fp8mm", gate_result=(idx, w))
+    close(got, ref, 1e-2)
+    assert got.shape == fused.shape
+
+
+@pytest.mark.parametrize("E", [2, 8])
+def test_other_expert_counts(dev, E):
+    dim = 256
+    sd, x = small_layer(seed=40 + E, dim=dim, tokens=333, weights="fp8", num_experts=E)
+    m = synth.build_module({k: v.to(dev) for k, v in sd.items()}, "fp8", dev, dim=dim, num_experts=E)
+    y = m(x.to(dev)).cpu()
+    idx, w, _, _ = O.gate_fixed_order(x.reshape(-1, dim), sd["gate.weight"])
+    ref = O.moe_forward(x, oracle_params(sd, E), "fp8mm", gate_result=(idx, w))
+    close(y, ref, 1e-2)
+
+
+def test_gate_module_signature(dev):
+    from comfyui_amd import hidream
+    g = hidream.MoEGate(512, 4, 2, dtype=BF16, device=dev)
+    with torch.no_grad():
+        g.weight.normal_(0, 512 ** -0.5)
+    x = torch.randn((2, 9, 512), device=dev).to(BF16)
+    idx, w, aux = g(x)
+    assert idx.dtype == torch.int64 and idx.shape == (18, 2) and w.dtype == BF16 and w.shape == (18, 2) and aux is None
+    ridx, rw, _, _ = O.gate_fixed_order(x.cpu().reshape(-1, 512), g.weight.detach().cpu())
+    assert torch.equal(idx.cpu(), ridx.long())
+
+
+def test_stacked_layers_at_32768_tokens(dev):
+    """Stacked sweep (benchmark configuration 4) on a reduced stack: 3 independent fp8 layers at 2 x 16384 tokens,
+    x <- x + FFN(LayerNorm(x)) with the block's affine-free LayerNorm (model.py:393,430) so the residual stream
+    stays in range. Tokens are independent through the whole stack, so the oracle follows a token subset."""
+    T, D, L = 32768, synth.DIM, 3
+    g = torch.Generator().manual_seed(99)
+    x0 = torch.randn((2, T // 2, D), generator=g).to(BF16)
+    sel = torch.randperm(T, generator=g)[:48].sort().values
+    xd = x0.to(dev)
+    ln = lambda t: torch.nn.functional.layer_norm(t.float(), (D,), eps=1e-6).to(BF16)
+    for layer in range(L):
+        master, _ = synth.make_weights(layer)
+        sd = synth.to_state_dict(master, "fp8")
+        del master
+        m = synth.build_module({k: v.to(dev) for k, v in sd.items()}, "fp8", dev)
+        # the oracle starts every layer from the device's own residual stream (for the token subset): rounding
+        # differences of one layer would otherwise flip e4m3 neighbours in the next and the two runs drift apart
+        xs = xd.reshape(-1, D)[sel].cpu().unsqueeze(0)
+        xd = xd + m(ln(xd))
+        h = ln(xs)
+        idx, w, _, _ = O.gate_fixed_order(h.reshape(-1, D), sd["gate.weight"])
+        ref = xs + O.moe_forward(h, oracle_params(sd, 4), "fp8mm", gate_result=(idx, w))
+        got = xd.reshape(-1, D)[sel].cpu()
+        met = O.error_metrics(got, ref.reshape(-1, D))
+        print(f"layer {layer}: rms(x)={float(got.float().pow(2).mean().sqrt()):.3f} {met}")
+        assert not bool(got.float().isnan().any())
+        assert met["rel_rms"] <= 1e-2 and met["max_over_max"] <= 3e-2, met
+        del m
