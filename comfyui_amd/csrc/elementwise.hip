@@ -54,19 +54,58 @@ __global__ __launch_bounds__(THREADS) void quant_rows_kernel(const uint4* __rest
     for (int u = lane; u < row16; u += 64) out[r * row16 + u] = quant8(x[r * row16 + u], inv);
 }
 
-__global__ __launch_bounds__(THREADS) void quant_permute_kernel(const uint4* __restrict__ x,
-                                                                const int32_t* __restrict__ perm,
-                                                                const int32_t* __restrict__ offsets, int rows, int E,
-                                                                int row16, ScalePtrs sp, uint2* __restrict__ out) {
+// Quantise the rows the expert GEMMs read: sorted rows [0, rows_routed) gather token perm[r]/2 with the
+// scale_input of the expert whose segment holds r; rows [rows_routed, rows_total) are the token-order copy for
+// the shared expert. Two rows per wave and iteration keep 2 x NCH 16-byte loads per lane in flight.
+// NCH * 64 == row16 selects the unrolled path, NCH == 0 the generic one.
+template <int NCH>
+__global__ __launch_bounds__(THREADS) void quant_dispatch_kernel(const uint4* __restrict__ x,
+                                                                 const int32_t* __restrict__ perm,
+                                                                 const int32_t* __restrict__ offsets, int rows_routed,
+                                                                 int rows_total, int E, int row16, ScalePtrs sp,
+                                                                 const float* shared_scale, uint2* __restrict__ out) {
   const int lane = threadIdx.x & 63;
   const int wave = blockIdx.x * WAVES + (threadIdx.x >> 6);
   const int nwaves = gridDim.x * WAVES;
-  for (int r = wave; r < rows; r += nwaves) {
-    const long t = perm[r] / HDMOE_TOPK;
-    int e = 0;
-    while (e + 1 < E && r >= offsets[e + 1]) ++e;
-    const float inv = inv_scale(sp.p[e]);
-    for (int u = lane; u < row16; u += 64) out[(long)r * row16 + u] = quant8(x[t * row16 + u], inv);
+  for (int r0 = wave * 2; r0 < rows_total; r0 += nwaves * 2) {
+    long t[2];
+    float inv[2];
+    bool ok[2];
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+      const int r = r0 + k;
+      ok[k] = r < rows_total;
+      t[k] = 0;
+      inv[k] = 1.0f;
+      if (!ok[k]) continue;
+      if (r < rows_routed) {
+        t[k] = perm[r] / HDMOE_TOPK;
+        int e = 0;
+        while (e + 1 < E && r >= offsets[e + 1]) ++e;
+        inv[k] = inv_scale(sp.p[e]);
+      } else {
+        t[k] = r - rows_routed;
+        inv[k] = inv_scale(shared_scale);
+      }
+    }
+    if constexpr (NCH > 0) {
+      uint4 v[2][NCH];
+#pragma unroll
+      for (int k = 0; k < 2; ++k)
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) v[k][c] = ok[k] ? x[t[k] * row16 + c * 64 + lane] : make_uint4(0, 0, 0, 0);
+#pragma unroll
+      for (int k = 0; k < 2; ++k)
+        if (ok[k]) {
+#pragma unroll
+          for (int c = 0; c < NCH; ++c) out[(long)(r0 + k) * row16 + c * 64 + lane] = quant8(v[k][c], inv[k]);
+        }
+    } else {
+#pragma unroll
+      for (int k = 0; k < 2; ++k)
+        if (ok[k])
+          for (int u = lane; u < row16; u += 64) out[(long)(r0 + k) * row16 + u] = quant8(x[t[k] * row16 + u], inv[k]);
+    }
   }
 }
 
@@ -182,6 +221,27 @@ inline int row_blocks(long rows) {
 
 }  // namespace
 
+// One launch for the routed rows [0,2T) and, optionally, the shared expert's token-order rows [2T,3T) of a_fp8.
+int hdmoe_launch_quant_dispatch(const void* x_bf16, const int32_t* perm, const int32_t* offsets, int T, int D, int E,
+                                const float* const* scale_input, const float* shared_scale, bool with_shared,
+                                void* a_fp8, hipStream_t s, const char* what) {
+  ScalePtrs sp;
+  for (int e = 0; e < HDMOE_MAX_EXPERTS; ++e) sp.p[e] = e < E ? scale_input[e] : nullptr;
+  const int rows_routed = T * HDMOE_TOPK;
+  const int rows_total = rows_routed + (with_shared ? T : 0);
+  const int row16 = D / 8;
+  const dim3 grid(row_blocks((rows_total + 1) / 2)), block(THREADS);
+  const uint4* xp = static_cast<const uint4*>(x_bf16);
+  uint2* op = static_cast<uint2*>(a_fp8);
+  if (row16 == 5 * 64)
+    hipLaunchKernelGGL(quant_dispatch_kernel<5>, grid, block, 0, s, xp, perm, offsets, rows_routed, rows_total, E, row16,
+                       sp, shared_scale, op);
+  else
+    hipLaunchKernelGGL(quant_dispatch_kernel<0>, grid, block, 0, s, xp, perm, offsets, rows_routed, rows_total, E, row16,
+                       sp, shared_scale, op);
+  return hdmoe_check_launch(what);
+}
+
 extern "C" int hdmoe_quant_fp8(const void* x_bf16, int64_t rows, int D, const float* scale_input_dev, void* out_fp8,
                                hdmoe_stream_t stream) {
   HDMOE_REQUIRE_PTR(x_bf16);
@@ -208,11 +268,8 @@ extern "C" int hdmoe_quant_permute_fp8(const void* x_bf16, const int32_t* perm, 
   if (T == 0) return HDMOE_OK;
   ScalePtrs sp;
   for (int e = 0; e < HDMOE_MAX_EXPERTS; ++e) sp.p[e] = e < E ? scale_input[e] : nullptr;
-  const int rows = T * HDMOE_TOPK;
-  hipLaunchKernelGGL(quant_permute_kernel, dim3(row_blocks(rows)), dim3(THREADS), 0,
-                     static_cast<hipStream_t>(stream), static_cast<const uint4*>(x_bf16), perm, offsets, rows, E,
-                     D / 8, sp, static_cast<uint2*>(a_fp8));
-  return hdmoe_check_launch("hdmoe_quant_permute_fp8");
+  return hdmoe_launch_quant_dispatch(x_bf16, perm, offsets, T, D, E, scale_input, nullptr, false, a_fp8,
+                                     static_cast<hipStream_t>(stream), "hdmoe_quant_permute_fp8");
 }
 
 extern "C" int hdmoe_permute_bf16(const void* x_bf16, const int32_t* perm, int T, int D, void* a_bf16,

@@ -131,7 +131,12 @@ __global__ __launch_bounds__(WAVES_PER_BLOCK * 64) void gate_top2_reg_kernel(
     for (int e = 0; e < E; ++e) {
       float acc = 0.0f;
 #pragma unroll
-      for (int c = 0; c < NCHUNK; ++c) acc = dot8(cur[c], w[e][c], acc);
+      for (int c = 0; c < NCHUNK; ++c) {
+        // keep the weight slice packed (bf16 pairs): without this the compiler hoists the unpacking out of the
+        // token loop and doubles the register footprint, which halves the waves in flight
+        asm volatile("" : "+v"(w[e][c].x), "+v"(w[e][c].y), "+v"(w[e][c].z), "+v"(w[e][c].w));
+        acc = dot8(cur[c], w[e][c], acc);
+      }
       logit[e] = acc;
     }
     finish_token<E>(logit, lane, t, idx, wout);
@@ -164,8 +169,8 @@ __global__ __launch_bounds__(WAVES_PER_BLOCK * 64) void gate_top2_generic_kernel
 
 template <int E>
 int launch_gate(const void* x, const void* wg, int T, int D, int32_t* idx, void* w, hipStream_t s) {
-  // about 8 tokens per wave amortise the register-resident weight slice
-  int blocks = (T + WAVES_PER_BLOCK * 8 - 1) / (WAVES_PER_BLOCK * 8);
+  // about 4 tokens per wave amortise the register-resident weight slice and still give 8 waves per CU at T = 8192
+  int blocks = (T + WAVES_PER_BLOCK * 4 - 1) / (WAVES_PER_BLOCK * 4);
   if (blocks < 1) blocks = 1;
   if (blocks > HDMOE_NUM_CU * 8) blocks = HDMOE_NUM_CU * 8;
   dim3 grid(blocks), block(WAVES_PER_BLOCK * 64);

@@ -9,6 +9,9 @@ int hdmoe_launch_ffn_gemm(bool swiglu, int weight_dtype, const uint8_t* a_dyn, c
                           int rows_static, const hdmoe_ffn_weights* shared, uint8_t* out_static, int K_dyn, int N_dyn,
                           int K_static, int N_static, hipStream_t s, const char* what);
 int hdmoe_check_gemm_shape(const char* what, int weight_dtype, long rows, int K, int N, int feat_per_tile);
+int hdmoe_launch_quant_dispatch(const void* x_bf16, const int32_t* perm, const int32_t* offsets, int T, int D, int E,
+                                const float* const* scale_input, const float* shared_scale, bool with_shared,
+                                void* a_fp8, hipStream_t s, const char* what);
 
 char* hdmoe_error_buffer() {
   static thread_local char buf[HDMOE_ERRBUF] = {0};
@@ -101,7 +104,7 @@ extern "C" int hdmoe_moe_ffn(const hdmoe_layer_args* p, hdmoe_stream_t stream) {
 
   int ev = 0;
   auto mark = [&]() {
-    if (p->stage_events) hipEventRecord(static_cast<hipEvent_t>(p->stage_events[ev]), s);
+    if (p->stage_events) (void)hipEventRecord(static_cast<hipEvent_t>(p->stage_events[ev]), s);
     ++ev;
   };
   mark();
@@ -116,11 +119,11 @@ extern "C" int hdmoe_moe_ffn(const hdmoe_layer_args* p, hdmoe_stream_t stream) {
   if (fp8) {
     const float* sin[HDMOE_MAX_EXPERTS];
     for (int e = 0; e < E; ++e) sin[e] = p->experts[e].scale_in1;
-    if (int rc = hdmoe_quant_permute_fp8(p->x, perm, offsets, T, D, E, sin, a_routed, stream)) return rc;
-    if (Hs > 0) {
-      if (int rc = hdmoe_quant_fp8(p->x, T, D, p->shared->scale_in1, a_shared, stream)) return rc;
-      a_static = a_shared;
-    }
+    // routed rows and the shared expert's token-order copy in one launch ([2T,D] then [T,D] of the same buffer)
+    if (int rc = hdmoe_launch_quant_dispatch(p->x, perm, offsets, T, D, E, sin, Hs > 0 ? p->shared->scale_in1 : nullptr,
+                                             Hs > 0, a_routed, s, "hdmoe_moe_ffn (quantise)"))
+      return rc;
+    if (Hs > 0) a_static = a_shared;
   } else {
     if (int rc = hdmoe_permute_bf16(p->x, perm, T, D, a_routed, stream)) return rc;
     a_static = static_cast<const uint8_t*>(p->x);

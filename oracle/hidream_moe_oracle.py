@@ -76,7 +76,7 @@ def e4m3fn_decode(b_u8):
 
 
 def quantize_weight_per_tensor(w_f32):
-    """BASELINE.json configs[1]: scale_weight = amax/448, W8 = (W/scale_weight) -> e4m3fn.
+    """Per-tensor weight quantisation of the scaled-fp8 benchmark layers: scale_weight = amax/448, W8 = (W/scale_weight) -> e4m3fn.
     Returns (W8 as torch.float8_e4m3fn, scale_weight fp32 scalar tensor)."""
     w = w_f32.to(torch.float32)
     s = (w.abs().amax() / 448.0).to(torch.float32)
