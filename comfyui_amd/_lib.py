@@ -77,6 +77,9 @@ SIGNATURES = {
     "hdmoe_combine": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p]),
     "hdmoe_layer_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int, c_int]),
     "hdmoe_moe_ffn": (c_int, [ctypes.POINTER(LayerArgs), c_void_p]),
+    "hdmoe_ffn_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
+    "hdmoe_ffn_swiglu": (c_int, [c_int, c_void_p, c_int, c_int, c_int, ctypes.POINTER(FfnWeights), c_void_p, c_void_p,
+                                 c_size_t, c_void_p]),
     "hdmoe_layer_layout_get": (c_int, [c_int, c_int, c_int, c_int, c_int, c_int, ctypes.POINTER(LayerLayout)]),
 }
 

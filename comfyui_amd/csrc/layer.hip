@@ -144,3 +144,44 @@ extern "C" int hdmoe_moe_ffn(const hdmoe_layer_args* p, hdmoe_stream_t stream) {
   mark();
   return rc;
 }
+
+extern "C" size_t hdmoe_ffn_workspace_bytes(int rows, int D, int H, int weight_dtype) {
+  if (rows < 0 || D <= 0 || H <= 0 || (weight_dtype != HDMOE_W_BF16 && weight_dtype != HDMOE_W_E4M3FN)) return 0;
+  const size_t eb = weight_dtype == HDMOE_W_E4M3FN ? 1 : 2;
+  // fp8: quantised copy of x, then h; bf16: h only (x itself is the GEMM operand)
+  const size_t a = weight_dtype == HDMOE_W_E4M3FN ? hdmoe_align_up((size_t)rows * D * eb, 256) : 0;
+  return a + hdmoe_align_up((size_t)rows * H * eb, 256);
+}
+
+extern "C" int hdmoe_ffn_swiglu(int weight_dtype, const void* x_bf16, int rows, int D, int H,
+                                const hdmoe_ffn_weights* w, void* out_bf16, void* workspace, size_t workspace_bytes,
+                                hdmoe_stream_t stream) {
+  HDMOE_REQUIRE_PTR(x_bf16);
+  HDMOE_REQUIRE_PTR(w);
+  HDMOE_REQUIRE_PTR(out_bf16);
+  HDMOE_REQUIRE_PTR(workspace);
+  if (int rc = hdmoe_check_gemm_shape("hdmoe_ffn_swiglu (gate/up)", weight_dtype, rows, D, H, 128)) return rc;
+  if (int rc = hdmoe_check_gemm_shape("hdmoe_ffn_swiglu (down)", weight_dtype, rows, H, D, 256)) return rc;
+  const size_t need = hdmoe_ffn_workspace_bytes(rows, D, H, weight_dtype);
+  if (workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255))
+    return hdmoe_fail(HDMOE_E_WORKSPACE, "hdmoe_ffn_swiglu: workspace %zu bytes, need %zu (256-byte aligned)",
+                      workspace_bytes, need);
+  if (rows == 0) return HDMOE_OK;
+  const bool fp8 = weight_dtype == HDMOE_W_E4M3FN;
+  if (fp8 && w->scale_in1 != w->scale_in3 && (w->scale_in1 == nullptr || w->scale_in3 == nullptr))
+    return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_ffn_swiglu: w1 and w3 disagree on having a scale_input");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  uint8_t* ws = static_cast<uint8_t*>(workspace);
+  const uint8_t* a = static_cast<const uint8_t*>(x_bf16);
+  uint8_t* h = ws;
+  if (fp8) {
+    if (int rc = hdmoe_quant_fp8(x_bf16, rows, D, w->scale_in1, ws, stream)) return rc;
+    a = ws;
+    h = ws + hdmoe_align_up((size_t)rows * D, 256);
+  }
+  if (int rc = hdmoe_launch_ffn_gemm(true, weight_dtype, nullptr, nullptr, 0, 0, nullptr, nullptr, a, rows, w, h, 0, 0, D, H,
+                                     s, "hdmoe_ffn_swiglu (gate/up)"))
+    return rc;
+  return hdmoe_launch_ffn_gemm(false, weight_dtype, nullptr, nullptr, 0, 0, nullptr, nullptr, h, rows, w,
+                               static_cast<uint8_t*>(out_bf16), 0, 0, H, D, s, "hdmoe_ffn_swiglu (down)");
+}

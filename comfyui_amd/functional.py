@@ -185,6 +185,20 @@ def grouped_down(h, offsets, experts, D):
     return y
 
 
+def ffn_swiglu(x2d, weights, H, weight_dtype):
+    """One dense SwiGLU feed-forward as three enqueues. weights: FfnWeights. x2d [rows,D] bf16 -> [rows,D] bf16."""
+    _need_hip(x2d, "ffn_swiglu x", BF16)
+    rows, D = x2d.shape
+    code = weight_dtype_code(weight_dtype)
+    nbytes = lib.hdmoe_ffn_workspace_bytes(rows, D, H, code)
+    ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=x2d.device)
+    out = torch.empty((rows, D), dtype=BF16, device=x2d.device)
+    fw = FfnWeights.from_buffer_copy(weights)
+    check(lib.hdmoe_ffn_swiglu(code, ptr(x2d), rows, D, H, ctypes.byref(fw), ptr(out), ptr(ws), ws.numel(),
+                               _stream(x2d)))
+    return out
+
+
 def layer_layout(T, D, H, Hs, E, code):
     lay = LayerLayout()
     check(lib.hdmoe_layer_layout_get(T, D, H, Hs, E, code, ctypes.byref(lay)))

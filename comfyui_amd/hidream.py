@@ -28,6 +28,77 @@ FP8 = torch.float8_e4m3fn
 BF16 = torch.bfloat16
 
 
+_scale_cache = {}
+
+
+def _scale_value(p):
+    """Host copy of an fp32 scalar Parameter, cached on (identity, version, address): read once per parameter
+    object, so steady-state forwards do not synchronise."""
+    key = (id(p), p._version, p.data_ptr())
+    v = _scale_cache.get(key)
+    if v is None:
+        if len(_scale_cache) > 4096:
+            _scale_cache.clear()
+        v = float(p.detach().float().cpu())
+        _scale_cache[key] = v
+    return v
+
+
+def _plain(lin):
+    return (len(getattr(lin, "weight_function", ())) == 0 and len(getattr(lin, "bias_function", ())) == 0
+            and lin.bias is None)
+
+
+def _pack_ffn(ffn, x, wdt, keep):
+    """hdmoe_ffn_weights for one FeedForwardSwiGLU whose Linears store `wdt`, or None when the three Linears
+    cannot be served by the fused kernels (w1/w3 quantising the same input with different scale_input values).
+    Tensors that must outlive the call are appended to `keep`."""
+    fp8 = wdt == FP8
+    dev = x.device
+    scales = {}
+    ws = []
+    for name, l in (("1", ffn.w1), ("2", ffn.w2), ("3", ffn.w3)):
+        if _plain(l) and l.weight.device == dev:
+            w = l.weight
+        else:
+            w, _ = amd_ops.cast_bias_weight(l, x, dtype=wdt)   # offloaded weights, weight functions (LowVramPatch)
+        w = w.contiguous()
+        keep.append(w)
+        ws.append(w)
+        if fp8:
+            sw = getattr(l, "scale_weight", None)
+            sw = amd_ops._one(dev) if sw is None else sw.to(dev)
+            si = getattr(l, "scale_input", None)
+            if si is not None:
+                si = si.to(dev)
+                keep.append(si)
+            keep.append(sw)
+            scales["scale_w" + name] = sw
+            scales["scale_in" + name] = si
+    if fp8:
+        s1, s3 = scales["scale_in1"], scales["scale_in3"]
+        if (s1 is None) != (s3 is None):
+            return None
+        if s1 is not None and s1.data_ptr() != s3.data_ptr() and _scale_value(s1) != _scale_value(s3):
+            return None  # w1 and w3 quantise the same input differently: one fp8 copy cannot serve both
+    return HF.make_ffn_weights(ws[0], ws[1], ws[2], scales)
+
+
+def _fusable_dtype(ffns):
+    """Common storage dtype of all Linears if the fused kernels can run them, else None."""
+    lins = [l for f in ffns for l in (f.w1, f.w2, f.w3)]
+    for l in lins:
+        # any Linear that follows the operations contract (this package's or ComfyUI's own classes)
+        if not isinstance(l, torch.nn.Linear) or l.bias is not None or len(getattr(l, "bias_function", ())) > 0:
+            return None
+    wdt = lins[0].weight.dtype
+    if wdt not in (BF16, FP8) or any(l.weight.dtype != wdt for l in lins):
+        return None
+    if wdt == FP8 and not all(getattr(l, "hdmoe_fp8_matrix_mult", isinstance(l, amd_ops.fp8_ops.Linear)) for l in lins):
+        return None  # scaled fp8 without fp8 matrix multiply: dequantising Linear path
+    return wdt
+
+
 class FeedForwardSwiGLU(nn.Module):
     def __init__(self, dim: int, hidden_dim: int, multiple_of: int = 256,
                  ffn_dim_multiplier: Optional[float] = None, dtype=None, device=None, operations=None):
@@ -42,6 +113,17 @@ class FeedForwardSwiGLU(nn.Module):
         self.w3 = operations.Linear(dim, hidden_dim, bias=False, dtype=dtype, device=device)
 
     def forward(self, x):
+        if x.is_cuda and x.dtype == BF16:
+            wdt = _fusable_dtype([self])
+            if wdt is not None:
+                x2 = x.reshape(-1, x.shape[-1]).contiguous()
+                keep = []
+                packed = _pack_ffn(self, x2, wdt, keep)
+                if packed is not None:
+                    y = HF.ffn_swiglu(x2, packed, self.w1.weight.shape[0], wdt)
+                    del keep
+                    return y.view(*x.shape[:-1], self.w2.weight.shape[0])
+        # per-Linear composition (also the place where a CPU tensor is refused)
         return self.w2(HF.silu_mul(self.w1(x), self.w3(x)))
 
 
@@ -81,11 +163,6 @@ class MoEGate(nn.Module):
         return idx.to(torch.int64), w, None
 
 
-def _plain(lin):
-    return (len(getattr(lin, "weight_function", ())) == 0 and len(getattr(lin, "bias_function", ())) == 0
-            and lin.bias is None)
-
-
 class MOEFeedForwardSwiGLU(nn.Module):
     def __init__(self, dim: int, hidden_dim: int, num_routed_experts: int, num_activated_experts: int,
                  dtype=None, device=None, operations=None):
@@ -97,72 +174,23 @@ class MOEFeedForwardSwiGLU(nn.Module):
                             num_activated_experts=num_activated_experts, dtype=dtype, device=device,
                             operations=operations)
         self.num_activated_experts = num_activated_experts
-        self._scale_cache = {}
 
     # ---- fused path ----------------------------------------------------------------
-
-    def _scale_value(self, p):
-        """Host copy of an fp32 scalar Parameter, cached on (identity, version): read once per
-        parameter object, so steady-state forwards do not synchronise."""
-        key = (id(p), p._version, p.data_ptr())
-        v = self._scale_cache.get(key)
-        if v is None:
-            if len(self._scale_cache) > 256:
-                self._scale_cache.clear()
-            v = float(p.detach().float().cpu())
-            self._scale_cache[key] = v
-        return v
 
     def _collect(self, x):
         """Device pointers of all 15 Linears for the one-call path, or None when the layer
         needs the per-Linear composition. Returned tensors are kept alive by the caller."""
         ffns = list(self.experts) + [self.shared_experts]
-        lins = [l for f in ffns for l in (f.w1, f.w2, f.w3)]
-        for l in lins:
-            # any Linear that follows the operations contract (this package's or ComfyUI's own classes)
-            if not isinstance(l, torch.nn.Linear) or l.bias is not None or len(getattr(l, "bias_function", ())) > 0:
-                return None
-        wdt = lins[0].weight.dtype
-        if wdt not in (BF16, FP8) or any(l.weight.dtype != wdt for l in lins):
+        wdt = _fusable_dtype(ffns)
+        if wdt is None:
             return None
-        fp8 = wdt == FP8
-        if fp8 and not all(getattr(l, "hdmoe_fp8_matrix_mult", isinstance(l, amd_ops.fp8_ops.Linear)) for l in lins):
-            return None  # scaled fp8 without fp8 matrix multiply: dequantising Linear path
-        dev = x.device
         keep = []
         packed = []
-        one = None
         for f in ffns:
-            scales = {}
-            ws = []
-            for name, l in (("1", f.w1), ("2", f.w2), ("3", f.w3)):
-                if _plain(l) and l.weight.device == dev:
-                    w = l.weight
-                else:
-                    w, _ = amd_ops.cast_bias_weight(l, x, dtype=wdt)
-                w = w.contiguous()
-                keep.append(w)
-                ws.append(w)
-                if fp8:
-                    sw = getattr(l, "scale_weight", None)
-                    if sw is None:
-                        one = one if one is not None else amd_ops._one(dev)
-                        sw = one
-                    sw = sw.to(dev)
-                    si = getattr(l, "scale_input", None)
-                    if si is not None:
-                        si = si.to(dev)
-                        keep.append(si)
-                    keep.append(sw)
-                    scales["scale_w" + name] = sw
-                    scales["scale_in" + name] = si
-            if fp8:
-                s1, s3 = scales["scale_in1"], scales["scale_in3"]
-                if (s1 is None) != (s3 is None):
-                    return None
-                if s1 is not None and s1.data_ptr() != s3.data_ptr() and self._scale_value(s1) != self._scale_value(s3):
-                    return None  # w1 and w3 quantise the same input differently: cannot share one fp8 copy
-            packed.append(HF.make_ffn_weights(ws[0], ws[1], ws[2], scales))
+            fw = _pack_ffn(f, x, wdt, keep)
+            if fw is None:
+                return None
+            packed.append(fw)
         return wdt, packed[:-1], packed[-1], keep
 
     def forward(self, x, stage_events=None):

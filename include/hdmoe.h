@@ -186,6 +186,16 @@ typedef struct hdmoe_layer_args {
 size_t hdmoe_layer_workspace_bytes(int T, int D, int H, int Hs, int E, int weight_dtype);
 int hdmoe_moe_ffn(const hdmoe_layer_args* args, hdmoe_stream_t stream);
 
+/* FeedForwardSwiGLU.forward, model.py:237-238, for one dense FFN (the shared expert on its own, the text-token
+ * feed-forward, or a block built with num_routed_experts == 0): out = w2( silu(w1 x) * w3 x ) with the same
+ * per-Linear semantics as above. x [rows,D] bf16 -> out [rows,D] bf16. Three launches (fp8: quantise, gate/up GEMM
+ * with the SiLU*mul epilogue, down GEMM; bf16: the two GEMMs). workspace: hdmoe_ffn_workspace_bytes(...) bytes,
+ * 256-byte aligned, device. */
+size_t hdmoe_ffn_workspace_bytes(int rows, int D, int H, int weight_dtype);
+int hdmoe_ffn_swiglu(int weight_dtype, const void* x_bf16, int rows, int D, int H,
+                     const hdmoe_ffn_weights* w, void* out_bf16, void* workspace,
+                     size_t workspace_bytes, hdmoe_stream_t stream);
+
 /* Where the pieces of the workspace live, for tests that inspect intermediates. */
 typedef struct hdmoe_layer_layout {
   size_t topk_idx, topk_weight, counts, offsets, perm, inv_perm, dispatch_ws;

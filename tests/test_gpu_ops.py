@@ -196,3 +196,25 @@ def test_stacked_layers_at_32768_tokens(dev):
         assert not bool(got.float().isnan().any())
         assert met["rel_rms"] <= 1e-2 and met["max_over_max"] <= 3e-2, met
         del m
+
+
+@pytest.mark.parametrize("weights", ["fp8", "bf16"])
+@pytest.mark.parametrize("rows", [1, 300, 1025])
+def test_dense_swiglu_ffn(dev, weights, rows):
+    """FeedForwardSwiGLU on its own (shared expert / text-token feed-forward): one quantise + two GEMM launches."""
+    dim = 512
+    sd, _ = small_layer(seed=50, dim=dim, tokens=8, weights=weights)
+    m = synth.build_module({k: v.to(dev) for k, v in sd.items()}, weights, dev, dim=dim)
+    g = torch.Generator().manual_seed(rows)
+    x = torch.randn((rows, dim), generator=g).to(BF16)
+    ffn = m.shared_experts
+    y = ffn(x.to(dev))
+    assert y.shape == x.shape and y.dtype == BF16
+    params = oracle_params(sd, 4)
+    ref = O.ffn_swiglu(x, params["shared"], "fp8mm" if weights == "fp8" else "plain")
+    close(y.cpu(), ref, 1e-2 if weights == "fp8" else 4e-3)
+    # the per-Linear composition gives the same result
+    y2 = ffn.w2(__import__("comfyui_amd").functional.silu_mul(ffn.w1(x.to(dev)), ffn.w3(x.to(dev))))
+    close(y2.cpu(), y.cpu(), 3e-3)
+    # 3-D input keeps its shape
+    assert ffn(x.to(dev).view(1, rows, dim)).shape == (1, rows, dim)
