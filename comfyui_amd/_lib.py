@@ -45,6 +45,8 @@ class LayerArgs(ctypes.Structure):
         ("out", c_void_p), ("workspace", c_void_p), ("workspace_bytes", c_size_t),
         ("topk_idx", c_void_p), ("topk_weight", c_void_p),
         ("stage_events", ctypes.POINTER(c_void_p)),
+        ("mod_scale", c_void_p), ("mod_shift", c_void_p), ("mod_gate", c_void_p),
+        ("tokens_per_batch", c_int), ("ln_eps", ctypes.c_float),
     ]
 
 
@@ -52,7 +54,7 @@ class LayerLayout(ctypes.Structure):
     """hdmoe_layer_layout"""
     _fields_ = [(n, c_size_t) for n in
                 ("topk_idx", "topk_weight", "counts", "offsets", "perm", "inv_perm", "dispatch_ws",
-                 "a", "h", "y", "total")]
+                 "a", "h", "y", "normed", "total")]
 
 
 # name -> (restype, argtypes); every symbol include/hdmoe.h declares
@@ -74,6 +76,10 @@ SIGNATURES = {
     "hdmoe_linear": (c_int, [c_int, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "hdmoe_silu_mul_bf16": (c_int, [c_void_p, c_void_p, c_int64, c_void_p, c_void_p]),
     "hdmoe_scale_to_bf16": (c_int, [c_int, c_void_p, c_int64, c_void_p, c_void_p, c_void_p]),
+    "hdmoe_ln_modulate_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, ctypes.c_float, c_void_p,
+                                       c_void_p]),
+    "hdmoe_combine_gated_residual": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
+                                             c_int, c_void_p, c_void_p]),
     "hdmoe_combine": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p]),
     "hdmoe_layer_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int, c_int]),
     "hdmoe_moe_ffn": (c_int, [ctypes.POINTER(LayerArgs), c_void_p]),

@@ -145,38 +145,52 @@ __global__ __launch_bounds__(THREADS) void silu_mul_kernel(const uint4* __restri
 // (/root/reference/comfy/ldm/hidream/model.py:319,324): each product is rounded to
 // bf16, the two-term sum is formed in fp32 and rounded, then the shared row is added
 // and the result rounded again.
-__device__ __forceinline__ float comb1(float y0, float y1, float w0, float w1, float sh, bool has_shared) {
+// Optional block epilogue on top: bf16( bf16(gate_mlp * .) + residual )  (model.py:432-433, 520-522).
+struct CombineExtra {
+  const uint4* gate;      // [B, D] bf16 or NULL
+  const uint4* residual;  // [T, D] bf16 (only read when gate != NULL)
+  int tokens_per_batch;
+};
+
+__device__ __forceinline__ float comb1(float y0, float y1, float w0, float w1, float sh, bool has_shared, float g,
+                                       float res, bool has_gate) {
   float s = round_bf16(round_bf16(y0 * w0) + round_bf16(y1 * w1));
-  return has_shared ? s + sh : s;
+  if (has_shared) s = has_gate ? round_bf16(s + sh) : s + sh;
+  if (has_gate) s = round_bf16(g * s) + res;
+  return s;
 }
 
-__device__ __forceinline__ uint32_t comb2(uint32_t y0, uint32_t y1, float w0, float w1, uint32_t sh, bool hs) {
-  return pack_bf16(comb1(bf16_lo(y0), bf16_lo(y1), w0, w1, bf16_lo(sh), hs),
-                   comb1(bf16_hi(y0), bf16_hi(y1), w0, w1, bf16_hi(sh), hs));
+__device__ __forceinline__ uint32_t comb2(uint32_t y0, uint32_t y1, float w0, float w1, uint32_t sh, bool hs, uint32_t g,
+                                          uint32_t res, bool hg) {
+  return pack_bf16(comb1(bf16_lo(y0), bf16_lo(y1), w0, w1, bf16_lo(sh), hs, bf16_lo(g), bf16_lo(res), hg),
+                   comb1(bf16_hi(y0), bf16_hi(y1), w0, w1, bf16_hi(sh), hs, bf16_hi(g), bf16_hi(res), hg));
 }
 
 __global__ __launch_bounds__(THREADS) void combine_kernel(const uint4* __restrict__ y, const int2* __restrict__ inv_perm,
                                                           const uint32_t* __restrict__ w, const uint4* __restrict__ shared,
-                                                          int T, int row16, uint4* __restrict__ out) {
+                                                          int T, int row16, CombineExtra ex, uint4* __restrict__ out) {
   const int lane = threadIdx.x & 63;
   const int wave = blockIdx.x * WAVES + (threadIdx.x >> 6);
   const int nwaves = gridDim.x * WAVES;
   const bool hs = shared != nullptr;
+  const bool hg = ex.gate != nullptr;
   for (int t = wave; t < T; t += nwaves) {
     const int2 r = inv_perm[t];
     const uint32_t wp = w[t];
     const float w0 = bf16_lo(wp), w1 = bf16_hi(wp);
     const uint4* y0 = y + (long)r.x * row16;
     const uint4* y1 = y + (long)r.y * row16;
+    const long brow = hg ? (long)(t / ex.tokens_per_batch) * row16 : 0;
     for (int u = lane; u < row16; u += 64) {
       const uint4 a = y0[u], b = y1[u];
-      uint4 sh = make_uint4(0, 0, 0, 0);
+      uint4 sh = make_uint4(0, 0, 0, 0), g = sh, res = sh;
       if (hs) sh = shared[(long)t * row16 + u];
+      if (hg) { g = ex.gate[brow + u]; res = ex.residual[(long)t * row16 + u]; }
       uint4 o;
-      o.x = comb2(a.x, b.x, w0, w1, sh.x, hs);
-      o.y = comb2(a.y, b.y, w0, w1, sh.y, hs);
-      o.z = comb2(a.z, b.z, w0, w1, sh.z, hs);
-      o.w = comb2(a.w, b.w, w0, w1, sh.w, hs);
+      o.x = comb2(a.x, b.x, w0, w1, sh.x, hs, g.x, res.x, hg);
+      o.y = comb2(a.y, b.y, w0, w1, sh.y, hs, g.y, res.y, hg);
+      o.z = comb2(a.z, b.z, w0, w1, sh.z, hs, g.z, res.z, hg);
+      o.w = comb2(a.w, b.w, w0, w1, sh.w, hs, g.w, res.w, hg);
       out[(long)t * row16 + u] = o;
     }
   }
@@ -302,6 +316,19 @@ extern "C" int hdmoe_silu_mul_bf16(const void* a_bf16, const void* b_bf16, int64
   return hdmoe_check_launch("hdmoe_silu_mul_bf16");
 }
 
+int hdmoe_launch_combine(const void* y_sorted_bf16, const int32_t* inv_perm, const void* topk_weight_bf16,
+                         const void* shared_bf16, const void* gate_bf16, const void* residual_bf16, int tokens_per_batch,
+                         int T, int D, void* out_bf16, hipStream_t s, const char* what) {
+  CombineExtra ex;
+  ex.gate = static_cast<const uint4*>(gate_bf16);
+  ex.residual = static_cast<const uint4*>(residual_bf16);
+  ex.tokens_per_batch = tokens_per_batch > 0 ? tokens_per_batch : 1;
+  hipLaunchKernelGGL(combine_kernel, dim3(row_blocks(T)), dim3(THREADS), 0, s, static_cast<const uint4*>(y_sorted_bf16),
+                     reinterpret_cast<const int2*>(inv_perm), static_cast<const uint32_t*>(topk_weight_bf16),
+                     static_cast<const uint4*>(shared_bf16), T, D / 8, ex, static_cast<uint4*>(out_bf16));
+  return hdmoe_check_launch(what);
+}
+
 extern "C" int hdmoe_combine(const void* y_sorted_bf16, const int32_t* inv_perm, const void* topk_weight_bf16,
                              const void* shared_bf16, int T, int D, void* out_bf16, hdmoe_stream_t stream) {
   HDMOE_REQUIRE_PTR(y_sorted_bf16);
@@ -310,11 +337,26 @@ extern "C" int hdmoe_combine(const void* y_sorted_bf16, const int32_t* inv_perm,
   HDMOE_REQUIRE_PTR(out_bf16);
   if (T < 0 || D <= 0 || D % 8 != 0) return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_combine: T=%d D=%d", T, D);
   if (T == 0) return HDMOE_OK;
-  hipLaunchKernelGGL(combine_kernel, dim3(row_blocks(T)), dim3(THREADS), 0, static_cast<hipStream_t>(stream),
-                     static_cast<const uint4*>(y_sorted_bf16), reinterpret_cast<const int2*>(inv_perm),
-                     static_cast<const uint32_t*>(topk_weight_bf16), static_cast<const uint4*>(shared_bf16), T, D / 8,
-                     static_cast<uint4*>(out_bf16));
-  return hdmoe_check_launch("hdmoe_combine");
+  return hdmoe_launch_combine(y_sorted_bf16, inv_perm, topk_weight_bf16, shared_bf16, nullptr, nullptr, 1, T, D, out_bf16,
+                              static_cast<hipStream_t>(stream), "hdmoe_combine");
+}
+
+extern "C" int hdmoe_combine_gated_residual(const void* y_sorted_bf16, const int32_t* inv_perm,
+                                            const void* topk_weight_bf16, const void* shared_bf16,
+                                            const void* gate_bf16, const void* residual_bf16, int tokens_per_batch,
+                                            int T, int D, void* out_bf16, hdmoe_stream_t stream) {
+  HDMOE_REQUIRE_PTR(y_sorted_bf16);
+  HDMOE_REQUIRE_PTR(inv_perm);
+  HDMOE_REQUIRE_PTR(topk_weight_bf16);
+  HDMOE_REQUIRE_PTR(gate_bf16);
+  HDMOE_REQUIRE_PTR(residual_bf16);
+  HDMOE_REQUIRE_PTR(out_bf16);
+  if (T < 0 || D <= 0 || D % 8 != 0 || tokens_per_batch <= 0)
+    return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_combine_gated_residual: T=%d D=%d tokens_per_batch=%d", T, D, tokens_per_batch);
+  if (T == 0) return HDMOE_OK;
+  return hdmoe_launch_combine(y_sorted_bf16, inv_perm, topk_weight_bf16, shared_bf16, gate_bf16, residual_bf16,
+                              tokens_per_batch, T, D, out_bf16, static_cast<hipStream_t>(stream),
+                              "hdmoe_combine_gated_residual");
 }
 
 extern "C" int hdmoe_scale_to_bf16(int src_dtype, const void* src, int64_t n, const float* scale_dev, void* out_bf16,

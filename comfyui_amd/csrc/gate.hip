@@ -185,6 +185,105 @@ int launch_gate(const void* x, const void* wg, int T, int D, int32_t* idx, void*
   return hdmoe_check_launch("hdmoe_gate_top2");
 }
 
+// ---- LayerNorm (no affine) + adaLN modulation in front of the feed-forward -----------------------------
+// n = bf16(LayerNorm(x)); out = bf16( bf16(n * bf16(1 + scale[b])) + shift[b] ), b = token / tokens_per_batch
+// (/root/reference/comfy/ldm/hidream/model.py:430-431, 516-517). One token per wave, same lane/element mapping
+// as the gate kernel; mean and variance are two passes over the registers with the same fixed fp32 order
+// (per-lane ascending elements, then the xor butterfly), so the CPU checker can restate it bit for bit.
+// The root is __builtin_sqrtf, which hipcc rounds correctly; __fsqrt_rn is the approximate native root here.
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) v = v + __shfl_xor(v, off, 64);
+  return v;
+}
+
+__device__ __forceinline__ void unpack8(const uint4& a, float (&f)[8]) {
+  f[0] = bf16_lo(a.x); f[1] = bf16_hi(a.x); f[2] = bf16_lo(a.y); f[3] = bf16_hi(a.y);
+  f[4] = bf16_lo(a.z); f[5] = bf16_hi(a.z); f[6] = bf16_lo(a.w); f[7] = bf16_hi(a.w);
+}
+
+__device__ __forceinline__ uint4 modulate8(const uint4& xv, const uint4& sc, const uint4& sh, float mean, float rstd) {
+  float x[8], a[8], b[8];
+  unpack8(xv, x);
+  unpack8(sc, a);
+  unpack8(sh, b);
+  uint32_t o[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    float r[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int i = 2 * j + h;
+      const float n = hdmoe_round_bf16((x[i] - mean) * rstd);     // LayerNorm output as a bf16 tensor
+      const float m = hdmoe_round_bf16(1.0f + a[i]);              // (1 + scale)
+      r[h] = hdmoe_round_bf16(hdmoe_round_bf16(n * m) + b[i]);    // n * (1 + scale) + shift
+    }
+    o[j] = (uint32_t)hdmoe_f32_to_bf16(r[0]) | ((uint32_t)hdmoe_f32_to_bf16(r[1]) << 16);
+  }
+  return make_uint4(o[0], o[1], o[2], o[3]);
+}
+
+template <int NCHUNK>  // NCHUNK * 512 == D: row held in registers; 0: any D % 8 == 0, row re-read from cache
+__global__ __launch_bounds__(WAVES_PER_BLOCK * 64) void ln_modulate_kernel(
+    const uint4* __restrict__ x, const uint4* __restrict__ scale, const uint4* __restrict__ shift, int T, int D,
+    int tokens_per_batch, float eps, uint4* __restrict__ out) {
+  const int lane = threadIdx.x & 63;
+  const int wave = blockIdx.x * WAVES_PER_BLOCK + (threadIdx.x >> 6);
+  const int nwaves = gridDim.x * WAVES_PER_BLOCK;
+  const int row16 = D / 8;
+  const float fD = (float)D;
+  for (int t = wave; t < T; t += nwaves) {
+    const uint4* xr = x + (size_t)t * row16;
+    const size_t brow = (size_t)(t / tokens_per_batch) * row16;
+    if constexpr (NCHUNK > 0) {
+      uint4 v[NCHUNK];
+#pragma unroll
+      for (int c = 0; c < NCHUNK; ++c) v[c] = xr[c * 64 + lane];
+      float s = 0.0f;
+#pragma unroll
+      for (int c = 0; c < NCHUNK; ++c) {
+        float f[8];
+        unpack8(v[c], f);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) s = s + f[j];
+      }
+      const float mean = __fdiv_rn(wave_sum(s), fD);
+      float s2 = 0.0f;
+#pragma unroll
+      for (int c = 0; c < NCHUNK; ++c) {
+        float f[8];
+        unpack8(v[c], f);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) { const float d = f[j] - mean; s2 = __builtin_fmaf(d, d, s2); }
+      }
+      const float rstd = __fdiv_rn(1.0f, __builtin_sqrtf(__fdiv_rn(wave_sum(s2), fD) + eps));
+#pragma unroll
+      for (int c = 0; c < NCHUNK; ++c)
+        out[(size_t)t * row16 + c * 64 + lane] =
+            modulate8(v[c], scale[brow + c * 64 + lane], shift[brow + c * 64 + lane], mean, rstd);
+    } else {
+      float s = 0.0f;
+      for (int u = lane; u < row16; u += 64) {
+        float f[8];
+        unpack8(xr[u], f);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) s = s + f[j];
+      }
+      const float mean = __fdiv_rn(wave_sum(s), fD);
+      float s2 = 0.0f;
+      for (int u = lane; u < row16; u += 64) {
+        float f[8];
+        unpack8(xr[u], f);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) { const float d = f[j] - mean; s2 = __builtin_fmaf(d, d, s2); }
+      }
+      const float rstd = __fdiv_rn(1.0f, __builtin_sqrtf(__fdiv_rn(wave_sum(s2), fD) + eps));
+      for (int u = lane; u < row16; u += 64)
+        out[(size_t)t * row16 + u] = modulate8(xr[u], scale[brow + u], shift[brow + u], mean, rstd);
+    }
+  }
+}
+
 }  // namespace
 
 extern "C" int hdmoe_gate_top2(const void* x_bf16, const void* gate_w_bf16, int T, int D, int E,
@@ -204,4 +303,27 @@ extern "C" int hdmoe_gate_top2(const void* x_bf16, const void* gate_w_bf16, int 
     case 16: return launch_gate<16>(x_bf16, gate_w_bf16, T, D, topk_idx, topk_weight_bf16, s);
     default: return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_gate_top2: E=%d not in {2,4,8,16}", E);
   }
+}
+
+extern "C" int hdmoe_ln_modulate_bf16(const void* x_bf16, const void* scale_bf16, const void* shift_bf16, int T, int D,
+                                      int tokens_per_batch, float eps, void* out_bf16, hdmoe_stream_t stream) {
+  HDMOE_REQUIRE_PTR(x_bf16);
+  HDMOE_REQUIRE_PTR(scale_bf16);
+  HDMOE_REQUIRE_PTR(shift_bf16);
+  HDMOE_REQUIRE_PTR(out_bf16);
+  if (T < 0 || D <= 0 || D % 8 != 0 || tokens_per_batch <= 0 || !(eps >= 0.0f))
+    return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_ln_modulate_bf16: T=%d D=%d tokens_per_batch=%d eps=%g", T, D,
+                      tokens_per_batch, (double)eps);
+  if (T == 0) return HDMOE_OK;
+  int blocks = (T + WAVES_PER_BLOCK - 1) / WAVES_PER_BLOCK;
+  if (blocks > HDMOE_NUM_CU * 16) blocks = HDMOE_NUM_CU * 16;
+  const dim3 grid(blocks), block(WAVES_PER_BLOCK * 64);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const uint4* xp = static_cast<const uint4*>(x_bf16);
+  const uint4* sc = static_cast<const uint4*>(scale_bf16);
+  const uint4* sh = static_cast<const uint4*>(shift_bf16);
+  uint4* op = static_cast<uint4*>(out_bf16);
+  if (D == 2560) hipLaunchKernelGGL(ln_modulate_kernel<5>, grid, block, 0, s, xp, sc, sh, T, D, tokens_per_batch, eps, op);
+  else hipLaunchKernelGGL(ln_modulate_kernel<0>, grid, block, 0, s, xp, sc, sh, T, D, tokens_per_batch, eps, op);
+  return hdmoe_check_launch("hdmoe_ln_modulate_bf16");
 }

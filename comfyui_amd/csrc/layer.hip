@@ -12,6 +12,9 @@ int hdmoe_check_gemm_shape(const char* what, int weight_dtype, long rows, int K,
 int hdmoe_launch_quant_dispatch(const void* x_bf16, const int32_t* perm, const int32_t* offsets, int T, int D, int E,
                                 const float* const* scale_input, const float* shared_scale, bool with_shared,
                                 void* a_fp8, hipStream_t s, const char* what);
+int hdmoe_launch_combine(const void* y_sorted_bf16, const int32_t* inv_perm, const void* topk_weight_bf16,
+                         const void* shared_bf16, const void* gate_bf16, const void* residual_bf16, int tokens_per_batch,
+                         int T, int D, void* out_bf16, hipStream_t s, const char* what);
 
 char* hdmoe_error_buffer() {
   static thread_local char buf[HDMOE_ERRBUF] = {0};
@@ -46,6 +49,8 @@ extern "C" int hdmoe_layer_layout_get(int T, int D, int H, int Hs, int E, int we
   out->h = take((n * H + (size_t)T * Hs) * eb);
   // y: routed [2T,D] then shared [T,D], bf16
   out->y = take((n + (Hs > 0 ? (size_t)T : 0)) * D * 2);
+  // normalised + modulated tokens of the optional block fusion, [T,D] bf16
+  out->normed = take((size_t)T * D * 2);
   out->total = off;
   return HDMOE_OK;
 }
@@ -77,6 +82,14 @@ extern "C" int hdmoe_moe_ffn(const hdmoe_layer_args* p, hdmoe_stream_t stream) {
     if (int rc = hdmoe_check_gemm_shape("hdmoe_moe_ffn (shared gate/up)", wd, T, D, Hs, 128)) return rc;
     if (int rc = hdmoe_check_gemm_shape("hdmoe_moe_ffn (shared down)", wd, T, Hs, D, 256)) return rc;
   }
+  const bool fused_block = p->mod_scale != nullptr || p->mod_shift != nullptr || p->mod_gate != nullptr;
+  if (fused_block) {
+    HDMOE_REQUIRE_PTR(p->mod_scale);
+    HDMOE_REQUIRE_PTR(p->mod_shift);
+    HDMOE_REQUIRE_PTR(p->mod_gate);
+    if (p->tokens_per_batch <= 0 || T % p->tokens_per_batch != 0)
+      return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_moe_ffn: tokens_per_batch=%d does not divide T=%d", p->tokens_per_batch, T);
+  }
   if (T == 0) return HDMOE_OK;
 
   const bool fp8 = wd == HDMOE_W_E4M3FN;
@@ -107,8 +120,17 @@ extern "C" int hdmoe_moe_ffn(const hdmoe_layer_args* p, hdmoe_stream_t stream) {
     if (p->stage_events) (void)hipEventRecord(static_cast<hipEvent_t>(p->stage_events[ev]), s);
     ++ev;
   };
+  // the tokens the feed-forward sees: x itself, or LayerNorm(x) * (1 + scale) + shift (timed with the gate stage)
+  const void* xin = p->x;
   mark();
-  if (int rc = hdmoe_gate_top2(p->x, p->gate_w, T, D, E, idx, tw, stream)) return rc;
+  if (fused_block) {
+    void* normed = ws + l.normed;
+    if (int rc = hdmoe_ln_modulate_bf16(p->x, p->mod_scale, p->mod_shift, T, D, p->tokens_per_batch, p->ln_eps, normed,
+                                        stream))
+      return rc;
+    xin = normed;
+  }
+  if (int rc = hdmoe_gate_top2(xin, p->gate_w, T, D, E, idx, tw, stream)) return rc;
   mark();
   if (int rc = hdmoe_dispatch(idx, T, E, counts, offsets, perm, inv_perm, ws + l.dispatch_ws,
                               hdmoe_dispatch_workspace_bytes(T, E), stream))
@@ -120,13 +142,13 @@ extern "C" int hdmoe_moe_ffn(const hdmoe_layer_args* p, hdmoe_stream_t stream) {
     const float* sin[HDMOE_MAX_EXPERTS];
     for (int e = 0; e < E; ++e) sin[e] = p->experts[e].scale_in1;
     // routed rows and the shared expert's token-order copy in one launch ([2T,D] then [T,D] of the same buffer)
-    if (int rc = hdmoe_launch_quant_dispatch(p->x, perm, offsets, T, D, E, sin, Hs > 0 ? p->shared->scale_in1 : nullptr,
+    if (int rc = hdmoe_launch_quant_dispatch(xin, perm, offsets, T, D, E, sin, Hs > 0 ? p->shared->scale_in1 : nullptr,
                                              Hs > 0, a_routed, s, "hdmoe_moe_ffn (quantise)"))
       return rc;
     if (Hs > 0) a_static = a_shared;
   } else {
-    if (int rc = hdmoe_permute_bf16(p->x, perm, T, D, a_routed, stream)) return rc;
-    a_static = static_cast<const uint8_t*>(p->x);
+    if (int rc = hdmoe_permute_bf16(xin, perm, T, D, a_routed, stream)) return rc;
+    a_static = static_cast<const uint8_t*>(xin);
   }
 
   mark();
@@ -140,7 +162,9 @@ extern "C" int hdmoe_moe_ffn(const hdmoe_layer_args* p, hdmoe_stream_t stream) {
                                      Hs > 0 ? T : 0, p->shared, y_shared, H, D, Hs, D, s, "hdmoe_moe_ffn (down)"))
     return rc;
   mark();
-  const int rc = hdmoe_combine(y_routed, inv_perm, tw, Hs > 0 ? y_shared : nullptr, T, D, p->out, stream);
+  const int rc = hdmoe_launch_combine(y_routed, inv_perm, tw, Hs > 0 ? y_shared : nullptr,
+                                      fused_block ? p->mod_gate : nullptr, fused_block ? p->x : nullptr,
+                                      fused_block ? p->tokens_per_batch : 1, T, D, p->out, s, "hdmoe_moe_ffn (combine)");
   mark();
   return rc;
 }

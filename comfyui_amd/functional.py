@@ -151,6 +151,47 @@ def combine(y_sorted, inv_perm, topk_weight, shared):
     return out
 
 
+def _per_batch(t, what, D, device):
+    """[B, D] (or [B, 1, D]) bf16 modulation rows -> contiguous [B, D]."""
+    _need_hip(t, what, BF16)
+    if t.dim() == 3 and t.shape[1] == 1:
+        t = t[:, 0]
+    if t.dim() != 2 or t.shape[1] != D or not t.is_contiguous():
+        raise ValueError(f"{what}: expected a contiguous [batch, {D}] tensor, got {tuple(t.shape)}")
+    return t
+
+
+def ln_modulate(x2d, scale, shift, tokens_per_batch, eps=1e-6):
+    """bf16 LayerNorm(x) * (1 + scale) + shift with scale/shift one row per batch item
+    (comfy/ldm/hidream/model.py:430-431, 516-517)."""
+    _need_hip(x2d, "ln_modulate x", BF16)
+    T, D = x2d.shape
+    scale = _per_batch(scale, "ln_modulate scale", D, x2d.device)
+    shift = _per_batch(shift, "ln_modulate shift", D, x2d.device)
+    if tokens_per_batch <= 0 or T != scale.shape[0] * tokens_per_batch or shift.shape != scale.shape:
+        raise ValueError(f"ln_modulate: T={T} is not batch={scale.shape[0]} x tokens_per_batch={tokens_per_batch}")
+    out = torch.empty_like(x2d)
+    check(lib.hdmoe_ln_modulate_bf16(ptr(x2d), ptr(scale), ptr(shift), T, D, tokens_per_batch, eps, ptr(out),
+                                     _stream(x2d)))
+    return out
+
+
+def combine_gated_residual(y_sorted, inv_perm, topk_weight, shared, gate, residual, tokens_per_batch):
+    """combine(), then gate * y + residual (comfy/ldm/hidream/model.py:432-433, 518-523)."""
+    _need_hip(y_sorted, "combine y", BF16)
+    _need_hip(topk_weight, "combine topk_weight", BF16)
+    _need_hip(residual, "combine residual", BF16)
+    T = topk_weight.shape[0]
+    D = y_sorted.shape[1]
+    gate = _per_batch(gate, "combine gate", D, y_sorted.device)
+    if tokens_per_batch <= 0 or T != gate.shape[0] * tokens_per_batch or tuple(residual.shape) != (T, D):
+        raise ValueError(f"combine_gated_residual: T={T}, batch={gate.shape[0]}, tokens_per_batch={tokens_per_batch}")
+    out = torch.empty((T, D), dtype=BF16, device=y_sorted.device)
+    check(lib.hdmoe_combine_gated_residual(ptr(y_sorted), ptr(inv_perm), ptr(topk_weight), ptr(shared), ptr(gate),
+                                           ptr(residual), tokens_per_batch, T, D, ptr(out), _stream(y_sorted)))
+    return out
+
+
 def make_ffn_weights(w1, w2, w3, scales=None):
     """Fill an hdmoe_ffn_weights. scales: dict with optional fp32 scalar tensors
     scale_w1/2/3 and scale_in1/2/3 (fp8 only)."""
@@ -206,8 +247,10 @@ def layer_layout(T, D, H, Hs, E, code):
 
 
 def moe_ffn(x2d, gate_w, experts, shared, H, Hs, weight_dtype, out=None, workspace=None, want_routing=False,
-            stage_events=None):
+            stage_events=None, modulation=None, tokens_per_batch=None, ln_eps=1e-6):
     """The whole layer as one enqueue. experts: list of FfnWeights, shared: FfnWeights or None.
+    modulation=(shift, scale, gate), each [B, D] bf16, turns the call into the block's feed-forward branch:
+    out = x + gate * layer(LayerNorm(x) * (1 + scale) + shift), with T == B * tokens_per_batch.
     Returns out [T,D] bf16 (and topk_idx int32, topk_weight bf16 when want_routing)."""
     _need_hip(x2d, "moe_ffn x", BF16)
     _need_hip(gate_w, "moe_ffn gate weight", BF16)
@@ -232,6 +275,12 @@ def moe_ffn(x2d, gate_w, experts, shared, H, Hs, weight_dtype, out=None, workspa
         sh = FfnWeights.from_buffer_copy(shared)
         args.shared = ctypes.pointer(sh)
     args.out, args.workspace, args.workspace_bytes = ptr(out), ptr(workspace), workspace.numel()
+    if modulation is not None:
+        shift, scale, gate = (_per_batch(m, "moe_ffn modulation", D, x2d.device) for m in modulation)
+        if not tokens_per_batch or T != shift.shape[0] * tokens_per_batch or not (shift.shape == scale.shape == gate.shape):
+            raise ValueError(f"moe_ffn: T={T} is not batch={shift.shape[0]} x tokens_per_batch={tokens_per_batch}")
+        args.mod_shift, args.mod_scale, args.mod_gate = ptr(shift), ptr(scale), ptr(gate)
+        args.tokens_per_batch, args.ln_eps = tokens_per_batch, ln_eps
     idx = tw = None
     if want_routing:
         idx = torch.empty((T, 2), dtype=torch.int32, device=x2d.device)

@@ -213,9 +213,34 @@ class MOEFeedForwardSwiGLU(nn.Module):
             return y.view(*orig_shape)
         return self._forward_composed(x2, gate_w).view(*orig_shape)
 
+    def forward_branch(self, x, shift, scale, gate, eps=1e-6, stage_events=None):
+        """The whole feed-forward branch of a block in one enqueue (not a method of the reference class; it is
+        the lines around its call, comfy/ldm/hidream/model.py:429-433 and 515-523):
+            x + gate * self(LayerNorm(x, eps, no affine) * (1 + scale) + shift)
+        x [B,S,dim]; shift, scale, gate [B,1,dim] (the chunks of adaLN_modulation) in bf16."""
+        if x.dtype != BF16 or not x.is_cuda or x.dim() != 3:
+            raise RuntimeError(f"MOEFeedForwardSwiGLU.forward_branch: expected a [B,S,dim] bfloat16 HIP tensor, got "
+                               f"{tuple(x.shape)} {x.dtype} on {x.device}; comfyui_amd has no CPU path")
+        self.gate._check()
+        B, S, D = x.shape
+        x2 = x.reshape(-1, D).contiguous()
+        mods = tuple(m.reshape(B, D).contiguous() for m in (shift, scale, gate))
+        gate_w = self.gate.device_weight(x2)
+        got = self._collect(x2)
+        if got is not None:
+            wdt, experts, shared, keep = got
+            H = self.experts[0].w1.weight.shape[0]
+            Hs = self.shared_experts.w1.weight.shape[0]
+            y = HF.moe_ffn(x2, gate_w, experts, shared, H, Hs, wdt, stage_events=stage_events, modulation=mods,
+                           tokens_per_batch=S, ln_eps=eps)
+            del keep
+            return y.view(B, S, D)
+        n = HF.ln_modulate(x2, mods[1], mods[0], S, eps)
+        return self._forward_composed(n, gate_w, gated_residual=(mods[2], x2, S)).view(B, S, D)
+
     # ---- composed path -----------------------------------------------------------------
 
-    def _forward_composed(self, x2, gate_w):
+    def _forward_composed(self, x2, gate_w, gated_residual=None):
         """Same stages, one expert at a time through the Linear modules (weight functions,
         offloaded or mixed-dtype weights, dequantising scaled-fp8 Linears)."""
         E = len(self.experts)
@@ -229,4 +254,7 @@ class MOEFeedForwardSwiGLU(nn.Module):
             if hi > lo:
                 y[lo:hi] = expert(xs[lo:hi])
         shared = self.shared_experts(x2)
+        if gated_residual is not None:
+            g, res, per_batch = gated_residual
+            return HF.combine_gated_residual(y, inv_perm, w, shared, g, res, per_batch)
         return HF.combine(y, inv_perm, w, shared)

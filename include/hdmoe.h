@@ -33,7 +33,7 @@
 extern "C" {
 #endif
 
-#define HDMOE_VERSION 100
+#define HDMOE_VERSION 101
 
 #define HDMOE_OK 0
 #define HDMOE_E_NULL (-1)      /* required pointer is NULL */
@@ -152,6 +152,18 @@ int hdmoe_scale_to_bf16(int src_dtype, const void* src, int64_t n, const float* 
 int hdmoe_combine(const void* y_sorted_bf16, const int32_t* inv_perm, const void* topk_weight_bf16,
                   const void* shared_bf16, int T, int D, void* out_bf16, hdmoe_stream_t stream);
 
+/* Feed-forward branch of a HiDream block around the layer (comfy/ldm/hidream/model.py:429-433, 515-523):
+ *   n   = LayerNorm(x, eps, no affine) * (1 + scale_mlp) + shift_mlp      -> hdmoe_ln_modulate_bf16
+ *   out = gate_mlp * FFN(n) + x                                          -> hdmoe_combine_gated_residual
+ * scale/shift/gate are [B, D] bf16 (one row per batch item; token t uses row t / tokens_per_batch); every
+ * elementwise op rounds to bf16 as the reference's torch ops do. */
+int hdmoe_ln_modulate_bf16(const void* x_bf16, const void* scale_bf16, const void* shift_bf16, int T, int D,
+                           int tokens_per_batch, float eps, void* out_bf16, hdmoe_stream_t stream);
+int hdmoe_combine_gated_residual(const void* y_sorted_bf16, const int32_t* inv_perm,
+                                 const void* topk_weight_bf16, const void* shared_bf16,
+                                 const void* gate_bf16, const void* residual_bf16, int tokens_per_batch,
+                                 int T, int D, void* out_bf16, hdmoe_stream_t stream);
+
 /* ---- whole layer -------------------------------------------------------------- */
 
 /* MOEFeedForwardSwiGLU.forward, model.py:307-325, as one call that enqueues
@@ -178,11 +190,20 @@ typedef struct hdmoe_layer_args {
    * Event i is recorded on `stream` before stage i and event i+1 after it; stages in order:
    * gate, dispatch, quantise/permute, gate-up GEMM, down GEMM, combine. */
   void** stage_events;
+  /* optional block fusion (all three NULL = the plain layer). When set, x is the un-normalised token stream and
+   * out = x + mod_gate * FFN( LayerNorm(x, ln_eps) * (1 + mod_scale) + mod_shift ); the normalised tokens live in
+   * the workspace. [B, D] bf16 each, B = T / tokens_per_batch. */
+  const void* mod_scale;
+  const void* mod_shift;
+  const void* mod_gate;
+  int tokens_per_batch;
+  float ln_eps;
 } hdmoe_layer_args;
 
 #define HDMOE_NUM_STAGES 6
 #define HDMOE_NUM_STAGE_EVENTS (HDMOE_NUM_STAGES + 1)
 
+/* The workspace size already includes room for the normalised tokens of the block fusion. */
 size_t hdmoe_layer_workspace_bytes(int T, int D, int H, int Hs, int E, int weight_dtype);
 int hdmoe_moe_ffn(const hdmoe_layer_args* args, hdmoe_stream_t stream);
 
@@ -199,7 +220,7 @@ int hdmoe_ffn_swiglu(int weight_dtype, const void* x_bf16, int rows, int D, int 
 /* Where the pieces of the workspace live, for tests that inspect intermediates. */
 typedef struct hdmoe_layer_layout {
   size_t topk_idx, topk_weight, counts, offsets, perm, inv_perm, dispatch_ws;
-  size_t a, h, y, total;
+  size_t a, h, y, normed, total;
 } hdmoe_layer_layout;
 int hdmoe_layer_layout_get(int T, int D, int H, int Hs, int E, int weight_dtype,
                            hdmoe_layer_layout* out);

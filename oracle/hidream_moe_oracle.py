@@ -45,6 +45,9 @@ def _lib():
         lib.ref_gate_top2.restype = ctypes.c_int
         lib.ref_dispatch.restype = ctypes.c_int
         lib.ref_combine.restype = None
+        lib.ref_ln_modulate.restype = ctypes.c_int
+        lib.ref_ln_modulate.argtypes = [ctypes.c_void_p] * 3 + [ctypes.c_int] * 3 + [ctypes.c_float, ctypes.c_void_p]
+        lib.ref_gated_residual.restype = None
         lib.ref_e4m3fn_encode.restype = None
         lib.ref_e4m3fn_decode_table.restype = None
         _LIB = lib
@@ -234,6 +237,51 @@ def moe_forward(x, params, mode, gate_result=None):
     y = (y.view(*topk_weight.shape, -1) * topk_weight.unsqueeze(-1)).sum(dim=1)
     y = y.view(*orig_shape).to(wtype)
     return y + ffn_swiglu(x, params["shared"], mode)
+
+
+# ------------------------------------------------------- feed-forward branch of a block
+
+def ln_modulate_torch(x3, shift, scale, eps=1e-6):
+    """model.py:430-431 / 516-517 with torch's own ops: x3 [B,S,D]; shift, scale [B,1,D], all one dtype."""
+    n = F.layer_norm(x3, (x3.shape[-1],), None, None, eps).to(x3.dtype)
+    return n * (1 + scale) + shift
+
+
+def ln_modulate_c(x2d_bf16, shift_bf16, scale_bf16, tokens_per_batch, eps=1e-6):
+    """The same in the fixed summation order of moe_ref.c ref_ln_modulate; x2d [T,D], shift/scale [B,D] bf16."""
+    T, D = x2d_bf16.shape
+    out = torch.empty((T, D), dtype=torch.bfloat16)
+    rc = _lib().ref_ln_modulate(_p(x2d_bf16.contiguous()), _p(scale_bf16.contiguous()), _p(shift_bf16.contiguous()),
+                                T, D, tokens_per_batch, eps, _p(out))
+    if rc != 0:
+        raise ValueError("ref_ln_modulate: bad shape")
+    return out
+
+
+def gated_residual_torch(y3, gate, residual3):
+    """model.py:432-433 / 518-523: gate [B,1,D] * y [B,S,D] + residual."""
+    return gate * y3 + residual3
+
+
+def gated_residual_c(y2d_bf16, gate_bf16, residual2d_bf16, tokens_per_batch):
+    T, D = y2d_bf16.shape
+    out = torch.empty((T, D), dtype=torch.bfloat16)
+    _lib().ref_gated_residual(_p(y2d_bf16.contiguous()), _p(gate_bf16.contiguous()), _p(residual2d_bf16.contiguous()),
+                              ctypes.c_int(T), ctypes.c_int(D), ctypes.c_int(tokens_per_batch), _p(out))
+    return out
+
+
+def ff_branch(x3, shift, scale, gate, params, mode, gate_result=None, fixed_order_norm=False):
+    """model.py:429-433: x + gate * ff(LayerNorm(x) * (1 + scale) + shift) for x3 [B,S,D], shift/scale/gate
+    [B,1,D]. fixed_order_norm takes the LayerNorm statistics in ref_ln_modulate's order (what the HIP kernel
+    does) instead of torch's. Returns (out, normed tokens)."""
+    B, S, D = x3.shape
+    if fixed_order_norm:
+        n = ln_modulate_c(x3.reshape(-1, D), shift.reshape(B, D), scale.reshape(B, D), S).view(B, S, D)
+    else:
+        n = ln_modulate_torch(x3, shift, scale)
+    y = moe_forward(n, params, mode, gate_result=gate_result)
+    return gated_residual_torch(y, gate, x3), n
 
 
 def moe_forward_dense(x, params, mode, topk_idx, topk_weight):

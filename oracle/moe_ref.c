@@ -170,6 +170,66 @@ int ref_dispatch(const int32_t* flat, int64_t n, int E, int32_t* counts, int32_t
 
 /* ---- combine ---------------------------------------------------------------- */
 
+/* adaLN prologue of the feed-forward branch (model.py:430-431, 516-517):
+ *   n = bf16(LayerNorm(x[t], eps))   (no affine, biased variance, fp32 statistics)
+ *   out[t] = bf16( bf16(n * bf16(1 + scale[b])) + shift[b] ),  b = t / tokens_per_batch.
+ * Mean and variance are two passes in ONE fixed fp32 order (the HIP kernel's: 64 partial sums over
+ * 8-element groups strided by 512 elements, then the pairwise tree), so the kernel compares bit for
+ * bit; agreement with torch's own layer_norm is checked in the tests to one bf16 step. */
+static float tree64(float* lane) {
+  for (int off = 32; off >= 1; off >>= 1)
+    for (int l = 0; l < off; ++l) lane[l] = lane[l] + lane[l + off];
+  return lane[0];
+}
+
+int ref_ln_modulate(const uint16_t* x, const uint16_t* scale, const uint16_t* shift, int T, int D,
+                    int tokens_per_batch, float eps, uint16_t* out) {
+  if (D % 8 != 0 || D <= 0 || T < 0 || tokens_per_batch <= 0) return -1;
+  for (int t = 0; t < T; ++t) {
+    const uint16_t* xr = x + (size_t)t * D;
+    const uint16_t* sc = scale + (size_t)(t / tokens_per_batch) * D;
+    const uint16_t* sh = shift + (size_t)(t / tokens_per_batch) * D;
+    float lane[64];
+    for (int l = 0; l < 64; ++l) {
+      float acc = 0.0f;
+      for (int base = l * 8; base < D; base += 512)
+        for (int j = 0; j < 8; ++j) acc = acc + bf16_to_f32(xr[base + j]);
+      lane[l] = acc;
+    }
+    const float mean = tree64(lane) / (float)D;
+    for (int l = 0; l < 64; ++l) {
+      float acc = 0.0f;
+      for (int base = l * 8; base < D; base += 512)
+        for (int j = 0; j < 8; ++j) {
+          const float d = bf16_to_f32(xr[base + j]) - mean;
+          acc = fmaf(d, d, acc);
+        }
+      lane[l] = acc;
+    }
+    const float rstd = 1.0f / sqrtf(tree64(lane) / (float)D + eps);
+    for (int d = 0; d < D; ++d) {
+      const float n = bf16_to_f32(f32_to_bf16((bf16_to_f32(xr[d]) - mean) * rstd));
+      const float m = bf16_to_f32(f32_to_bf16(1.0f + bf16_to_f32(sc[d])));
+      const float p = bf16_to_f32(f32_to_bf16(n * m));
+      out[(size_t)t * D + d] = f32_to_bf16(p + bf16_to_f32(sh[d]));
+    }
+  }
+  return 0;
+}
+
+/* Gated residual epilogue (model.py:432-433, 518-523): out = bf16( bf16(gate[b] * y[t]) + residual[t] ). */
+void ref_gated_residual(const uint16_t* y, const uint16_t* gate, const uint16_t* residual, int T, int D,
+                        int tokens_per_batch, uint16_t* out) {
+  for (int t = 0; t < T; ++t) {
+    const uint16_t* g = gate + (size_t)(t / tokens_per_batch) * D;
+    for (int d = 0; d < D; ++d) {
+      const size_t i = (size_t)t * D + d;
+      const float p = bf16_to_f32(f32_to_bf16(bf16_to_f32(g[d]) * bf16_to_f32(y[i])));
+      out[i] = f32_to_bf16(p + bf16_to_f32(residual[i]));
+    }
+  }
+}
+
 /* y_sorted [2T,D] bf16 (row r = expert output of flat slot perm[r]); w [T,2] bf16;
  * shared [T,D] bf16 or NULL. out[t] = bf16( bf16( f32(bf16(y0*w0)) + f32(bf16(y1*w1)) ) + shared[t] )
  * which is how a bf16 `(y*w).sum(1)` then `+ shared` rounds (model.py:319,324). */

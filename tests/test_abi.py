@@ -25,7 +25,8 @@ def test_every_declared_symbol_is_exported_and_bound():
         assert hasattr(_lib.lib, n), n
         assert n in _lib.SIGNATURES, f"{n} has no ctypes signature"
     assert sorted(_lib.SIGNATURES) == names
-    assert _lib.lib.hdmoe_version() == 100
+    version = int(re.search(r"#define\s+HDMOE_VERSION\s+(\d+)", open(HEADER).read()).group(1))
+    assert _lib.lib.hdmoe_version() == version >= 101
 
 
 def test_header_constants_match_binding():
@@ -38,7 +39,30 @@ def test_header_constants_match_binding():
     assert (int(consts["HDMOE_E_NULL"]), int(consts["HDMOE_E_SHAPE"]), int(consts["HDMOE_E_WORKSPACE"]),
             int(consts["HDMOE_E_LAUNCH"])) == (_lib.E_NULL, _lib.E_SHAPE, _lib.E_WORKSPACE, _lib.E_LAUNCH)
     assert ctypes.sizeof(_lib.FfnWeights) == 9 * 8
-    assert ctypes.sizeof(_lib.LayerLayout) == 11 * 8
+    assert ctypes.sizeof(_lib.LayerLayout) == 12 * 8
+
+
+def test_struct_layouts_match_what_a_c_compiler_sees(tmp_path):
+    """sizeof/offsetof of every struct of the header as gcc lays them out == the ctypes mirrors."""
+    import subprocess
+    from comfyui_amd import _lib
+    structs = {"hdmoe_ffn_weights": _lib.FfnWeights, "hdmoe_layer_args": _lib.LayerArgs,
+               "hdmoe_layer_layout": _lib.LayerLayout}
+    lines = []
+    for cname, cls in structs.items():
+        lines.append(f'printf("{cname} %zu\\n", sizeof({cname}));')
+        for fname, _ in cls._fields_:
+            lines.append(f'printf("{cname}.{fname} %zu\\n", offsetof({cname}, {fname}));')
+    src = tmp_path / "layout.c"
+    src.write_text('#include <stdio.h>\n#include <stddef.h>\n#include "hdmoe.h"\nint main(void) {\n'
+                   + "\n".join(lines) + "\nreturn 0; }\n")
+    exe = tmp_path / "layout"
+    subprocess.check_call(["gcc", "-std=c11", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)])
+    got = dict(l.split() for l in subprocess.check_output([str(exe)], text=True).splitlines())
+    for cname, cls in structs.items():
+        assert int(got[cname]) == ctypes.sizeof(cls), cname
+        for fname, _ in cls._fields_:
+            assert int(got[f"{cname}.{fname}"]) == getattr(cls, fname).offset, f"{cname}.{fname}"
 
 
 def test_argument_errors_are_reported_without_a_device():
