@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the HiDream MoE SwiGLU feed-forward layer on one MI355X.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg3|cfg2|cfg1] [--no-cpu-baseline]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg3|cfg2|cfg1|cfg5-256|cfg5-4096] [--no-cpu-baseline]
 
 A step is one forward of comfyui_amd.hidream.MOEFeedForwardSwiGLU (gate, dispatch, quantise,
 grouped fp8 GEMMs, combine, shared expert) over one synthetic batch that is already resident in
@@ -109,7 +109,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="cfg3", choices=["cfg1", "cfg2", "cfg3"])
+    ap.add_argument("--workload", default="cfg3", choices=["cfg1", "cfg2", "cfg3", "cfg5-256", "cfg5-4096"])
     ap.add_argument("--cpu-sample-tokens", type=int, default=8192)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--pmc-calibration", action="store_true",
@@ -203,6 +203,10 @@ def main():
         "config": {
             "workload": {"cfg1": "cfg1: 1x1024 tokens, bf16 weights",
                          "cfg2": "cfg2: 1x4096 tokens, scaled fp8 e4m3fn weights, scale_input 1.0",
+                         "cfg5-256": "cfg5: 256 tokens, fp8 weights, skewed routing (about 70% of tokens pick expert 0) "
+                                     "with exact logit ties on every 64th token",
+                         "cfg5-4096": "cfg5: 4096 tokens, fp8 weights, skewed routing (about 70% of tokens pick expert "
+                                      "0) with exact logit ties on every 64th token",
                          "cfg3": "cfg3 (headline): 2x4096 = 8192 tokens x 2560, scaled fp8 e4m3fn weights "
                                  "(scale_weight = amax/448, scale_input = 1.0), bf16 gate, x ~ N(0,1) with 1% "
                                  "outlier channels x20, 4 routed experts (hidden 6912) top-2 + shared expert (hidden 3584)"}[args.workload],

@@ -157,17 +157,28 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
 
   // source of the tile being loaded (buffer resources are kept as plain locals: the opaque resource type
   // cannot be a struct member)
+  //
+  // Weight rows of the tile. SwiGLU: LDS half h (128 rows) holds rows n0..n0+127 of w1 (h=0) / w3 (h=1).
+  // Plain: wave column wq multiplies LDS rows wq*32..+32 of both halves, and its 64 output features should be
+  // contiguous in memory, so LDS row (h, wq, i) holds weight row n0 + wq*64 + h*32 + i.
   __amdgpu_buffer_rsrc_t src_a = make_rsrc(nullptr, 0), src_b0 = src_a, src_b1 = src_a;
   int src_voff[4] = {0, 0, 0, 0};
+  int src_voff_b[2] = {0, 0};
   auto set_src = [&](const Tile& d) {
     const GemmGroup& gg = args.g[d.g];
     src_a = make_rsrc(gg.a + (size_t)d.row0 * d.kbytes, (uint32_t)d.rows_here * (uint32_t)d.kbytes);
     const uint8_t* b_half0 = gg.b0 + (size_t)d.n0 * d.kbytes;
-    const uint8_t* b_half1 = SWIGLU ? gg.b1 + (size_t)d.n0 * d.kbytes : gg.b0 + (size_t)(d.n0 + BN / 2) * d.kbytes;
-    src_b0 = make_rsrc(b_half0, (uint32_t)(BN / 2) * (uint32_t)d.kbytes);
-    src_b1 = make_rsrc(b_half1, (uint32_t)(BN / 2) * (uint32_t)d.kbytes);
+    const uint8_t* b_half1 = SWIGLU ? gg.b1 + (size_t)d.n0 * d.kbytes : gg.b0 + (size_t)(d.n0 + 32) * d.kbytes;
+    const uint32_t b_rows = SWIGLU ? BN / 2 : BN - 32;
+    src_b0 = make_rsrc(b_half0, b_rows * (uint32_t)d.kbytes);
+    src_b1 = make_rsrc(b_half1, b_rows * (uint32_t)d.kbytes);
 #pragma unroll
     for (int j = 0; j < 4; ++j) src_voff[j] = (j * 64 + ld_row) * d.kbytes + ld_chunk * 16;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int r = j * 64 + ld_row;  // row within the 128-row LDS half
+      src_voff_b[j] = (SWIGLU ? r : (r >> 5) * 64 + (r & 31)) * d.kbytes + ld_chunk * 16;
+    }
   };
   auto issue_loads = [&](int stage, int kt) {
     uint8_t* sa = smem + stage * STAGE_BYTES;
@@ -178,10 +189,10 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
       __builtin_amdgcn_raw_ptr_buffer_load_lds(src_a, (lds_ptr_t)(sa + ld_lds + j * 64 * BK), 16, src_voff[j], k0, 0, 0);
 #pragma unroll
     for (int j = 0; j < 2; ++j)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(src_b0, (lds_ptr_t)(sb + ld_lds + j * 64 * BK), 16, src_voff[j], k0, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(src_b0, (lds_ptr_t)(sb + ld_lds + j * 64 * BK), 16, src_voff_b[j], k0, 0, 0);
 #pragma unroll
     for (int j = 0; j < 2; ++j)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(src_b1, (lds_ptr_t)(sb + ld_lds + (j + 2) * 64 * BK), 16, src_voff[j], k0, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(src_b1, (lds_ptr_t)(sb + ld_lds + (j + 2) * 64 * BK), 16, src_voff_b[j], k0, 0, 0);
   };
 
   // ---- LDS -> MFMA fragment addressing -------------------------------------------
@@ -243,26 +254,48 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
 
   // ---- epilogue ----------------------------------------------------------------------
   // acc[ft][tt][i]: feature = (i>>2)*8 + (lane>>5)*4 + (i&3) within the 32-row MFMA tile (ft = weight half),
-  // token = lane&31 within the 32-token MFMA tile. Stores go through a buffer resource covering exactly the
-  // valid rows of the tile: rows past the segment end are dropped by the range check.
-  const int tok_lane = wt * 128 + (lane & 31);
-  const int feat_lane = wq * 32 + (lane >> 5) * 4;
+  // token = lane&31 within the 32-token MFMA tile: a lane owns 4 consecutive features of one token, and one store
+  // instruction issued from that layout would touch 32 different rows with 8 or 16 bytes each. The packed values
+  // therefore go through LDS (stage 1, free once the K loop is over) and leave as 16 bytes per lane, 8 lanes to
+  // a 128-byte row piece. Staging rows are 128 bytes (256 for bf16 SwiGLU) with the 16-byte chunk index XORed
+  // with (token & 7). Stores go through a buffer resource covering exactly the valid rows of the tile: rows past
+  // the segment end are dropped by the range check.
+  const int tok32 = lane & 31;
+  const int hi32 = lane >> 5;
+  uint8_t* const stg = smem + STAGE_BYTES;
+  auto wave_sync = [] {
+    // orders this wave's LDS writes before its LDS reads of other lanes' data (LDS executes a wave's requests
+    // in order; this only stops the compiler from moving them)
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  };
+  // Per-tile epilogue factors. They are loaded before the K loop: a load issued after the next tile's
+  // global->LDS requests would make the epilogue wait for those as well (one in-order counter).
+  float ep_a = 1.0f, ep_b = 1.0f, ep_next = 1.0f;
+  auto load_scales = [&](const Tile& d) {
+    if constexpr (FP8) {
+      const GemmGroup& gg = args.g[d.g];
+      const float s_in = gg.s_in ? *gg.s_in : 1.0f;
+      ep_a = s_in * *gg.sb0;
+      if constexpr (SWIGLU) {
+        ep_b = s_in * *gg.sb1;
+        ep_next = gg.s_next ? hdmoe_dev_round_bf16(__fdiv_rn(1.0f, *gg.s_next)) : -1.0f;
+      }
+    }
+  };
   auto epilogue = [&](const Tile& d) {
     const GemmGroup& gg = args.g[d.g];
-    float s_in = 1.0f;
-    if constexpr (FP8) s_in = gg.s_in ? *gg.s_in : 1.0f;
     if constexpr (SWIGLU) {
-      float sg = 1.0f, su = 1.0f, inv_next = 1.0f;
-      if constexpr (FP8) {
-        sg = s_in * *gg.sb0;
-        su = s_in * *gg.sb1;
-        inv_next = gg.s_next ? hdmoe_dev_round_bf16(__fdiv_rn(1.0f, *gg.s_next)) : -1.0f;
-      }
-      const int ldo = gg.n_out * (FP8 ? 1 : 2);
+      const float sg = ep_a, su = ep_b, inv_next = ep_next;
+      constexpr int EB = FP8 ? 1 : 2;
+      constexpr int ROWB = (BN / 2) * EB;  // bytes of one staged token row: the tile's 128 features
+      const int ldo = gg.n_out * EB;
       const __amdgpu_buffer_rsrc_t ro = make_rsrc(gg.out + (size_t)d.row0 * ldo, (uint32_t)d.rows_here * (uint32_t)ldo);
 #pragma unroll
       for (int tt = 0; tt < 4; ++tt) {
-        const int rowoff = (tok_lane + tt * 32) * ldo;
+        const int tok = wt * 128 + tt * 32 + tok32;
+        uint8_t* const row = stg + tok * ROWB;
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           float m[4];
@@ -273,7 +306,8 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
             const float sl = hdmoe_dev_round_bf16(h1 * __builtin_amdgcn_rcpf(1.0f + __expf(-h1)));  // silu(.)
             m[i] = hdmoe_dev_round_bf16(sl * h3);                               // silu(.) * w3(x)
           }
-          const int feat = d.n0 + feat_lane + q * 8;
+          const int byte = (wq * 32 + q * 8 + hi32 * 4) * EB;  // position of the 4 features in the staged row
+          uint8_t* const dst = row + ((((byte >> 4) ^ (tok32 & 7)) << 4) | (byte & 15));
           if constexpr (FP8) {
             // activation cast of the w2 Linear (ops.py:337-343)
 #pragma unroll
@@ -281,34 +315,52 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
               if (inv_next < 0.0f) m[i] = m[i] < -448.0f ? -448.0f : (m[i] > 448.0f ? 448.0f : m[i]);
               else m[i] = hdmoe_dev_round_bf16(m[i] * inv_next);
             }
-            const uint32_t pk = hdmoe_dev_pack_e4m3fn(m[0], m[1]) | (hdmoe_dev_pack_e4m3fn(m[2], m[3]) << 16);
-            __builtin_amdgcn_raw_buffer_store_b32(pk, ro, rowoff + feat, 0, 0);
+            *reinterpret_cast<uint32_t*>(dst) = hdmoe_dev_pack_e4m3fn(m[0], m[1]) | (hdmoe_dev_pack_e4m3fn(m[2], m[3]) << 16);
           } else {
             u32x2 pk;
             pk.x = hdmoe_dev_pack_bf16(m[0], m[1]);
             pk.y = hdmoe_dev_pack_bf16(m[2], m[3]);
-            __builtin_amdgcn_raw_buffer_store_b64(pk, ro, rowoff + feat * 2, 0, 0);
+            *reinterpret_cast<u32x2*>(dst) = pk;
           }
         }
       }
+      __syncthreads();  // the tile's 256 x 128 outputs are staged
+      constexpr int LANES_PER_ROW = ROWB / 16;
+      constexpr int ROWS_PER_PASS = 64 / LANES_PER_ROW;
+      const int c = lane % LANES_PER_ROW;
+#pragma unroll
+      for (int p = 0; p < 32 / ROWS_PER_PASS; ++p) {
+        const int r = wave * 32 + p * ROWS_PER_PASS + lane / LANES_PER_ROW;
+        const v4i v = *reinterpret_cast<const v4i*>(stg + r * ROWB + ((c ^ (r & 7)) << 4));
+        __builtin_amdgcn_raw_buffer_store_b128(v, ro, r * ldo + d.n0 * EB + c * 16, 0, 0);
+      }
     } else {
-      float sc = 1.0f;
-      if constexpr (FP8) sc = s_in * *gg.sb0;
+      const float sc = ep_a;
       const int ldo = gg.n_out * 2;
       const __amdgpu_buffer_rsrc_t ro = make_rsrc(gg.out + (size_t)d.row0 * ldo, (uint32_t)d.rows_here * (uint32_t)ldo);
+      // each wave stages its own 32 tokens x 64 features (128 bytes per token) at a time, two buffers in turn
+      uint8_t* const mine = stg + wave * 8192;
+      const int rd_row = lane >> 3, rd_c = lane & 7;
 #pragma unroll
       for (int tt = 0; tt < 4; ++tt) {
-        const int rowoff = (tok_lane + tt * 32) * ldo;
+        uint8_t* const buf = mine + (tt & 1) * 4096;
+        wave_sync();  // the reads of two rounds ago are ahead of these writes
 #pragma unroll
         for (int ft = 0; ft < 2; ++ft) {
 #pragma unroll
           for (int q = 0; q < 4; ++q) {
-            const int feat = d.n0 + ft * 128 + feat_lane + q * 8;
             u32x2 pk;
             pk.x = hdmoe_dev_pack_bf16(acc[ft][tt][q * 4 + 0] * sc, acc[ft][tt][q * 4 + 1] * sc);
             pk.y = hdmoe_dev_pack_bf16(acc[ft][tt][q * 4 + 2] * sc, acc[ft][tt][q * 4 + 3] * sc);
-            __builtin_amdgcn_raw_buffer_store_b64(pk, ro, rowoff + feat * 2, 0, 0);
+            *reinterpret_cast<u32x2*>(buf + tok32 * 128 + (((ft * 4 + q) ^ (tok32 & 7)) << 4) + hi32 * 8) = pk;
           }
+        }
+        wave_sync();
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+          const int r = p * 8 + rd_row;
+          const v4i v = *reinterpret_cast<const v4i*>(buf + r * 128 + ((rd_c ^ rd_row) << 4));
+          __builtin_amdgcn_raw_buffer_store_b128(v, ro, (wt * 128 + tt * 32 + r) * ldo + (d.n0 + wq * 64) * 2 + rd_c * 16, 0, 0);
         }
       }
     }
@@ -324,6 +376,7 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
   issue_loads(0, 0);
   for (int i = 0; cur.g >= 0; ++i) {
     const int KT = cur.kbytes / BK;
+    load_scales(cur);
 #pragma unroll
     for (int a2 = 0; a2 < 2; ++a2)
 #pragma unroll
@@ -343,9 +396,10 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
       }
     }
     const Tile nxt = decode(i + 1);
+    // Every wave is done reading both stages: stage 0 can take the next tile's first K step, stage 1 the
+    // staged outputs of this one (it is not loaded into again before the barrier of that K step).
+    __syncthreads();
     if (nxt.g >= 0) {
-      // stage 0 was last read in the second-to-last K step when KT is even; with an odd KT it was read just now
-      if (KT & 1) __syncthreads();
       set_src(nxt);
       issue_loads(0, 0);
     }
