@@ -10,7 +10,8 @@
 // 32 (fp8) or 16 (bf16) consecutive K bytes of one row. Weights take the MFMA "A"
 // slot (rows of the 32x32 result = output features) and tokens the "B" slot (columns
 // = tokens), so a lane ends up with 4 consecutive features of one token per
-// accumulator quad and can store them as one packed word.
+// accumulator quad; the packed quads are transposed through LDS and leave as
+// 128-byte row pieces.
 //
 // Block = 512 threads = 8 waves (2 per SIMD), block tile 256 tokens x 256 weight rows,
 // K step 128 bytes, 2 LDS stages of 64 KiB filled by buffer_load ... lds (global ->
@@ -30,8 +31,6 @@
 // from its index and exits if its index is past the real tile count. Block ids are
 // remapped so that each XCD (ids congruent mod 8) walks a contiguous range of tiles,
 // 4 m-tiles deep, and its L2 sees each operand tile reused by neighbouring blocks.
-#include <type_traits>
-
 #include "common.h"
 #include "numfmt.h"
 
@@ -205,41 +204,52 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
   const int a_base = (wt * 128 + fr_row) * BK;               // token operand, + tt*32*BK
   const int b_base = TILE_BYTES + (wq * 32 + fr_row) * BK;   // weight operand, + ft*128*BK
 
-  // Fragments are software-pipelined one MFMA K slice ahead (a slice is 64 K bytes for fp8, 32 for bf16) and
-  // refilled in place: a slice first runs the four MFMAs of weight fragment 0 and re-reads it for the next
-  // slice, then the four of weight fragment 1, re-reading each token fragment right after its last use. Every
-  // LDS read so has at least three MFMAs of lead, and the matrix pipe does not wait for LDS after a barrier.
-  using frag_t = typename std::conditional<FP8, v8i, v8bf>::type;
-  constexpr int NS = FP8 ? 2 : 4;  // MFMA K slices per 128-byte K step
-  auto ld_frag = [&](const uint8_t* rowp, int ks) -> frag_t {
-    if constexpr (FP8) {
-      const int c0 = ((ks * 4 + fr_grp * 2) ^ fr_swz) * 16;
-      const v4i lo = *reinterpret_cast<const v4i*>(rowp + c0);
-      const v4i hi = *reinterpret_cast<const v4i*>(rowp + (c0 ^ 16));
-      return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-    } else {
-      return *reinterpret_cast<const v8bf*>(rowp + ((ks * 2 + fr_grp) ^ fr_swz) * 16);
-    }
-  };
-  auto mma = [](const frag_t& w, const frag_t& t, const v16f& c) -> v16f {
-    if constexpr (FP8) return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(w, t, c, 0, 0, 0, 0, 0, 0);
-    else return __builtin_amdgcn_mfma_f32_32x32x16_bf16(w, t, c, 0, 0, 0);
-  };
-
   v16f acc[2][4];
-  frag_t fa[4], fb[2];
-  // One slice: multiply with the fragments held, refilling them from slice ks_next of stage st_next.
-  auto slice = [&](const uint8_t* st_next, int ks_next) {
+  auto compute = [&](int stage) {
+    const uint8_t* st = smem + stage * STAGE_BYTES;
+    if constexpr (FP8) {
 #pragma unroll
-    for (int tt = 0; tt < 4; ++tt) acc[0][tt] = mma(fb[0], fa[tt], acc[0][tt]);
-    fb[0] = ld_frag(st_next + b_base, ks_next);
-    __builtin_amdgcn_sched_barrier(0);
+      for (int ks = 0; ks < 2; ++ks) {
+        const int c0 = ((ks * 4 + fr_grp * 2) ^ fr_swz) * 16;
+        const int c1 = c0 ^ 16;
+        v8i fa[4], fb[2];
 #pragma unroll
-    for (int tt = 0; tt < 4; ++tt) {
-      acc[1][tt] = mma(fb[1], fa[tt], acc[1][tt]);
-      fa[tt] = ld_frag(st_next + a_base + tt * 32 * BK, ks_next);
-      if (tt == 3) fb[1] = ld_frag(st_next + b_base + 128 * BK, ks_next);
-      __builtin_amdgcn_sched_barrier(0);
+        for (int tt = 0; tt < 4; ++tt) {
+          const uint8_t* p = st + a_base + tt * 32 * BK;
+          const v4i lo = *reinterpret_cast<const v4i*>(p + c0);
+          const v4i hi = *reinterpret_cast<const v4i*>(p + c1);
+          fa[tt] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        }
+#pragma unroll
+        for (int ft = 0; ft < 2; ++ft) {
+          const uint8_t* p = st + b_base + ft * 128 * BK;
+          const v4i lo = *reinterpret_cast<const v4i*>(p + c0);
+          const v4i hi = *reinterpret_cast<const v4i*>(p + c1);
+          fb[ft] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        }
+#pragma unroll
+        for (int ft = 0; ft < 2; ++ft)
+#pragma unroll
+          for (int tt = 0; tt < 4; ++tt)
+            acc[ft][tt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[ft], fa[tt], acc[ft][tt], 0, 0, 0, 0, 0, 0);
+      }
+    } else {
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) {
+        const int c0 = ((ks * 2 + fr_grp) ^ fr_swz) * 16;
+        v8bf fa[4], fb[2];
+#pragma unroll
+        for (int tt = 0; tt < 4; ++tt)
+          fa[tt] = *reinterpret_cast<const v8bf*>(st + a_base + tt * 32 * BK + c0);
+#pragma unroll
+        for (int ft = 0; ft < 2; ++ft)
+          fb[ft] = *reinterpret_cast<const v8bf*>(st + b_base + ft * 128 * BK + c0);
+#pragma unroll
+        for (int ft = 0; ft < 2; ++ft)
+#pragma unroll
+          for (int tt = 0; tt < 4; ++tt)
+            acc[ft][tt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[ft], fa[tt], acc[ft][tt], 0, 0, 0);
+      }
     }
   };
 
@@ -358,25 +368,15 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
   };
 
   // ---- persistent loop over this block's tiles ------------------------------------------------------
-  // Per tile: K steps of 128 bytes through two LDS stages. The one barrier of a K step sits in front of its
-  // last slice: by then every wave holds the step's last fragments in registers, so the stage can be refilled
-  // (K step kt+2) and the other stage, complete since the loads of step kt+1 were waited for, can be read.
-  // The barrier of a tile's last K step frees both stages: the first K step of the NEXT tile is requested
-  // there, and stage 1 stages the outputs of this one.
-  auto block_sync = [] {
-    // this wave's global->LDS loads have landed and its LDS reads have returned; then everyone's
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
-    __builtin_amdgcn_s_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-  };
+  // Per tile: K steps of 128 bytes through two LDS stages, one barrier per step (the loads of step kt+1 fly
+  // while step kt is multiplied). The first K step of the NEXT tile is requested before the epilogue of the
+  // current one, so its latency hides behind the stores.
   Tile cur = decode(0);
   if (cur.g < 0) return;
   set_src(cur);
   issue_loads(0, 0);
   for (int i = 0; cur.g >= 0; ++i) {
     const int KT = cur.kbytes / BK;
-    const Tile nxt = decode(i + 1);
     load_scales(cur);
 #pragma unroll
     for (int a2 = 0; a2 < 2; ++a2)
@@ -384,31 +384,25 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
       for (int b2 = 0; b2 < 4; ++b2)
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[a2][b2][r] = 0.0f;
-    block_sync();  // K step 0 is in stage 0; stage 1 (outputs staged by the previous tile) has been drained
-    if (KT > 1) issue_loads(1, 1);
-    fb[0] = ld_frag(smem + b_base, 0);
-    fb[1] = ld_frag(smem + b_base + 128 * BK, 0);
-#pragma unroll
-    for (int tt = 0; tt < 4; ++tt) fa[tt] = ld_frag(smem + a_base + tt * 32 * BK, 0);
-
-    auto kstep = [&](int stage, int kt) {
-      const uint8_t* st = smem + stage * STAGE_BYTES;
-      const uint8_t* sn = smem + (stage ^ 1) * STAGE_BYTES;
-#pragma unroll
-      for (int ks = 0; ks + 1 < NS; ++ks) slice(st, ks + 1);
-      block_sync();
-      if (kt + 2 < KT) {
-        issue_loads(stage, kt + 2);
-      } else if (kt + 1 == KT && nxt.g >= 0) {
-        set_src(nxt);
-        issue_loads(0, 0);
-      }
-      // after the tile's last K step this reads data nobody uses
-      slice(sn, 0);
-    };
     for (int kt = 0; kt < KT; kt += 2) {
-      kstep(0, kt);
-      if (kt + 1 < KT) kstep(1, kt + 1);
+      __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's part of the stage has landed
+      __syncthreads();                      // everyone's part has; everyone is done reading the other stage
+      if (kt + 1 < KT) issue_loads(1, kt + 1);
+      compute(0);
+      if (kt + 1 < KT) {
+        __builtin_amdgcn_s_waitcnt(0x0f70);
+        __syncthreads();
+        if (kt + 2 < KT) issue_loads(0, kt + 2);
+        compute(1);
+      }
+    }
+    const Tile nxt = decode(i + 1);
+    // Every wave is done reading both stages: stage 0 can take the next tile's first K step, stage 1 the
+    // staged outputs of this one (it is not loaded into again before the barrier of that K step).
+    __syncthreads();
+    if (nxt.g >= 0) {
+      set_src(nxt);
+      issue_loads(0, 0);
     }
     epilogue(cur);
     cur = nxt;
