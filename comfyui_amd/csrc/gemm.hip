@@ -31,6 +31,8 @@
 // from its index and exits if its index is past the real tile count. Block ids are
 // remapped so that each XCD (ids congruent mod 8) walks a contiguous range of tiles,
 // 4 m-tiles deep, and its L2 sees each operand tile reused by neighbouring blocks.
+#include <type_traits>
+
 #include "common.h"
 #include "numfmt.h"
 
@@ -285,6 +287,11 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
       }
     }
   };
+  auto round2_bf16 = [](float& a, float& b) {
+    const uint32_t p = hdmoe_dev_pack_bf16(a, b);
+    a = __uint_as_float(p << 16);
+    b = __uint_as_float(p & 0xffff0000u);
+  };
   auto epilogue = [&](const Tile& d) {
     const GemmGroup& gg = args.g[d.g];
     if constexpr (SWIGLU) {
@@ -293,37 +300,62 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
       constexpr int ROWB = (BN / 2) * EB;  // bytes of one staged token row: the tile's 128 features
       const int ldo = gg.n_out * EB;
       const __amdgpu_buffer_rsrc_t ro = make_rsrc(gg.out + (size_t)d.row0 * ldo, (uint32_t)d.rows_here * (uint32_t)ldo);
+      // The cast in front of the w2 Linear (ops.py:337-343) has three forms, fixed per tile: clamp to +-448 when
+      // that Linear has no scale_input, nothing when 1/scale_input is 1, else multiply and round. The choice is
+      // made once, outside the element loop.
+      auto swiglu_tile = [&](auto next_mode) {
+        constexpr int NEXT = decltype(next_mode)::value;  // 0 clamp, 1 unit scale, 2 general scale
 #pragma unroll
-      for (int tt = 0; tt < 4; ++tt) {
-        const int tok = wt * 128 + tt * 32 + tok32;
-        uint8_t* const row = stg + tok * ROWB;
+        for (int tt = 0; tt < 4; ++tt) {
+          const int tok = wt * 128 + tt * 32 + tok32;
+          uint8_t* const row = stg + tok * ROWB;
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          float m[4];
+          for (int q = 0; q < 4; ++q) {
+            float m[4];
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const float h1 = hdmoe_dev_round_bf16(acc[0][tt][q * 4 + i] * sg);  // w1(x) as a bf16 tensor
-            const float h3 = hdmoe_dev_round_bf16(acc[1][tt][q * 4 + i] * su);  // w3(x)
-            const float sl = hdmoe_dev_round_bf16(h1 * __builtin_amdgcn_rcpf(1.0f + __expf(-h1)));  // silu(.)
-            m[i] = hdmoe_dev_round_bf16(sl * h3);                               // silu(.) * w3(x)
-          }
-          const int byte = (wq * 32 + q * 8 + hi32 * 4) * EB;  // position of the 4 features in the staged row
-          uint8_t* const dst = row + ((((byte >> 4) ^ (tok32 & 7)) << 4) | (byte & 15));
-          if constexpr (FP8) {
-            // activation cast of the w2 Linear (ops.py:337-343)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-              if (inv_next < 0.0f) m[i] = m[i] < -448.0f ? -448.0f : (m[i] > 448.0f ? 448.0f : m[i]);
-              else m[i] = hdmoe_dev_round_bf16(m[i] * inv_next);
+            for (int i = 0; i < 4; i += 2) {
+              // two elements at a time: one packed conversion rounds both to bf16
+              float h1a = acc[0][tt][q * 4 + i] * sg, h1b = acc[0][tt][q * 4 + i + 1] * sg;   // w1(x)
+              float h3a = acc[1][tt][q * 4 + i] * su, h3b = acc[1][tt][q * 4 + i + 1] * su;   // w3(x)
+              round2_bf16(h1a, h1b);
+              round2_bf16(h3a, h3b);
+              float sa = h1a * __builtin_amdgcn_rcpf(1.0f + __expf(-h1a));                     // silu(.)
+              float sb = h1b * __builtin_amdgcn_rcpf(1.0f + __expf(-h1b));
+              round2_bf16(sa, sb);
+              float ma = sa * h3a, mb = sb * h3b;                                              // silu(.) * w3(x)
+              round2_bf16(ma, mb);
+              if constexpr (FP8 && NEXT == 2) {
+                ma *= inv_next;
+                mb *= inv_next;
+                round2_bf16(ma, mb);
+              }
+              if constexpr (FP8 && NEXT == 0) {
+                ma = ma < -448.0f ? -448.0f : (ma > 448.0f ? 448.0f : ma);
+                mb = mb < -448.0f ? -448.0f : (mb > 448.0f ? 448.0f : mb);
+              }
+              m[i] = ma;
+              m[i + 1] = mb;
             }
-            *reinterpret_cast<uint32_t*>(dst) = hdmoe_dev_pack_e4m3fn(m[0], m[1]) | (hdmoe_dev_pack_e4m3fn(m[2], m[3]) << 16);
-          } else {
-            u32x2 pk;
-            pk.x = hdmoe_dev_pack_bf16(m[0], m[1]);
-            pk.y = hdmoe_dev_pack_bf16(m[2], m[3]);
-            *reinterpret_cast<u32x2*>(dst) = pk;
+            const int byte = (wq * 32 + q * 8 + hi32 * 4) * EB;  // position of the 4 features in the staged row
+            uint8_t* const dst = row + ((((byte >> 4) ^ (tok32 & 7)) << 4) | (byte & 15));
+            if constexpr (FP8) {
+              *reinterpret_cast<uint32_t*>(dst) = hdmoe_dev_pack_e4m3fn(m[0], m[1]) | (hdmoe_dev_pack_e4m3fn(m[2], m[3]) << 16);
+            } else {
+              u32x2 pk;
+              pk.x = hdmoe_dev_pack_bf16(m[0], m[1]);
+              pk.y = hdmoe_dev_pack_bf16(m[2], m[3]);
+              *reinterpret_cast<u32x2*>(dst) = pk;
+            }
           }
         }
+      };
+      if constexpr (FP8) {
+        const int next = __builtin_amdgcn_readfirstlane(inv_next < 0.0f ? 0 : (inv_next == 1.0f ? 1 : 2));
+        if (next == 0) swiglu_tile(std::integral_constant<int, 0>{});
+        else if (next == 1) swiglu_tile(std::integral_constant<int, 1>{});
+        else swiglu_tile(std::integral_constant<int, 2>{});
+      } else {
+        swiglu_tile(std::integral_constant<int, 1>{});
       }
       __syncthreads();  // the tile's 256 x 128 outputs are staged
       constexpr int LANES_PER_ROW = ROWB / 16;
