@@ -15,6 +15,8 @@ LIB_PATH = os.path.join(_HERE, "libhdmoe.so")
 
 W_BF16 = 0
 W_E4M3FN = 1
+SRC_BF16 = 0
+SRC_F32 = 2
 MAX_EXPERTS = 16
 E_NULL, E_SHAPE, E_WORKSPACE, E_LAUNCH = -1, -2, -3, -4
 TOPK = 2
@@ -76,6 +78,8 @@ SIGNATURES = {
     "hdmoe_linear": (c_int, [c_int, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "hdmoe_silu_mul_bf16": (c_int, [c_void_p, c_void_p, c_int64, c_void_p, c_void_p]),
     "hdmoe_scale_to_bf16": (c_int, [c_int, c_void_p, c_int64, c_void_p, c_void_p, c_void_p]),
+    "hdmoe_stochastic_round_e4m3fn": (c_int, [c_int, c_void_p, ctypes.c_int64, c_void_p, ctypes.c_uint64, c_void_p,
+                                              c_void_p]),
     "hdmoe_ln_modulate_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, ctypes.c_float, c_void_p,
                                        c_void_p]),
     "hdmoe_combine_gated_residual": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,

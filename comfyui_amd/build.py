@@ -11,7 +11,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libhdmoe.so")
-SOURCES = ["gate.hip", "dispatch.hip", "elementwise.hip", "gemm.hip", "layer.hip"]
+SOURCES = ["gate.hip", "dispatch.hip", "elementwise.hip", "gemm.hip", "layer.hip", "weights.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",

@@ -2,8 +2,10 @@
 scaled-fp8 Linear's `set_weight` when ModelPatcher merges a LoRA into fp8 weights
 (reference: comfy/float.py:14-67, called from comfy/ops.py:419-426).
 
-This is weight maintenance on the host side of the boundary, not part of the forward
-path, and is written with torch tensor ops. Each value is rounded to one of its two
+On a HIP device float32 / bfloat16 values going to float8_e4m3fn take the library's kernel
+(hdmoe_stochastic_round_e4m3fn, uniform numbers from Philox keyed by seed and element index). Everything
+else -- host tensors of an offloaded model, float8_e5m2, other source dtypes -- is weight plumbing on the
+host side of the boundary and is written with torch tensor ops below. Each value is rounded to one of its two
 neighbouring fp8 values, the upper one with probability equal to its fractional
 position between them; like the reference the arithmetic runs in float16 and the
 uniform draws come from one generator seeded per tensor and consumed slice by slice.
@@ -40,6 +42,10 @@ def _round_slice(x, dtype, generator):
 def stochastic_rounding(value, dtype, seed=0):
     if dtype in (torch.float32, torch.float16, torch.bfloat16):
         return value.to(dtype=dtype)
+    if (dtype == torch.float8_e4m3fn and value.is_cuda and value.is_contiguous()
+            and value.dtype in (torch.float32, torch.bfloat16)):
+        from . import functional as HF
+        return HF.stochastic_round_e4m3fn(value, None, seed)
     if dtype in _FORMATS:
         generator = torch.Generator(device=value.device)
         generator.manual_seed(seed)

@@ -151,6 +151,23 @@ def combine(y_sorted, inv_perm, topk_weight, shared):
     return out
 
 
+def stochastic_round_e4m3fn(weight, scale=None, seed=0):
+    """weight (fp32 or bf16, HIP) / scale (fp32 scalar tensor or None) -> float8_e4m3fn by stochastic rounding
+    (comfy/float.py:14-67 behind comfy/ops.py:419-426), one kernel."""
+    _need_hip(weight, "stochastic_round_e4m3fn weight")
+    if weight.dtype == torch.float32:
+        code = _lib.SRC_F32
+    elif weight.dtype == BF16:
+        code = _lib.SRC_BF16
+    else:
+        raise TypeError(f"stochastic_round_e4m3fn: expected float32 or bfloat16, got {weight.dtype}")
+    out = torch.empty(weight.shape, dtype=FP8, device=weight.device)
+    check(lib.hdmoe_stochastic_round_e4m3fn(code, ptr(weight), weight.numel(),
+                                            _scale_ptr(scale, weight.device, "stochastic_round_e4m3fn scale"),
+                                            int(seed) & 0xFFFFFFFFFFFFFFFF, ptr(out), _stream(weight)))
+    return out
+
+
 def _per_batch(t, what, D, device):
     """[B, D] (or [B, 1, D]) bf16 modulation rows -> contiguous [B, D]."""
     _need_hip(t, what, BF16)

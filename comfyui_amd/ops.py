@@ -244,8 +244,14 @@ def scaled_fp8_ops(fp8_matrix_mult=False, scale_input=False, override_dtype=None
 
             def set_weight(self, weight, inplace_update=False, seed=None, return_weight=False, **kwargs):
                 from .float_round import stochastic_rounding
-                weight = stochastic_rounding(weight / self.scale_weight.to(device=weight.device, dtype=weight.dtype),
-                                             self.weight.dtype, seed=seed)
+                if (weight.is_cuda and self.weight.dtype == torch.float8_e4m3fn and weight.is_contiguous()
+                        and weight.dtype in (torch.float32, torch.bfloat16)):
+                    # division, float16 rounding and stochastic rounding in one kernel
+                    from . import functional as HF
+                    weight = HF.stochastic_round_e4m3fn(weight, self.scale_weight.to(weight.device), seed or 0)
+                else:
+                    weight = stochastic_rounding(weight / self.scale_weight.to(device=weight.device, dtype=weight.dtype),
+                                                 self.weight.dtype, seed=seed)
                 if return_weight:
                     return weight
                 if inplace_update:

@@ -33,7 +33,7 @@
 extern "C" {
 #endif
 
-#define HDMOE_VERSION 101
+#define HDMOE_VERSION 102
 
 #define HDMOE_OK 0
 #define HDMOE_E_NULL (-1)      /* required pointer is NULL */
@@ -151,6 +151,17 @@ int hdmoe_scale_to_bf16(int src_dtype, const void* src, int64_t n, const float* 
  * Deterministic (a gather, no atomics). D % 8 == 0. */
 int hdmoe_combine(const void* y_sorted_bf16, const int32_t* inv_perm, const void* topk_weight_bf16,
                   const void* shared_bf16, int T, int D, void* out_bf16, hdmoe_stream_t stream);
+
+/* Weight maintenance of a scaled-fp8 Linear (comfy/ops.py:419-426 set_weight, comfy/float.py:14-67):
+ * out[i] = stochastic_round_e4m3fn( float16( src[i] / *scale_dev ) ), scale_dev NULL = 1. Each value lands on one of
+ * its two e4m3fn neighbours, the upper one with probability equal to its position between them; |v| >= 448
+ * saturates. The uniform numbers are Philox4x32-10(counter = i/4, key = seed), word i%4, not torch's generator:
+ * same (src, scale, seed) -> same bytes, whatever the launch. src_dtype: HDMOE_SRC_F32 or HDMOE_SRC_BF16 (then the
+ * scale and the quotient are rounded to bf16 first, as a bf16 tensor division does). out must be 4-byte aligned. */
+#define HDMOE_SRC_BF16 0
+#define HDMOE_SRC_F32 2
+int hdmoe_stochastic_round_e4m3fn(int src_dtype, const void* src, int64_t n, const float* scale_dev, uint64_t seed,
+                                  void* out_e4m3fn, hdmoe_stream_t stream);
 
 /* Feed-forward branch of a HiDream block around the layer (comfy/ldm/hidream/model.py:429-433, 515-523):
  *   n   = LayerNorm(x, eps, no affine) * (1 + scale_mlp) + shift_mlp      -> hdmoe_ln_modulate_bf16

@@ -48,6 +48,10 @@ def _lib():
         lib.ref_ln_modulate.restype = ctypes.c_int
         lib.ref_ln_modulate.argtypes = [ctypes.c_void_p] * 3 + [ctypes.c_int] * 3 + [ctypes.c_float, ctypes.c_void_p]
         lib.ref_gated_residual.restype = None
+        lib.ref_philox4x32_10.restype = None
+        lib.ref_stochastic_round_e4m3fn.restype = None
+        lib.ref_stochastic_round_e4m3fn.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p, ctypes.c_uint64,
+                                                    ctypes.c_int, ctypes.c_void_p]
         lib.ref_e4m3fn_encode.restype = None
         lib.ref_e4m3fn_decode_table.restype = None
         _LIB = lib
@@ -237,6 +241,29 @@ def moe_forward(x, params, mode, gate_result=None):
     y = (y.view(*topk_weight.shape, -1) * topk_weight.unsqueeze(-1)).sum(dim=1)
     y = y.view(*orig_shape).to(wtype)
     return y + ffn_swiglu(x, params["shared"], mode)
+
+
+# ------------------------------------------------------------- weight maintenance
+
+def philox4x32_10(ctr, key):
+    """The checker's Philox4x32-10: 4 counter words, 2 key words -> 4 output words."""
+    c = (ctypes.c_uint32 * 4)(*ctr)
+    k = (ctypes.c_uint32 * 2)(*key)
+    o = (ctypes.c_uint32 * 4)()
+    _lib().ref_philox4x32_10(c, k, o)
+    return list(o)
+
+
+def stochastic_round_e4m3fn(weight, scale=None, seed=0):
+    """float.py:14-67 behind ops.py:419-426 (weight / scale_weight, float16, stochastic rounding to e4m3fn) with
+    the uniform numbers of moe_ref.c (Philox, keyed by seed and element index). weight fp32 or bf16 -> e4m3fn."""
+    is_bf16 = weight.dtype == torch.bfloat16
+    src = weight.float().contiguous()
+    out = torch.empty(weight.shape, dtype=torch.uint8)
+    sc = None if scale is None else scale.detach().float().reshape(1).contiguous()
+    _lib().ref_stochastic_round_e4m3fn(_p(src), src.numel(), None if sc is None else _p(sc), seed, int(is_bf16),
+                                       _p(out))
+    return out.view(torch.float8_e4m3fn)
 
 
 # ------------------------------------------------------- feed-forward branch of a block

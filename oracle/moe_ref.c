@@ -248,3 +248,83 @@ void ref_combine(const uint16_t* y_sorted, const int32_t* inv_perm, const uint16
     }
   }
 }
+
+/* ---- stochastic rounding to float8_e4m3fn (float.py:14-67, ops.py:419-426) ---------------------- */
+
+/* Philox4x32-10 (Salmon et al., SC'11), restated here so the checker shares no code with the kernels.
+ * Pinned by the paper's known-answer vectors in the tests. */
+void ref_philox4x32_10(const uint32_t ctr_in[4], const uint32_t key_in[2], uint32_t out[4]) {
+  uint32_t c[4] = {ctr_in[0], ctr_in[1], ctr_in[2], ctr_in[3]};
+  uint32_t k[2] = {key_in[0], key_in[1]};
+  for (int round = 0; round < 10; ++round) {
+    uint64_t a = 0xD2511F53ull * (uint64_t)c[0];
+    uint64_t b = 0xCD9E8D57ull * (uint64_t)c[2];
+    uint32_t n[4];
+    n[0] = (uint32_t)(b >> 32) ^ c[1] ^ k[0];
+    n[1] = (uint32_t)(b & 0xffffffffu);
+    n[2] = (uint32_t)(a >> 32) ^ c[3] ^ k[1];
+    n[3] = (uint32_t)(a & 0xffffffffu);
+    memcpy(c, n, sizeof(c));
+    k[0] += 0x9E3779B9u;
+    k[1] += 0xBB67AE85u;
+  }
+  memcpy(out, c, sizeof(c));
+}
+
+/* fp32 -> nearest float16 value (round to nearest even), returned as fp32; overflow -> inf */
+static float round_to_f16(float f) {
+  if (f != f) return f;
+  float a = fabsf(f);
+  if (a >= 65520.0f) return copysignf(INFINITY, f);
+  if (a == 0.0f) return f;
+  int e;
+  (void)frexpf(a, &e);                 /* a = m * 2^e, m in [0.5,1) */
+  int lsb = (e - 1) - 10;              /* exponent of the last kept bit of a normal float16 */
+  if (lsb < -24) lsb = -24;            /* subnormal float16: fixed step 2^-24 */
+  float q = nearbyintf(ldexpf(a, -lsb)); /* default rounding mode: to nearest, ties to even */
+  return copysignf(ldexpf(q, lsb), f);
+}
+
+/* The procedure of float.py with the uniform number u in [0,1) passed in. Returns the e4m3fn value as fp32. */
+static float stochastic_round_value(float h, float u) {
+  if (h != h) return h;
+  float a = fabsf(h);
+  if (a == 0.0f) return 0.0f;
+  float exponent = floorf(log2f(a)) + 7.0f;       /* exact: log2f is exact on powers of two and monotone */
+  if (isinf(a)) exponent = 15.0f;
+  if (exponent < 0.0f) exponent = 0.0f;
+  if (exponent > 15.0f) exponent = 15.0f;
+  float pos, value;
+  if (exponent != 0.0f) {
+    pos = (a / ldexpf(1.0f, (int)exponent - 7) - 1.0f) * 8.0f;
+    value = ldexpf(1.0f, (int)exponent - 7) * (1.0f + floorf(pos + u) / 8.0f);
+  } else {
+    pos = a / ldexpf(1.0f, -9);
+    value = ldexpf(1.0f, -6) * (floorf(pos + u) / 8.0f);
+  }
+  if (!(value <= 448.0f)) value = 448.0f;
+  return copysignf(value, h);
+}
+
+/* src [n] fp32, *scale (NULL = 1) -> out [n] e4m3fn codes. src_is_bf16: src holds bf16 values (as fp32) and the
+ * division is a bf16 tensor division (scale and quotient rounded to bf16). */
+void ref_stochastic_round_e4m3fn(const float* src, int64_t n, const float* scale, uint64_t seed, int src_is_bf16,
+                                 uint8_t* out) {
+  const uint32_t key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)};
+  float s = scale ? *scale : 1.0f;
+  if (src_is_bf16) s = bf16_to_f32(f32_to_bf16(s));
+  for (int64_t i = 0; i < n; ++i) {
+    const uint64_t g = (uint64_t)i >> 2;
+    const uint32_t ctr[4] = {(uint32_t)g, (uint32_t)(g >> 32), 0u, 0u};
+    uint32_t r[4];
+    ref_philox4x32_10(ctr, key, r);
+    const float u = (float)(r[i & 3] >> 8) * (1.0f / 16777216.0f);
+    float x = src[i] / s;
+    if (src_is_bf16) x = bf16_to_f32(f32_to_bf16(x));
+    const float v = stochastic_round_value(round_to_f16(x), u);
+    uint8_t code;
+    ref_e4m3fn_encode(&v, &code, 1);                 /* v is representable: the search returns its code */
+    if (v == 0.0f) code = (x == 0.0f || !signbit(v)) ? 0x00 : 0x80;
+    out[i] = code;
+  }
+}
