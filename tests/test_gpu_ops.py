@@ -245,3 +245,27 @@ def test_layer_is_graph_capturable(dev):
             torch.cuda.synchronize()
             assert torch.equal(static_y, want)
             assert torch.equal(m(v), want)      # eager work between replays
+
+
+def test_checkpoint_file_onto_the_device_and_forward(dev, tmp_path):
+    """A scaled-fp8 .safetensors file is read tensor by tensor onto the GPU; the modules built from it take the
+    one-call fp8 path and match the oracle run on the same file's tensors."""
+    import os
+    from safetensors.torch import save_file
+    from comfyui_amd import checkpoint as C
+    from tests.test_gpu_layer import check_layer
+    pre = "model.diffusion_model."
+    layer = pre + "double_stream_blocks.0.block.ff_i"
+    sd, x = small_layer(seed=31, dim=512, tokens=300, weights="fp8")
+    full = {f"{layer}.{k}": v for k, v in sd.items()}
+    full[pre + "scaled_fp8"] = C.scaled_fp8_marker(torch.float8_e4m3fn, True)
+    path = os.path.join(tmp_path, "m.safetensors")
+    save_file(full, path)
+    modules, info = C.load_moe_layers(path, prefix=pre, device=dev)
+    m = modules[layer]
+    assert info["fp8_optimizations"] and m.experts[0].w1.weight.is_cuda and m.experts[0].w1.hdmoe_fp8_matrix_mult
+    assert m._collect(x.to(dev).reshape(-1, 512)) is not None          # the one-call path applies
+    from comfyui_amd import functional as HF
+    y = m(x.to(dev))
+    idx, w = HF.gate_top2(x.to(dev).reshape(-1, 512), m.gate.weight)
+    check_layer(sd, x, "fp8", y.cpu(), idx.cpu(), w.cpu(), 4)
