@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the HiDream MoE SwiGLU feed-forward layer on one MI355X.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg3|cfg2|cfg1|cfg5-256|cfg5-4096] [--no-cpu-baseline]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg3|cfg2|cfg1|cfg5-256|cfg5-4096|cfg3-branch] [--aux-kernels] [--no-cpu-baseline]
 
 A step is one forward of comfyui_amd.hidream.MOEFeedForwardSwiGLU (gate, dispatch, quantise,
 grouped fp8 GEMMs, combine, shared expert) over one synthetic batch that is already resident in
@@ -104,14 +104,52 @@ def cpu_baseline(cfg, sd, sample_tokens):
                        f"per call), {dt:.2f} s, torch CPU threads={torch.get_num_threads()}, os.cpu_count()={os.cpu_count()}")
 
 
+def aux_kernels(dev, module, x):
+    """Stand-alone timings of the kernels around the layer: algorithmic bytes / time against the HBM figure."""
+    from comfyui_amd import functional as HF
+    B, S, D = x.shape
+    T = B * S
+    g = torch.Generator().manual_seed(2)
+    shift, scale, gate = ((torch.randn((B, D), generator=g) * 0.3).to(torch.bfloat16).to(dev) for _ in range(3))
+    x2 = x.reshape(T, D)
+    idx, w = HF.gate_top2(x2, module.gate.weight)
+    _, _, perm, inv = HF.dispatch(idx, len(module.experts))
+    y = torch.randn((2 * T, D), device=dev).to(torch.bfloat16)
+    sh = torch.randn((T, D), device=dev).to(torch.bfloat16)
+    wt = module.experts[0].w1
+    w32 = torch.randn(wt.weight.shape, device=dev) * 0.02
+
+    def timed(fn, nbytes, reps=50):
+        for _ in range(5):
+            fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / reps
+        return {"ms": ms, "bytes": nbytes, "GBps": nbytes / ms / 1e6, "frac_of_hbm_peak": nbytes / ms / 1e6 / PEAK_HBM_GBPS}
+
+    return {
+        "ln_modulate": timed(lambda: HF.ln_modulate(x2, scale, shift, S), 2 * T * D * 2),
+        "combine": timed(lambda: HF.combine(y, inv, w, sh), 4 * T * D * 2 + T * 12),
+        "combine_gated_residual": timed(lambda: HF.combine_gated_residual(y, inv, w, sh, gate, x2, S), 5 * T * D * 2 + T * 12),
+        "stochastic_round_e4m3fn": timed(lambda: HF.stochastic_round_e4m3fn(w32, wt.scale_weight, 1), w32.numel() * 5),
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="cfg3", choices=["cfg1", "cfg2", "cfg3", "cfg5-256", "cfg5-4096"])
+    ap.add_argument("--workload", default="cfg3", choices=["cfg1", "cfg2", "cfg3", "cfg5-256", "cfg5-4096", "cfg3-branch"])
     ap.add_argument("--cpu-sample-tokens", type=int, default=8192)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--aux-kernels", action="store_true",
+                    help="also time the stand-alone kernels outside the layer (LayerNorm+modulation, gated-residual "
+                         "combine, stochastic rounding of one expert weight) and report them under \"aux\"")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also run one plain 256 MiB device copy, whose FETCH_SIZE/WRITE_SIZE readings calibrate the counters")
     args = ap.parse_args()
@@ -128,7 +166,8 @@ def main():
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    cfg = synth.make_config(args.workload)
+    branch = args.workload.endswith("-branch")   # the block's whole feed-forward branch: x + gate * layer(LN-mod(x))
+    cfg = synth.make_config(args.workload.replace("-branch", ""))
     sd = synth.to_state_dict(cfg["master"], cfg["weights"])
     cfg["master"] = None
     module = synth.build_module({k: v.to(dev) for k, v in sd.items()}, cfg["weights"], dev)
@@ -146,17 +185,24 @@ def main():
         torch.cuda.synchronize()
         del src_cal, dst_cal
 
+    if branch:
+        g = torch.Generator().manual_seed(1)
+        shift, scale, gate_mlp = ((torch.randn((B, 1, D), generator=g) * 0.3).to(torch.bfloat16).to(dev) for _ in range(3))
+        forward = lambda **kw: module.forward_branch(x, shift, scale, gate_mlp, **kw)
+    else:
+        forward = lambda **kw: module(x, **kw)
+
     hip = HipEvents()
     with torch.no_grad():
         for _ in range(args.warmup):
-            y = module(x)
+            y = forward()
         torch.cuda.synchronize()
         # K timed steps; every step also records the per-stage events on the launch stream
         ev_sets = [hip.create(len(STAGE_NAMES) + 1) for _ in range(args.steps)]
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for k in range(args.steps):
-            y = module(x, stage_events=ev_sets[k])
+            y = forward(stage_events=ev_sets[k])
         torch.cuda.synchronize()
         t1 = time.perf_counter()
     if bool(torch.isnan(y.float()).any()):
@@ -207,6 +253,9 @@ def main():
                                      "with exact logit ties on every 64th token",
                          "cfg5-4096": "cfg5: 4096 tokens, fp8 weights, skewed routing (about 70% of tokens pick expert "
                                       "0) with exact logit ties on every 64th token",
+                         "cfg3-branch": "cfg3 tokens and weights through the block's whole feed-forward branch: x + gate_mlp * "
+                                        "layer(LayerNorm(x) * (1 + scale_mlp) + shift_mlp), one enqueue (stage 'gate' "
+                                        "includes the LayerNorm kernel, stage 'combine' the gated residual)",
                          "cfg3": "cfg3 (headline): 2x4096 = 8192 tokens x 2560, scaled fp8 e4m3fn weights "
                                  "(scale_weight = amax/448, scale_input = 1.0), bf16 gate, x ~ N(0,1) with 1% "
                                  "outlier channels x20, 4 routed experts (hidden 6912) top-2 + shared expert (hidden 3584)"}[args.workload],
@@ -234,6 +283,8 @@ def main():
             "avg_launch_ms": stage_ms["gemm_gate_up"],
         },
     }
+    if args.aux_kernels:
+        out["aux"] = aux_kernels(dev, module, x)
     if not args.no_cpu_baseline:
         del module
         torch.cuda.empty_cache()

@@ -202,6 +202,12 @@ __device__ __forceinline__ void unpack8(const uint4& a, float (&f)[8]) {
   f[4] = bf16_lo(a.z); f[5] = bf16_hi(a.z); f[6] = bf16_lo(a.w); f[7] = bf16_hi(a.w);
 }
 
+__device__ __forceinline__ void round2(float& a, float& b) {
+  const uint32_t p = hdmoe_dev_pack_bf16(a, b);
+  a = __uint_as_float(p << 16);
+  b = __uint_as_float(p & 0xffff0000u);
+}
+
 __device__ __forceinline__ uint4 modulate8(const uint4& xv, const uint4& sc, const uint4& sh, float mean, float rstd) {
   float x[8], a[8], b[8];
   unpack8(xv, x);
@@ -210,15 +216,14 @@ __device__ __forceinline__ uint4 modulate8(const uint4& xv, const uint4& sc, con
   uint32_t o[4];
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    float r[2];
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      const int i = 2 * j + h;
-      const float n = hdmoe_round_bf16((x[i] - mean) * rstd);     // LayerNorm output as a bf16 tensor
-      const float m = hdmoe_round_bf16(1.0f + a[i]);              // (1 + scale)
-      r[h] = hdmoe_round_bf16(hdmoe_round_bf16(n * m) + b[i]);    // n * (1 + scale) + shift
-    }
-    o[j] = (uint32_t)hdmoe_f32_to_bf16(r[0]) | ((uint32_t)hdmoe_f32_to_bf16(r[1]) << 16);
+    // two elements at a time: one packed conversion (v_cvt_pk_bf16_f32, round to nearest even) per rounding point
+    float n0 = (x[2 * j] - mean) * rstd, n1 = (x[2 * j + 1] - mean) * rstd;  // LayerNorm output as a bf16 tensor
+    round2(n0, n1);
+    float m0 = 1.0f + a[2 * j], m1 = 1.0f + a[2 * j + 1];                    // (1 + scale)
+    round2(m0, m1);
+    float p0 = n0 * m0, p1 = n1 * m1;                                        // n * (1 + scale)
+    round2(p0, p1);
+    o[j] = hdmoe_dev_pack_bf16(p0 + b[2 * j], p1 + b[2 * j + 1]);            // + shift
   }
   return make_uint4(o[0], o[1], o[2], o[3]);
 }
