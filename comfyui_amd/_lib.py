@@ -17,6 +17,8 @@ W_BF16 = 0
 W_E4M3FN = 1
 SRC_BF16 = 0
 SRC_F32 = 2
+ACT_NONE = 0
+ACT_GELU = 1
 MAX_EXPERTS = 16
 E_NULL, E_SHAPE, E_WORKSPACE, E_LAUNCH = -1, -2, -3, -4
 TOPK = 2
@@ -36,6 +38,11 @@ class FfnWeights(ctypes.Structure):
         ("scale_w1", c_void_p), ("scale_w2", c_void_p), ("scale_w3", c_void_p),
         ("scale_in1", c_void_p), ("scale_in2", c_void_p), ("scale_in3", c_void_p),
     ]
+
+
+class LinearWeights(ctypes.Structure):
+    """hdmoe_linear_weights"""
+    _fields_ = [("weight", c_void_p), ("bias", c_void_p)]
 
 
 class LayerArgs(ctypes.Structure):
@@ -78,6 +85,8 @@ SIGNATURES = {
     "hdmoe_linear": (c_int, [c_int, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "hdmoe_silu_mul_bf16": (c_int, [c_void_p, c_void_p, c_int64, c_void_p, c_void_p]),
     "hdmoe_scale_to_bf16": (c_int, [c_int, c_void_p, c_int64, c_void_p, c_void_p, c_void_p]),
+    "hdmoe_grouped_linear": (c_int, [c_void_p, c_void_p, c_int, c_int, ctypes.POINTER(LinearWeights), c_void_p, c_void_p,
+                                     c_int, ctypes.POINTER(LinearWeights), c_void_p, c_int, c_int, c_int, c_void_p]),
     "hdmoe_stochastic_round_e4m3fn": (c_int, [c_int, c_void_p, ctypes.c_int64, c_void_p, ctypes.c_uint64, c_void_p,
                                               c_void_p]),
     "hdmoe_ln_modulate_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, ctypes.c_float, c_void_p,

@@ -302,11 +302,12 @@ extern "C" int hdmoe_gate_top2(const void* x_bf16, const void* gate_w_bf16, int 
   if (T == 0) return HDMOE_OK;
   hipStream_t s = static_cast<hipStream_t>(stream);
   switch (E) {
-    case 2: return launch_gate<2>(x_bf16, gate_w_bf16, T, D, topk_idx, topk_weight_bf16, s);
-    case 4: return launch_gate<4>(x_bf16, gate_w_bf16, T, D, topk_idx, topk_weight_bf16, s);
-    case 8: return launch_gate<8>(x_bf16, gate_w_bf16, T, D, topk_idx, topk_weight_bf16, s);
-    case 16: return launch_gate<16>(x_bf16, gate_w_bf16, T, D, topk_idx, topk_weight_bf16, s);
-    default: return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_gate_top2: E=%d not in {2,4,8,16}", E);
+#define HDMOE_GATE_CASE(n) case n: return launch_gate<n>(x_bf16, gate_w_bf16, T, D, topk_idx, topk_weight_bf16, s);
+    HDMOE_GATE_CASE(2) HDMOE_GATE_CASE(3) HDMOE_GATE_CASE(4) HDMOE_GATE_CASE(5) HDMOE_GATE_CASE(6)
+    HDMOE_GATE_CASE(7) HDMOE_GATE_CASE(8) HDMOE_GATE_CASE(9) HDMOE_GATE_CASE(10) HDMOE_GATE_CASE(11)
+    HDMOE_GATE_CASE(12) HDMOE_GATE_CASE(13) HDMOE_GATE_CASE(14) HDMOE_GATE_CASE(15) HDMOE_GATE_CASE(16)
+#undef HDMOE_GATE_CASE
+    default: return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_gate_top2: E=%d not in 2..16", E);
   }
 }
 

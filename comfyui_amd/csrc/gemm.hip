@@ -54,7 +54,7 @@ constexpr int GROUP_M = 4;     // m-tiles per raster band
 constexpr int NTHREADS = 512;
 constexpr int MAX_GROUPS = HDMOE_MAX_EXPERTS + 1;
 
-enum Mode { FP8_SWIGLU = 0, FP8_PLAIN = 1, BF16_SWIGLU = 2, BF16_PLAIN = 3 };
+enum Mode { FP8_SWIGLU = 0, FP8_PLAIN = 1, BF16_SWIGLU = 2, BF16_PLAIN = 3, BF16_PLAIN_BIAS = 4 };
 
 struct GemmGroup {
   const uint8_t* a;     // activations; row indices below are relative to this base
@@ -68,6 +68,8 @@ struct GemmGroup {
   int row_begin;        // >= 0: static segment [row_begin, row_end); < 0: offsets[dyn], offsets[dyn+1]
   int row_end;
   int dyn;
+  const uint16_t* bias; // BF16_PLAIN_BIAS: bf16 [n_out] added before the output is rounded, NULL = none
+  int act;              // BF16_PLAIN_BIAS: 0 = none, 1 = erf GELU on the rounded output
   int n_out;            // output features (H for swiglu, N for plain)
   int kbytes;           // bytes per row of a and of the weights
 };
@@ -93,6 +95,7 @@ template <int MODE>
 __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs args) {
   constexpr bool FP8 = (MODE == FP8_SWIGLU || MODE == FP8_PLAIN);
   constexpr bool SWIGLU = (MODE == FP8_SWIGLU || MODE == BF16_SWIGLU);
+  constexpr bool BIAS = (MODE == BF16_PLAIN_BIAS);  // Linear with bias and optional GELU (bf16 weights)
   constexpr int FEAT_PER_TILE = SWIGLU ? BN / 2 : BN;  // output features per block tile
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
 
@@ -276,7 +279,20 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
   // Per-tile epilogue factors. They are loaded before the K loop: a load issued after the next tile's
   // global->LDS requests would make the epilogue wait for those as well (one in-order counter).
   float ep_a = 1.0f, ep_b = 1.0f, ep_next = 1.0f;
+  u32x2 ep_bias[2][4];  // BIAS: the 2 x 4 feature quads of this lane, 4 bf16 each
   auto load_scales = [&](const Tile& d) {
+    if constexpr (BIAS) {
+      const GemmGroup& gg = args.g[d.g];
+#pragma unroll
+      for (int ft = 0; ft < 2; ++ft)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          u32x2 z = {0u, 0u};
+          if (gg.bias != nullptr)
+            z = *reinterpret_cast<const u32x2*>(gg.bias + d.n0 + wq * 64 + ft * 32 + q * 8 + (lane >> 5) * 4);
+          ep_bias[ft][q] = z;
+        }
+    }
     if constexpr (FP8) {
       const GemmGroup& gg = args.g[d.g];
       const float s_in = gg.s_in ? *gg.s_in : 1.0f;
@@ -383,8 +399,27 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
 #pragma unroll
           for (int q = 0; q < 4; ++q) {
             u32x2 pk;
-            pk.x = hdmoe_dev_pack_bf16(acc[ft][tt][q * 4 + 0] * sc, acc[ft][tt][q * 4 + 1] * sc);
-            pk.y = hdmoe_dev_pack_bf16(acc[ft][tt][q * 4 + 2] * sc, acc[ft][tt][q * 4 + 3] * sc);
+            if constexpr (BIAS) {
+              // F.linear with bias: bf16(acc + bias); then F.gelu (erf form) of that bf16 tensor, rounded again
+              // (/root/reference/comfy/ldm/hunyuan3dv2_1/hunyuandit.py:14-26, 44-50)
+              const u32x2 bq = ep_bias[ft][q];
+              float v[4] = {acc[ft][tt][q * 4 + 0] + __uint_as_float(bq.x << 16),
+                            acc[ft][tt][q * 4 + 1] + __uint_as_float(bq.x & 0xffff0000u),
+                            acc[ft][tt][q * 4 + 2] + __uint_as_float(bq.y << 16),
+                            acc[ft][tt][q * 4 + 3] + __uint_as_float(bq.y & 0xffff0000u)};
+              if (gg.act == 1) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                  const float h = hdmoe_dev_round_bf16(v[i]);
+                  v[i] = 0.5f * h * (1.0f + erff(h * 0.70710678118654752440f));
+                }
+              }
+              pk.x = hdmoe_dev_pack_bf16(v[0], v[1]);
+              pk.y = hdmoe_dev_pack_bf16(v[2], v[3]);
+            } else {
+              pk.x = hdmoe_dev_pack_bf16(acc[ft][tt][q * 4 + 0] * sc, acc[ft][tt][q * 4 + 1] * sc);
+              pk.y = hdmoe_dev_pack_bf16(acc[ft][tt][q * 4 + 2] * sc, acc[ft][tt][q * 4 + 3] * sc);
+            }
             *reinterpret_cast<u32x2*>(buf + tok32 * 128 + (((ft * 4 + q) ^ (tok32 & 7)) << 4) + hi32 * 8) = pk;
           }
         }
@@ -530,6 +565,49 @@ int hdmoe_launch_ffn_gemm(bool swiglu, int weight_dtype, const uint8_t* a_dyn, c
                 : launch_grouped<BF16_PLAIN>(args, tile_bound, s, what);
 }
 
+// Linear with bias and optional GELU over expert row segments plus an optional static group (bf16 weights):
+// the two stages of a GELU feed-forward (/root/reference/comfy/ldm/hunyuan3dv2_1/hunyuandit.py:28-50, 114-188).
+int hdmoe_launch_linear_groups(const uint8_t* a_dyn, const int32_t* offsets, int rows_dyn, int n_dyn,
+                               const hdmoe_linear_weights* experts, uint8_t* out_dyn, const uint8_t* a_static,
+                               int rows_static, const hdmoe_linear_weights* shared, uint8_t* out_static, int K, int N,
+                               int act, hipStream_t s, const char* what) {
+  GemmArgs args;
+  memset(&args, 0, sizeof(args));
+  args.offsets = offsets;
+  args.n_offsets = n_dyn;
+  int G = 0, tile_bound = 0;
+  auto fill = [&](GemmGroup& gg, const hdmoe_linear_weights& w) {
+    gg.b0 = static_cast<const uint8_t*>(w.weight);
+    gg.bias = static_cast<const uint16_t*>(w.bias);
+    gg.act = act;
+    gg.n_out = N;
+    gg.kbytes = K * 2;
+  };
+  for (int e = 0; e < n_dyn; ++e, ++G) {
+    GemmGroup& gg = args.g[G];
+    fill(gg, experts[e]);
+    gg.a = a_dyn;
+    gg.out = out_dyn;
+    gg.row_begin = -1;
+    gg.dyn = e;
+    if (!gg.b0) return hdmoe_fail(HDMOE_E_NULL, "%s: expert %d has a NULL weight", what, e);
+  }
+  if (n_dyn > 0) tile_bound += (rows_dyn / BM + n_dyn) * (N / BN);
+  if (shared != nullptr && rows_static > 0) {
+    GemmGroup& gg = args.g[G];
+    fill(gg, *shared);
+    gg.a = a_static;
+    gg.out = out_static;
+    gg.row_begin = 0;
+    gg.row_end = rows_static;
+    if (!gg.b0) return hdmoe_fail(HDMOE_E_NULL, "%s: static group has a NULL weight", what);
+    tile_bound += ((rows_static + BM - 1) / BM) * (N / BN);
+    ++G;
+  }
+  args.G = G;
+  return launch_grouped<BF16_PLAIN_BIAS>(args, tile_bound, s, what);
+}
+
 // Size rules shared by the entry points: K bytes per row must be a multiple of the
 // 128-byte K step; total bytes of each operand must fit the 32-bit buffer range.
 int hdmoe_check_gemm_shape(const char* what, int weight_dtype, long rows, int K, int N, int feat_per_tile) {
@@ -588,4 +666,31 @@ extern "C" int hdmoe_linear(int weight_dtype, const void* a, int rows, int K, in
   return hdmoe_launch_ffn_gemm(false, weight_dtype, nullptr, nullptr, 0, 0, nullptr, nullptr,
                                static_cast<const uint8_t*>(a), rows, &fw, static_cast<uint8_t*>(out_bf16), 0, 0, K, N,
                                static_cast<hipStream_t>(stream), "hdmoe_linear");
+}
+
+extern "C" int hdmoe_grouped_linear(const void* a_bf16, const int32_t* offsets, int rows_total, int E,
+                                    const hdmoe_linear_weights* experts, void* out_bf16, const void* a_static_bf16,
+                                    int rows_static, const hdmoe_linear_weights* shared, void* out_static_bf16, int K,
+                                    int N, int act, hdmoe_stream_t stream) {
+  if (E < 0 || E > HDMOE_MAX_EXPERTS) return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_grouped_linear: E=%d", E);
+  if (act != HDMOE_ACT_NONE && act != HDMOE_ACT_GELU) return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_grouped_linear: act=%d", act);
+  if (E > 0) {
+    HDMOE_REQUIRE_PTR(a_bf16);
+    HDMOE_REQUIRE_PTR(offsets);
+    HDMOE_REQUIRE_PTR(experts);
+    HDMOE_REQUIRE_PTR(out_bf16);
+  }
+  if (rows_static > 0) {
+    HDMOE_REQUIRE_PTR(a_static_bf16);
+    HDMOE_REQUIRE_PTR(shared);
+    HDMOE_REQUIRE_PTR(out_static_bf16);
+  }
+  if (rows_static < 0) return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_grouped_linear: rows_static=%d", rows_static);
+  const long rows_max = rows_total > rows_static ? rows_total : rows_static;
+  if (int rc = hdmoe_check_gemm_shape("hdmoe_grouped_linear", HDMOE_W_BF16, rows_max, K, N, BN)) return rc;
+  if ((E == 0 || rows_total == 0) && rows_static == 0) return HDMOE_OK;
+  return hdmoe_launch_linear_groups(static_cast<const uint8_t*>(a_bf16), offsets, rows_total, rows_total > 0 ? E : 0,
+                                    experts, static_cast<uint8_t*>(out_bf16), static_cast<const uint8_t*>(a_static_bf16),
+                                    rows_static, shared, static_cast<uint8_t*>(out_static_bf16), K, N, act,
+                                    static_cast<hipStream_t>(stream), "hdmoe_grouped_linear");
 }

@@ -7,7 +7,7 @@ import ctypes
 import torch
 
 from . import _lib
-from ._lib import FfnWeights, LayerArgs, LayerLayout, W_BF16, W_E4M3FN, check, lib, ptr
+from ._lib import FfnWeights, LayerArgs, LayerLayout, LinearWeights, W_BF16, W_E4M3FN, check, lib, ptr
 
 FP8 = torch.float8_e4m3fn
 BF16 = torch.bfloat16
@@ -149,6 +149,44 @@ def combine(y_sorted, inv_perm, topk_weight, shared):
     check(lib.hdmoe_combine(ptr(y_sorted), ptr(inv_perm), ptr(topk_weight), ptr(shared), T, D, ptr(out),
                             _stream(y_sorted)))
     return out
+
+
+def _linear_weights(weight, bias, K, N, what):
+    _need_hip(weight, f"{what} weight", BF16)
+    if tuple(weight.shape) != (N, K):
+        raise ValueError(f"{what}: weight shape {tuple(weight.shape)} != ({N}, {K})")
+    lw = LinearWeights()
+    lw.weight = ptr(weight)
+    if bias is not None:
+        _need_hip(bias, f"{what} bias", BF16)
+        if tuple(bias.shape) != (N,):
+            raise ValueError(f"{what}: bias shape {tuple(bias.shape)} != ({N},)")
+        lw.bias = ptr(bias)
+    return lw
+
+
+def grouped_linear(a_sorted, offsets, experts, a_static=None, shared=None, act="none"):
+    """Linear (+ bias, + erf GELU) of every expert over its row segment of `a_sorted` [rows, K] and, optionally, of
+    one more (weight, bias) over all rows of `a_static`, in one launch. experts: list of (weight [N,K], bias [N] or
+    None). Returns (out_sorted [rows, N], out_static [rows_static, N] or None)."""
+    code = {"none": _lib.ACT_NONE, "gelu": _lib.ACT_GELU}[act]
+    _need_hip(a_sorted, "grouped_linear a", BF16)
+    rows, K = a_sorted.shape
+    N = experts[0][0].shape[0] if experts else shared[0].shape[0]
+    E = len(experts)
+    arr = (LinearWeights * max(E, 1))(*[_linear_weights(w, b, K, N, f"grouped_linear expert {i}")
+                                        for i, (w, b) in enumerate(experts)])
+    out = torch.empty((rows, N), dtype=BF16, device=a_sorted.device)
+    out_static, sh, rows_static = None, None, 0
+    if shared is not None:
+        _need_hip(a_static, "grouped_linear a_static", BF16)
+        rows_static = a_static.shape[0]
+        sh = _linear_weights(shared[0], shared[1], K, N, "grouped_linear shared")
+        out_static = torch.empty((rows_static, N), dtype=BF16, device=a_sorted.device)
+    check(lib.hdmoe_grouped_linear(ptr(a_sorted), ptr(offsets), rows, E, arr, ptr(out), ptr(a_static), rows_static,
+                                   ctypes.byref(sh) if sh is not None else None, ptr(out_static), K, N, code,
+                                   _stream(a_sorted)))
+    return out, out_static
 
 
 def stochastic_round_e4m3fn(weight, scale=None, seed=0):

@@ -33,7 +33,7 @@
 extern "C" {
 #endif
 
-#define HDMOE_VERSION 102
+#define HDMOE_VERSION 103
 
 #define HDMOE_OK 0
 #define HDMOE_E_NULL (-1)      /* required pointer is NULL */
@@ -60,7 +60,7 @@ const char* hdmoe_last_error(void);
  * Writes topk_idx [T,2] int32 and topk_weight [T,2] bf16; slot 0 holds the larger
  * score, equal scores go to the lower expert index. Logits and scores are rounded
  * to bf16 between the three steps as the three torch kernels do.
- * D % 8 == 0, E in {2,4,8,16}. */
+ * D % 8 == 0, 2 <= E <= 16. The same gate serves comfy/ldm/hunyuan3dv2_1/hunyuandit.py:73-112 (E = 6 or 8). */
 int hdmoe_gate_top2(const void* x_bf16, const void* gate_w_bf16, int T, int D, int E,
                     int32_t* topk_idx, void* topk_weight_bf16, hdmoe_stream_t stream);
 
@@ -151,6 +151,22 @@ int hdmoe_scale_to_bf16(int src_dtype, const void* src, int64_t n, const float* 
  * Deterministic (a gather, no atomics). D % 8 == 0. */
 int hdmoe_combine(const void* y_sorted_bf16, const int32_t* inv_perm, const void* topk_weight_bf16,
                   const void* shared_bf16, int T, int D, void* out_bf16, hdmoe_stream_t stream);
+
+/* Linear with bias (and optional erf GELU) over the expert row segments of a dispatched batch, plus optionally one
+ * more group over all rows of another input (a shared expert), in one launch: the two stages of the GELU
+ * feed-forward experts of comfy/ldm/hunyuan3dv2_1/hunyuandit.py:28-50 as MoEBlock (:114-188) runs them.
+ *   out[r, :] = act( bf16( a[r, :] . W_e^T + bias_e ) ),  r in [offsets[e], offsets[e+1])
+ * bf16 activations, weights [N,K] and biases [N] (bias NULL = none); K % 64 == 0, N % 256 == 0. */
+#define HDMOE_ACT_NONE 0
+#define HDMOE_ACT_GELU 1
+typedef struct {
+  const void* weight; /* [N,K] bf16 */
+  const void* bias;   /* [N] bf16 or NULL */
+} hdmoe_linear_weights;
+int hdmoe_grouped_linear(const void* a_bf16, const int32_t* offsets, int rows_total, int E,
+                         const hdmoe_linear_weights* experts, void* out_bf16, const void* a_static_bf16,
+                         int rows_static, const hdmoe_linear_weights* shared, void* out_static_bf16, int K, int N,
+                         int act, hdmoe_stream_t stream);
 
 /* Weight maintenance of a scaled-fp8 Linear (comfy/ops.py:419-426 set_weight, comfy/float.py:14-67):
  * out[i] = stochastic_round_e4m3fn( float16( src[i] / *scale_dev ) ), scale_dev NULL = 1. Each value lands on one of

@@ -243,6 +243,72 @@ def moe_forward(x, params, mode, gate_result=None):
     return y + ffn_swiglu(x, params["shared"], mode)
 
 
+# --------------------------------------------- Hunyuan3D-2.1 MoEBlock (hunyuandit.py:8-188)
+
+def linear_bias(x, weight, bias):
+    """operations.Linear with bias at x.dtype: the contraction and the bias add in fp32, one rounding to x.dtype
+    (what a GEMM with a bias epilogue does; torch's own bf16 F.linear agrees to one step, see the tests)."""
+    acc = x.float() @ weight.float().t()
+    if bias is not None:
+        acc = acc + bias.float()
+    return acc.to(x.dtype)
+
+
+def gelu_feed_forward(x, ff):
+    """hunyuandit.py:28-50: Linear -> F.gelu (erf form) -> Dropout(0) -> Linear. ff = (w_in, b_in, w_out, b_out)."""
+    w_in, b_in, w_out, b_out = ff
+    return linear_bias(F.gelu(linear_bias(x, w_in, b_in)), w_out, b_out)
+
+
+def hunyuan_moe_block(x, params, gate_result=None):
+    """hunyuandit.py:131-187 (inference branch), literally: gate, argsort of the flat expert ids, per expert the
+    tokens in sorted order, output times the routing weight, index_add_ into a zero cache in expert order, plus
+    the shared expert. params: dict(gate=Wg [E,D], experts=[(w_in,b_in,w_out,b_out)]*E, shared=(...))."""
+    orig_shape = x.shape
+    x2 = x.reshape(-1, x.shape[-1])
+    if gate_result is None:
+        topk_idx, topk_weight, _, _ = gate_torch(x2, params["gate"])
+    else:
+        topk_idx, topk_weight = gate_result
+        topk_idx = topk_idx.long()
+        topk_weight = topk_weight.to(x.dtype)
+    top_k = topk_idx.shape[1]
+    flat_idx = topk_idx.reshape(-1)
+    flat_w = topk_weight.reshape(-1, 1)
+    cache = torch.zeros_like(x2)
+    idxs = flat_idx.argsort(stable=True)
+    ends = flat_idx.bincount(minlength=len(params["experts"])).cumsum(0)
+    token_idxs = idxs // top_k
+    for i, end in enumerate(ends.tolist()):
+        start = 0 if i == 0 else int(ends[i - 1])
+        if start == end:
+            continue
+        tok = token_idxs[start:end]
+        out = gelu_feed_forward(x2[tok], params["experts"][i])
+        out.mul_(flat_w[idxs[start:end]])
+        cache.index_add_(0, tok, out)
+    return cache.view(*orig_shape) + gelu_feed_forward(x, params["shared"])
+
+
+def hunyuan_moe_block_dense(x, params, topk_idx, topk_weight):
+    """Brute force used to pin hunyuan_moe_block: every expert on every token, selected by mask."""
+    x2 = x.reshape(-1, x.shape[-1])
+    outs = torch.stack([gelu_feed_forward(x2, ff) for ff in params["experts"]], dim=0)   # [E,T,D]
+    T = x2.shape[0]
+    sel = outs[topk_idx.long().t(), torch.arange(T).unsqueeze(0)]                        # [K,T,D]
+    y = (sel.permute(1, 0, 2) * topk_weight.to(x.dtype).unsqueeze(-1)).sum(dim=1)
+    return y.view(x.shape).to(x.dtype) + gelu_feed_forward(x, params["shared"])
+
+
+def hunyuan_params(state_dict, num_experts):
+    """MoEBlock state dict (keys experts.N.net.0.proj.*, experts.N.net.2.*, shared_experts.*, gate.weight)."""
+    def ff(prefix):
+        return (state_dict[prefix + "net.0.proj.weight"], state_dict.get(prefix + "net.0.proj.bias"),
+                state_dict[prefix + "net.2.weight"], state_dict.get(prefix + "net.2.bias"))
+    return dict(gate=state_dict["gate.weight"], experts=[ff(f"experts.{i}.") for i in range(num_experts)],
+                shared=ff("shared_experts."))
+
+
 # ------------------------------------------------------------- weight maintenance
 
 def philox4x32_10(ctr, key):

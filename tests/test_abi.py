@@ -73,7 +73,8 @@ def test_argument_errors_are_reported_without_a_device():
     assert L.hdmoe_gate_top2(None, p, 4, 2560, 4, p, p, None) == _lib.E_NULL
     assert b"x_bf16" in L.hdmoe_last_error()
     assert L.hdmoe_gate_top2(p, p, 4, 2561, 4, p, p, None) == _lib.E_SHAPE
-    assert L.hdmoe_gate_top2(p, p, 4, 2560, 3, p, p, None) == _lib.E_SHAPE
+    assert L.hdmoe_gate_top2(p, p, 4, 2560, 1, p, p, None) == _lib.E_SHAPE
+    assert L.hdmoe_gate_top2(p, p, 4, 2560, 17, p, p, None) == _lib.E_SHAPE
     assert L.hdmoe_gate_top2(p, p, 0, 2560, 4, p, p, None) == 0                 # empty input: nothing to do
     assert L.hdmoe_dispatch(p, 8, 17, p, p, p, p, p, 4096, None) == _lib.E_SHAPE
     assert L.hdmoe_dispatch(p, 100000, 4, p, p, p, p, p, 16, None) == _lib.E_WORKSPACE
