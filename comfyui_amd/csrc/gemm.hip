@@ -478,12 +478,16 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
 
 template <int MODE>
 int launch_grouped(const GemmArgs& args, int tile_bound, hipStream_t s, const char* what) {
-  static bool attr_set = false;  // per process and instantiation; setting it twice is harmless
-  if (!attr_set) {
+  // The opt-in for more than 64 KiB of dynamic LDS is a per-device function attribute: remembered per device
+  // and instantiation (a race between two threads sets it twice, which is harmless).
+  static bool attr_set[64] = {};
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) device = -1;
+  if (device < 0 || !attr_set[device]) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&grouped_gemm_kernel<MODE>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES);
     if (e != hipSuccess) return hdmoe_fail(HDMOE_E_LAUNCH, "%s: hipFuncSetAttribute: %s", what, hipGetErrorString(e));
-    attr_set = true;
+    if (device >= 0) attr_set[device] = true;
   }
   if (tile_bound <= 0) return HDMOE_OK;
   // persistent blocks: one per CU (128 KiB of LDS allow no second one), a multiple of the XCD count

@@ -116,8 +116,12 @@ extern "C" int hdmoe_moe_ffn(const hdmoe_layer_args* p, hdmoe_stream_t stream) {
   }
 
   int ev = 0;
+  hipError_t ev_err = hipSuccess;
   auto mark = [&]() {
-    if (p->stage_events) (void)hipEventRecord(static_cast<hipEvent_t>(p->stage_events[ev]), s);
+    if (p->stage_events) {
+      const hipError_t e = hipEventRecord(static_cast<hipEvent_t>(p->stage_events[ev]), s);
+      if (e != hipSuccess && ev_err == hipSuccess) ev_err = e;
+    }
     ++ev;
   };
   // the tokens the feed-forward sees: x itself, or LayerNorm(x) * (1 + scale) + shift (timed with the gate stage)
@@ -166,6 +170,8 @@ extern "C" int hdmoe_moe_ffn(const hdmoe_layer_args* p, hdmoe_stream_t stream) {
                                       fused_block ? p->mod_gate : nullptr, fused_block ? p->x : nullptr,
                                       fused_block ? p->tokens_per_batch : 1, T, D, p->out, s, "hdmoe_moe_ffn (combine)");
   mark();
+  if (rc == HDMOE_OK && ev_err != hipSuccess)
+    return hdmoe_fail(HDMOE_E_LAUNCH, "hdmoe_moe_ffn: hipEventRecord on a stage event: %s", hipGetErrorString(ev_err));
   return rc;
 }
 

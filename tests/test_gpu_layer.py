@@ -136,3 +136,27 @@ def test_benchmark_configs(dev, name, subset):
     got = HF.dispatch(idx.to(dev), 4)
     for a, b in zip(got, (counts_r, offs_r, perm_r, inv_r)):
         assert torch.equal(a.cpu(), b)
+
+
+def test_production_row_counts_are_ragged(dev):
+    """A single-stream block feeds image + text tokens: 2 x 4480 rows, not a multiple of any tile size, through the
+    full-size fp8 layer. Routing bit-exact on every token; outputs checked on a token subset that includes the
+    rows of the last, partial tile of every expert segment and of the shared expert."""
+    from comfyui_amd import functional as HF
+    cfg = synth.make_config("cfg2")
+    sd = synth.to_state_dict(cfg["master"], "fp8")
+    g = torch.Generator().manual_seed(77)
+    x = synth.make_input(g, 2 * 4480, batch=2)
+    y, idx, w, m = run_gpu(sd, x, "fp8", dev, synth.DIM)
+    T = x.shape[0] * x.shape[1]
+    xd = x.to(dev).reshape(T, -1)
+    _, offsets, perm, _ = HF.dispatch(idx.to(dev), 4)
+    offsets, perm = offsets.cpu().tolist(), perm.cpu()
+    picks = [torch.arange(T - 64, T), torch.arange(0, 32)]
+    for e in range(4):
+        seg_end = offsets[e + 1]
+        tail_start = offsets[e] + ((seg_end - offsets[e]) // 256) * 256      # first row of the segment's partial tile
+        rows = torch.arange(max(offsets[e], min(tail_start, seg_end - 16)), seg_end)
+        picks.append(perm[rows].long() // 2)
+    subset = torch.unique(torch.cat(picks))
+    check_layer(sd, x, "fp8", y, idx, w, 4, token_subset=subset)
