@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the HiDream MoE SwiGLU feed-forward layer on one MI355X.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg3|cfg2|cfg1|cfg5-256|cfg5-4096|cfg3-branch] [--aux-kernels] [--no-cpu-baseline]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg3|cfg2|cfg1|cfg5-256|cfg5-4096|cfg3-branch|cfg4 [--layers L]] [--aux-kernels] [--no-cpu-baseline]
 
 A step is one forward of comfyui_amd.hidream.MOEFeedForwardSwiGLU (gate, dispatch, quantise,
 grouped fp8 GEMMs, combine, shared expert) over one synthetic batch that is already resident in
@@ -144,7 +144,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="cfg3", choices=["cfg1", "cfg2", "cfg3", "cfg5-256", "cfg5-4096", "cfg3-branch"])
+    ap.add_argument("--workload", default="cfg3", choices=["cfg1", "cfg2", "cfg3", "cfg5-256", "cfg5-4096", "cfg3-branch", "cfg4"])
+    ap.add_argument("--layers", type=int, default=48, help="cfg4 only: number of stacked layers")
     ap.add_argument("--cpu-sample-tokens", type=int, default=8192)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--aux-kernels", action="store_true",
@@ -167,11 +168,25 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     branch = args.workload.endswith("-branch")   # the block's whole feed-forward branch: x + gate * layer(LN-mod(x))
-    cfg = synth.make_config(args.workload.replace("-branch", ""))
-    sd = synth.to_state_dict(cfg["master"], cfg["weights"])
-    cfg["master"] = None
-    module = synth.build_module({k: v.to(dev) for k, v in sd.items()}, cfg["weights"], dev)
-    x = cfg["x"].to(dev)
+    stack = args.workload == "cfg4"              # 48 independent fp8 layers, x <- x + layer(LayerNorm(x)), 32768 tokens
+    if stack:
+        # weights and tokens are drawn on the device (11.5 GB of fp8 weights; the CPU generator would take minutes)
+        modules = []
+        for layer in range(args.layers):
+            master, _ = synth.make_weights(layer, device=dev)
+            modules.append(synth.build_module(synth.to_state_dict(master, "fp8"), "fp8", dev))
+            del master
+        g = torch.Generator(device=dev).manual_seed(1000)
+        x = torch.randn((2, 16384, synth.DIM), generator=g, device=dev).to(torch.bfloat16)
+        cfg, sd, module = dict(weights="fp8", x=None), None, modules[0]
+        args.no_cpu_baseline = True              # the CPU baseline is quoted on the headline workload
+    else:
+        cfg = synth.make_config(args.workload.replace("-branch", ""))
+        sd = synth.to_state_dict(cfg["master"], cfg["weights"])
+        cfg["master"] = None
+        module = synth.build_module({k: v.to(dev) for k, v in sd.items()}, cfg["weights"], dev)
+        modules = [module]
+        x = cfg["x"].to(dev)
     B, S, D = x.shape
     T = B * S
     H, Hs, E = synth.H_ROUTED, synth.H_SHARED, synth.NUM_EXPERTS
@@ -185,7 +200,18 @@ def main():
         torch.cuda.synchronize()
         del src_cal, dst_cal
 
-    if branch:
+    n_layers = len(modules)
+    if stack:
+        zero = torch.zeros((B, 1, D), dtype=torch.bfloat16, device=dev)
+        one = torch.ones((B, 1, D), dtype=torch.bfloat16, device=dev)
+
+        def forward(stage_events=None):
+            h = x
+            for i, m in enumerate(modules):
+                ev = None if stage_events is None else stage_events[i * (len(STAGE_NAMES) + 1):(i + 1) * (len(STAGE_NAMES) + 1)]
+                h = m.forward_branch(h, zero, zero, one, stage_events=ev)
+            return h
+    elif branch:
         g = torch.Generator().manual_seed(1)
         shift, scale, gate_mlp = ((torch.randn((B, 1, D), generator=g) * 0.3).to(torch.bfloat16).to(dev) for _ in range(3))
         forward = lambda **kw: module.forward_branch(x, shift, scale, gate_mlp, **kw)
@@ -198,7 +224,7 @@ def main():
             y = forward()
         torch.cuda.synchronize()
         # K timed steps; every step also records the per-stage events on the launch stream
-        ev_sets = [hip.create(len(STAGE_NAMES) + 1) for _ in range(args.steps)]
+        ev_sets = [hip.create((len(STAGE_NAMES) + 1) * n_layers) for _ in range(args.steps)]
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for k in range(args.steps):
@@ -212,17 +238,19 @@ def main():
     sec = (t1 - t0) / args.steps
     stage_ms = {n: 0.0 for n in STAGE_NAMES}
     for evs in ev_sets:
-        for i, n in enumerate(STAGE_NAMES):
-            stage_ms[n] += hip.elapsed_ms(evs[i], evs[i + 1])
+        for l in range(n_layers):
+            base = l * (len(STAGE_NAMES) + 1)
+            for i, n in enumerate(STAGE_NAMES):
+                stage_ms[n] += hip.elapsed_ms(evs[base + i], evs[base + i + 1])
     for n in stage_ms:
-        stage_ms[n] /= args.steps
+        stage_ms[n] /= args.steps * n_layers      # per layer
     for evs in ev_sets:
         hip.destroy(evs)
 
     fp8 = cfg["weights"] == "fp8"
     peak = PEAK_FP8_TFLOPS if fp8 else PEAK_BF16_TFLOPS
-    tokens_per_s = T / sec
-    tflops = tokens_per_s * fl["total"] / 1e12
+    tokens_per_s = T / sec                        # through the whole stack when there is more than one layer
+    tflops = tokens_per_s * n_layers * fl["total"] / 1e12
     gemm1_tflops = T * fl["gate_up"] / (stage_ms["gemm_gate_up"] * 1e-3) / 1e12
     gemm2_tflops = T * fl["down"] / (stage_ms["gemm_down"] * 1e-3) / 1e12
     eb = 1 if fp8 else 2
@@ -253,13 +281,16 @@ def main():
                                      "with exact logit ties on every 64th token",
                          "cfg5-4096": "cfg5: 4096 tokens, fp8 weights, skewed routing (about 70% of tokens pick expert "
                                       "0) with exact logit ties on every 64th token",
+                         "cfg4": f"cfg4: {n_layers} independent fp8 layers applied in sequence as x <- x + layer(LayerNorm(x)) "
+                                 "(one enqueue per layer through forward_branch), 2x16384 = 32768 tokens; value counts "
+                                 "tokens through the whole stack; stage_ms and roofline are per layer",
                          "cfg3-branch": "cfg3 tokens and weights through the block's whole feed-forward branch: x + gate_mlp * "
                                         "layer(LayerNorm(x) * (1 + scale_mlp) + shift_mlp), one enqueue (stage 'gate' "
                                         "includes the LayerNorm kernel, stage 'combine' the gated residual)",
                          "cfg3": "cfg3 (headline): 2x4096 = 8192 tokens x 2560, scaled fp8 e4m3fn weights "
                                  "(scale_weight = amax/448, scale_input = 1.0), bf16 gate, x ~ N(0,1) with 1% "
                                  "outlier channels x20, 4 routed experts (hidden 6912) top-2 + shared expert (hidden 3584)"}[args.workload],
-            "tokens": T, "dim": D, "hidden_routed": H, "hidden_shared": Hs, "experts": E, "top_k": 2,
+            "tokens": T, "layers": n_layers, "dim": D, "hidden_routed": H, "hidden_shared": Hs, "experts": E, "top_k": 2,
         },
         "tflops": tflops,
         "pct_of_mfma_peak": 100.0 * tflops / peak,

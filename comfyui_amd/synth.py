@@ -35,22 +35,23 @@ def quantize_per_tensor(w_fp32):
     return (w_fp32 / s).to(FP8), s
 
 
-def make_weights(seed=0, dim=DIM, hidden_arg=None, num_experts=NUM_EXPERTS, sigma=0.02, generator=None):
-    """fp32 master weights as a flat dict keyed like the module's state dict."""
+def make_weights(seed=0, dim=DIM, hidden_arg=None, num_experts=NUM_EXPERTS, sigma=0.02, generator=None, device=None):
+    """fp32 master weights as a flat dict keyed like the module's state dict. `device` draws them there (its own
+    generator stream: not the same numbers as on the CPU, the same distribution)."""
     hidden_arg = hidden_arg if hidden_arg is not None else 4 * dim
-    g = generator if generator is not None else torch.Generator().manual_seed(seed)
+    g = generator if generator is not None else torch.Generator(device=device if device is not None else "cpu").manual_seed(seed)
     hs, hr = swiglu_hidden(hidden_arg // 2), swiglu_hidden(hidden_arg)
     sd = {}
 
     def ffn(prefix, h):
-        sd[prefix + "w1.weight"] = torch.randn((h, dim), generator=g) * sigma
-        sd[prefix + "w2.weight"] = torch.randn((dim, h), generator=g) * sigma
-        sd[prefix + "w3.weight"] = torch.randn((h, dim), generator=g) * sigma
+        sd[prefix + "w1.weight"] = torch.randn((h, dim), generator=g, device=device) * sigma
+        sd[prefix + "w2.weight"] = torch.randn((dim, h), generator=g, device=device) * sigma
+        sd[prefix + "w3.weight"] = torch.randn((h, dim), generator=g, device=device) * sigma
 
     ffn("shared_experts.", hs)
     for e in range(num_experts):
         ffn(f"experts.{e}.", hr)
-    sd["gate.weight"] = torch.randn((num_experts, dim), generator=g) / math.sqrt(dim)
+    sd["gate.weight"] = torch.randn((num_experts, dim), generator=g, device=device) / math.sqrt(dim)
     return sd, g
 
 
@@ -67,7 +68,7 @@ def to_state_dict(master, weights="fp8", scale_input=True):
         out[k] = w8
         out[k.replace(".weight", ".scale_weight")] = s
         if scale_input:
-            out[k.replace(".weight", ".scale_input")] = torch.ones((), dtype=torch.float32)
+            out[k.replace(".weight", ".scale_input")] = torch.ones((), dtype=torch.float32, device=v.device)
     return out
 
 
