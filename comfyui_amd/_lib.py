@@ -93,6 +93,7 @@ SIGNATURES = {
                                        c_void_p]),
     "hdmoe_combine_gated_residual": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
                                              c_int, c_void_p, c_void_p]),
+    "hdmoe_gated_residual_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p]),
     "hdmoe_combine": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p]),
     "hdmoe_layer_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int, c_int]),
     "hdmoe_moe_ffn": (c_int, [ctypes.POINTER(LayerArgs), c_void_p]),

@@ -196,6 +196,26 @@ __global__ __launch_bounds__(THREADS) void combine_kernel(const uint4* __restric
   }
 }
 
+// out[t] = bf16( bf16(gate[b] * y[t]) + residual[t] ), b = t / tokens_per_batch: the gate and residual behind a dense
+// feed-forward (/root/reference/comfy/ldm/hidream/model.py:519-523, text stream).
+__global__ __launch_bounds__(THREADS) void gated_residual_kernel(const uint4* __restrict__ y, const uint4* __restrict__ gate,
+                                                                 const uint4* __restrict__ residual, int T, int row16,
+                                                                 int tokens_per_batch, uint4* __restrict__ out) {
+  const int lane = threadIdx.x & 63;
+  const int wave = blockIdx.x * WAVES + (threadIdx.x >> 6);
+  const int nwaves = gridDim.x * WAVES;
+  auto gr = [](uint32_t g, uint32_t v, uint32_t r) {
+    return pack_bf16(round_bf16(bf16_lo(g) * bf16_lo(v)) + bf16_lo(r), round_bf16(bf16_hi(g) * bf16_hi(v)) + bf16_hi(r));
+  };
+  for (int t = wave; t < T; t += nwaves) {
+    const long brow = (long)(t / tokens_per_batch) * row16;
+    for (int u = lane; u < row16; u += 64) {
+      const uint4 v = y[(long)t * row16 + u], g = gate[brow + u], r = residual[(long)t * row16 + u];
+      out[(long)t * row16 + u] = make_uint4(gr(g.x, v.x, r.x), gr(g.y, v.y, r.y), gr(g.z, v.z, r.z), gr(g.w, v.w, r.w));
+    }
+  }
+}
+
 // out = bf16( bf16(src) * bf16(scale) ): the `weight * scale_weight` / `input * scale_weight`
 // products of the scaled-fp8 Linear without fp8 matmul (/root/reference/comfy/ops.py:407-410),
 // whose operands have already been cast to the compute dtype.
@@ -357,6 +377,21 @@ extern "C" int hdmoe_combine_gated_residual(const void* y_sorted_bf16, const int
   return hdmoe_launch_combine(y_sorted_bf16, inv_perm, topk_weight_bf16, shared_bf16, gate_bf16, residual_bf16,
                               tokens_per_batch, T, D, out_bf16, static_cast<hipStream_t>(stream),
                               "hdmoe_combine_gated_residual");
+}
+
+extern "C" int hdmoe_gated_residual_bf16(const void* y_bf16, const void* gate_bf16, const void* residual_bf16,
+                                         int tokens_per_batch, int T, int D, void* out_bf16, hdmoe_stream_t stream) {
+  HDMOE_REQUIRE_PTR(y_bf16);
+  HDMOE_REQUIRE_PTR(gate_bf16);
+  HDMOE_REQUIRE_PTR(residual_bf16);
+  HDMOE_REQUIRE_PTR(out_bf16);
+  if (T < 0 || D <= 0 || D % 8 != 0 || tokens_per_batch <= 0)
+    return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_gated_residual_bf16: T=%d D=%d tokens_per_batch=%d", T, D, tokens_per_batch);
+  if (T == 0) return HDMOE_OK;
+  hipLaunchKernelGGL(gated_residual_kernel, dim3(row_blocks(T)), dim3(THREADS), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const uint4*>(y_bf16), static_cast<const uint4*>(gate_bf16),
+                     static_cast<const uint4*>(residual_bf16), T, D / 8, tokens_per_batch, static_cast<uint4*>(out_bf16));
+  return hdmoe_check_launch("hdmoe_gated_residual_bf16");
 }
 
 extern "C" int hdmoe_scale_to_bf16(int src_dtype, const void* src, int64_t n, const float* scale_dev, void* out_bf16,

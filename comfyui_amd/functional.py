@@ -247,6 +247,20 @@ def combine_gated_residual(y_sorted, inv_perm, topk_weight, shared, gate, residu
     return out
 
 
+def gated_residual(y2d, gate, residual2d, tokens_per_batch):
+    """gate * y + residual behind a dense feed-forward (comfy/ldm/hidream/model.py:519-523)."""
+    _need_hip(y2d, "gated_residual y", BF16)
+    _need_hip(residual2d, "gated_residual residual", BF16)
+    T, D = y2d.shape
+    gate = _per_batch(gate, "gated_residual gate", D, y2d.device)
+    if tokens_per_batch <= 0 or T != gate.shape[0] * tokens_per_batch or tuple(residual2d.shape) != (T, D):
+        raise ValueError(f"gated_residual: T={T}, batch={gate.shape[0]}, tokens_per_batch={tokens_per_batch}")
+    out = torch.empty_like(y2d)
+    check(lib.hdmoe_gated_residual_bf16(ptr(y2d), ptr(gate), ptr(residual2d), tokens_per_batch, T, D, ptr(out),
+                                        _stream(y2d)))
+    return out
+
+
 def make_ffn_weights(w1, w2, w3, scales=None):
     """Fill an hdmoe_ffn_weights. scales: dict with optional fp32 scalar tensors
     scale_w1/2/3 and scale_in1/2/3 (fp8 only)."""

@@ -126,6 +126,20 @@ class FeedForwardSwiGLU(nn.Module):
         # per-Linear composition (also the place where a CPU tensor is refused)
         return self.w2(HF.silu_mul(self.w1(x), self.w3(x)))
 
+    def forward_branch(self, x, shift, scale, gate, eps=1e-6):
+        """The whole feed-forward branch of a block around a dense feed-forward (the text stream's `ff_t`, or `ff_i`
+        of a block without routed experts; comfy/ldm/hidream/model.py:518-523, 402-403):
+            x + gate * self(LayerNorm(x, eps, no affine) * (1 + scale) + shift)
+        x [B,S,dim]; shift, scale, gate [B,1,dim] in bf16. Not a method of the reference class."""
+        if x.dtype != BF16 or not x.is_cuda or x.dim() != 3:
+            raise RuntimeError(f"FeedForwardSwiGLU.forward_branch: expected a [B,S,dim] bfloat16 HIP tensor, got "
+                               f"{tuple(x.shape)} {x.dtype} on {x.device}; comfyui_amd has no CPU path")
+        B, S, D = x.shape
+        x2 = x.reshape(-1, D).contiguous()
+        n = HF.ln_modulate(x2, scale.reshape(B, D).contiguous(), shift.reshape(B, D).contiguous(), S, eps)
+        y = self.forward(n.view(B, S, D)).reshape(-1, D)
+        return HF.gated_residual(y, gate.reshape(B, D).contiguous(), x2, S).view(B, S, D)
+
 
 class MoEGate(nn.Module):
     def __init__(self, embed_dim, num_routed_experts=4, num_activated_experts=2, aux_loss_alpha=0.01,

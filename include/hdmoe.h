@@ -33,7 +33,7 @@
 extern "C" {
 #endif
 
-#define HDMOE_VERSION 103
+#define HDMOE_VERSION 104
 
 #define HDMOE_OK 0
 #define HDMOE_E_NULL (-1)      /* required pointer is NULL */
@@ -190,6 +190,11 @@ int hdmoe_combine_gated_residual(const void* y_sorted_bf16, const int32_t* inv_p
                                  const void* topk_weight_bf16, const void* shared_bf16,
                                  const void* gate_bf16, const void* residual_bf16, int tokens_per_batch,
                                  int T, int D, void* out_bf16, hdmoe_stream_t stream);
+
+/* The same gate and residual behind a dense feed-forward (text stream, comfy/ldm/hidream/model.py:519-523):
+ * out[t] = bf16( bf16(gate[t / tokens_per_batch] * y[t]) + residual[t] ). */
+int hdmoe_gated_residual_bf16(const void* y_bf16, const void* gate_bf16, const void* residual_bf16,
+                              int tokens_per_batch, int T, int D, void* out_bf16, hdmoe_stream_t stream);
 
 /* ---- whole layer -------------------------------------------------------------- */
 

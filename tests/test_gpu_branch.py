@@ -144,3 +144,31 @@ def test_branch_at_headline_size_properties(dev):
     err = (n.float() - n_torch.float()).abs()
     bound = torch.maximum((ln.float() * (1 + scale).float()).abs(), n_torch.float().abs()) * (3 * 2.0 ** -7)
     assert bool((err <= bound + 1e-30).all())
+
+
+@pytest.mark.parametrize("weights", ["fp8", "bf16"])
+def test_dense_feed_forward_branch(dev, weights):
+    """Text-stream branch: ln_modulate -> dense SwiGLU feed-forward -> gate and residual (model.py:518-523)."""
+    from comfyui_amd import functional as HF
+    dim, B, S = 512, 2, 130
+    sd, _ = small_layer(seed=13, dim=dim, tokens=B * S, weights=weights, batch=B)
+    x, shift, scale, gate = make(B, S, dim, seed=14)
+    gate = (gate * 64).to(BF16)
+    m = synth.build_module({k: v.to(dev) for k, v in sd.items()}, weights, dev, dim=dim)
+    ff = m.shared_experts
+    out = ff.forward_branch(x.to(dev), shift.to(dev), scale.to(dev), gate.to(dev)).cpu()
+    # the gated residual kernel alone: bit-exact against the restatement and torch's bf16 expression
+    g = torch.Generator().manual_seed(3)
+    y = torch.randn((B * S, dim), generator=g).to(BF16)
+    got = HF.gated_residual(y.to(dev), gate.to(dev), x.reshape(-1, dim).to(dev), S).cpu()
+    assert torch.equal(bits(got), bits(O.gated_residual_c(y, gate.reshape(B, dim), x.reshape(-1, dim), S)))
+    assert torch.equal(bits(got), bits((gate * y.view(B, S, dim) + x).reshape(-1, dim)))
+    # the branch against the oracle's pieces
+    params = oracle_params(sd, 4)
+    mode = "fp8mm" if weights == "fp8" else "plain"
+    n = O.ln_modulate_c(x.reshape(-1, dim), shift.reshape(B, dim), scale.reshape(B, dim), S).view(B, S, dim)
+    ref = O.gated_residual_torch(O.ffn_swiglu(n, params["shared"], mode), gate, x)
+    d_all = O.error_metrics(out, ref)
+    d_ff = O.error_metrics(out.float() - x.float(), ref.float() - x.float())
+    assert d_all["rel_rms"] <= TOL_RMS_SAME_DATAFLOW[weights] and d_ff["rel_rms"] <= TOL[weights], (d_all, d_ff)
+    assert torch.equal(ff.forward_branch(x.to(dev), shift.to(dev), scale.to(dev), torch.zeros_like(gate).to(dev)).cpu(), x)
