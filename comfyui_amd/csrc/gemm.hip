@@ -140,9 +140,12 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
       L -= tiles;
     }
     if (g >= args.G) return d;
-    const int band = L / (GROUP_M * ntiles);
+    // bands of GROUP_M m-tiles; a short remainder joins the last band, so that the cheap partial m-tile at the
+    // end of a segment is interleaved with full ones instead of forming a run of its own
+    const int nbands = max(1, (mtiles + GROUP_M / 2) / GROUP_M);
+    const int band = min(L / (GROUP_M * ntiles), nbands - 1);
     const int first_m = band * GROUP_M;
-    const int gm = min(mtiles - first_m, GROUP_M);
+    const int gm = band == nbands - 1 ? mtiles - first_m : GROUP_M;
     const int within = L - band * (GROUP_M * ntiles);
     d.g = g;
     d.row0 = rb + (first_m + within % gm) * BM;
@@ -210,7 +213,10 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
   const int b_base = TILE_BYTES + (wq * 32 + fr_row) * BK;   // weight operand, + ft*128*BK
 
   v16f acc[2][4];
-  auto compute = [&](int stage) {
+  // n_tt: how many of this wave's four 32-token blocks hold rows of the tile (4 except in the last, partial
+  // m-tile of a segment); the others are neither read from LDS nor multiplied.
+  auto compute = [&](int stage, auto full_c, int n_tt) {
+    constexpr bool FULL = decltype(full_c)::value;
     const uint8_t* st = smem + stage * STAGE_BYTES;
     if constexpr (FP8) {
 #pragma unroll
@@ -220,11 +226,13 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
         v8i fa[4], fb[2];
 #pragma unroll
         for (int tt = 0; tt < 4; ++tt) {
+          if (!FULL && tt >= n_tt) continue;
           const uint8_t* p = st + a_base + tt * 32 * BK;
           const v4i lo = *reinterpret_cast<const v4i*>(p + c0);
           const v4i hi = *reinterpret_cast<const v4i*>(p + c1);
           fa[tt] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
         }
+        if (!FULL && n_tt == 0) continue;
 #pragma unroll
         for (int ft = 0; ft < 2; ++ft) {
           const uint8_t* p = st + b_base + ft * 128 * BK;
@@ -235,8 +243,10 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
 #pragma unroll
         for (int ft = 0; ft < 2; ++ft)
 #pragma unroll
-          for (int tt = 0; tt < 4; ++tt)
+          for (int tt = 0; tt < 4; ++tt) {
+            if (!FULL && tt >= n_tt) continue;
             acc[ft][tt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[ft], fa[tt], acc[ft][tt], 0, 0, 0, 0, 0, 0);
+          }
       }
     } else {
 #pragma unroll
@@ -244,16 +254,21 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
         const int c0 = ((ks * 2 + fr_grp) ^ fr_swz) * 16;
         v8bf fa[4], fb[2];
 #pragma unroll
-        for (int tt = 0; tt < 4; ++tt)
+        for (int tt = 0; tt < 4; ++tt) {
+          if (!FULL && tt >= n_tt) continue;
           fa[tt] = *reinterpret_cast<const v8bf*>(st + a_base + tt * 32 * BK + c0);
+        }
+        if (!FULL && n_tt == 0) continue;
 #pragma unroll
         for (int ft = 0; ft < 2; ++ft)
           fb[ft] = *reinterpret_cast<const v8bf*>(st + b_base + ft * 128 * BK + c0);
 #pragma unroll
         for (int ft = 0; ft < 2; ++ft)
 #pragma unroll
-          for (int tt = 0; tt < 4; ++tt)
+          for (int tt = 0; tt < 4; ++tt) {
+            if (!FULL && tt >= n_tt) continue;
             acc[ft][tt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[ft], fa[tt], acc[ft][tt], 0, 0, 0);
+          }
       }
     }
   };
@@ -451,18 +466,23 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
       for (int b2 = 0; b2 < 4; ++b2)
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[a2][b2][r] = 0.0f;
-    for (int kt = 0; kt < KT; kt += 2) {
-      __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's part of the stage has landed
-      __syncthreads();                      // everyone's part has; everyone is done reading the other stage
-      if (kt + 1 < KT) issue_loads(1, kt + 1);
-      compute(0);
-      if (kt + 1 < KT) {
-        __builtin_amdgcn_s_waitcnt(0x0f70);
-        __syncthreads();
-        if (kt + 2 < KT) issue_loads(0, kt + 2);
-        compute(1);
+    auto k_loop = [&](auto full_c, int n_tt) {
+      for (int kt = 0; kt < KT; kt += 2) {
+        __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's part of the stage has landed
+        __syncthreads();                      // everyone's part has; everyone is done reading the other stage
+        if (kt + 1 < KT) issue_loads(1, kt + 1);
+        compute(0, full_c, n_tt);
+        if (kt + 1 < KT) {
+          __builtin_amdgcn_s_waitcnt(0x0f70);
+          __syncthreads();
+          if (kt + 2 < KT) issue_loads(0, kt + 2);
+          compute(1, full_c, n_tt);
+        }
       }
-    }
+    };
+    const int my_rows = __builtin_amdgcn_readfirstlane(cur.rows_here) - wt * 128;  // rows of the tile in this wave's half
+    if (my_rows >= 97) k_loop(std::true_type{}, 4);
+    else k_loop(std::false_type{}, my_rows <= 0 ? 0 : (my_rows + 31) / 32);
     const Tile nxt = decode(i + 1);
     // Every wave is done reading both stages: stage 0 can take the next tile's first K step, stage 1 the
     // staged outputs of this one (it is not loaded into again before the barrier of that K step).
