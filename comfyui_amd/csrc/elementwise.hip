@@ -5,44 +5,21 @@
 // one row.
 #include "common.h"
 #include "numfmt.h"
+#include "quant.h"
 
 namespace {
 
 constexpr int THREADS = 256;
 constexpr int WAVES = THREADS / 64;
 
-struct ScalePtrs {
-  const float* p[HDMOE_MAX_EXPERTS];
-};
+typedef HdmoeScalePtrs ScalePtrs;
 
 __device__ __forceinline__ float bf16_lo(uint32_t u) { return __uint_as_float(u << 16); }
 __device__ __forceinline__ float bf16_hi(uint32_t u) { return __uint_as_float(u & 0xffff0000u); }
 __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) { return hdmoe_dev_pack_bf16(lo, hi); }
 __device__ __forceinline__ float round_bf16(float f) { return hdmoe_dev_round_bf16(f); }
-
-// fp8_linear's activation cast (/root/reference/comfy/ops.py:337-343).
-// inv < 0 selects the scale_input-is-None rule (clamp to +-448, scale 1).
-__device__ __forceinline__ float quant_pre(float v, float inv) {
-  if (inv < 0.0f) return v < -448.0f ? -448.0f : (v > 448.0f ? 448.0f : v);
-  return round_bf16(v * inv);  // bf16 tensor times bf16 scalar, rounded to bf16
-}
-
-__device__ __forceinline__ uint32_t quant2x(uint32_t u, float inv) {
-  return hdmoe_dev_pack_e4m3fn(quant_pre(bf16_lo(u), inv), quant_pre(bf16_hi(u), inv));
-}
-
-__device__ __forceinline__ uint2 quant8(const uint4& v, float inv) {
-  uint2 o;
-  o.x = quant2x(v.x, inv) | (quant2x(v.y, inv) << 16);
-  o.y = quant2x(v.z, inv) | (quant2x(v.w, inv) << 16);
-  return o;
-}
-
-// (1.0 / scale_input).to(bfloat16) as fp32; NULL pointer -> clamp rule marker
-__device__ __forceinline__ float inv_scale(const float* s) {
-  if (s == nullptr) return -1.0f;
-  return round_bf16(__fdiv_rn(1.0f, *s));
-}
+__device__ __forceinline__ uint2 quant8(const uint4& v, float inv) { return hdmoe_q_8(v, inv); }
+__device__ __forceinline__ float inv_scale(const float* s) { return hdmoe_q_inv_scale(s); }
 
 __global__ __launch_bounds__(THREADS) void quant_rows_kernel(const uint4* __restrict__ x, long rows, int row16,
                                                              const float* scale_in, uint2* __restrict__ out) {

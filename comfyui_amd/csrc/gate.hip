@@ -15,6 +15,7 @@
 // bandwidth bound (the E x D weight is 20 KiB and stays in registers / L2).
 #include "common.h"
 #include "numfmt.h"
+#include "quant.h"
 
 #pragma clang fp contract(off)
 
@@ -59,7 +60,7 @@ __device__ __forceinline__ float dot8(const uint4& a, const uint4& b, float acc)
 
 template <int E>
 __device__ __forceinline__ void finish_token(float (&logit)[E], int lane, int t, int32_t* idx,
-                                             uint16_t* wout) {
+                                             uint16_t* wout, int& first, int& second) {
 #pragma unroll
   for (int e = 0; e < E; ++e) {
     float v = logit[e];
@@ -93,6 +94,8 @@ __device__ __forceinline__ void finish_token(float (&logit)[E], int lane, int t,
     if (e == i0) continue;
     if (i1 < 0 || score[e] > s1) { s1 = score[e]; i1 = e; }
   }
+  first = i0;
+  second = i1;
   if (lane == 0) {
     reinterpret_cast<int2*>(idx)[t] = make_int2(i0, i1);
     reinterpret_cast<uint32_t*>(wout)[t] =
@@ -101,10 +104,20 @@ __device__ __forceinline__ void finish_token(float (&logit)[E], int lane, int t,
 }
 
 // D == NCHUNK * 512: the lane's Wg slice lives in registers.
-template <int E, int NCHUNK>
+// Optional second output of both kernels (QUANT): the token's fp8 rows for the expert GEMMs, cast while the row
+// is at hand. Row 2t+s of xq_routed is x[t] cast with the scale_input of the expert in slot s, row t of xq_shared
+// the cast for the shared expert; the GEMM reads them through the dispatch permutation.
+struct GateQuant {
+  HdmoeScalePtrs scale_in;    // per expert, NULL = clamp rule
+  const float* shared_scale;
+  uint2* xq_routed;           // [2T, D] e4m3fn
+  uint2* xq_shared;           // [T, D] e4m3fn or NULL
+};
+
+template <int E, int NCHUNK, bool QUANT>
 __global__ __launch_bounds__(WAVES_PER_BLOCK * 64) void gate_top2_reg_kernel(
     const uint4* __restrict__ x, const uint4* __restrict__ wg, int T, int32_t* __restrict__ idx,
-    uint16_t* __restrict__ wout) {
+    uint16_t* __restrict__ wout, GateQuant q) {
   const int lane = threadIdx.x & 63;
   const int wave = blockIdx.x * WAVES_PER_BLOCK + (threadIdx.x >> 6);
   const int nwaves = gridDim.x * WAVES_PER_BLOCK;
@@ -139,17 +152,32 @@ __global__ __launch_bounds__(WAVES_PER_BLOCK * 64) void gate_top2_reg_kernel(
       }
       logit[e] = acc;
     }
-    finish_token<E>(logit, lane, t, idx, wout);
+    int i0, i1;
+    finish_token<E>(logit, lane, t, idx, wout, i0, i1);
+    if constexpr (QUANT) {
+      const float inv0 = hdmoe_q_inv_scale(q.scale_in.p[i0]), inv1 = hdmoe_q_inv_scale(q.scale_in.p[i1]);
+      const float invs = hdmoe_q_inv_scale(q.shared_scale);
+      uint2* r0 = q.xq_routed + (size_t)(2 * t) * ROW16;
+      const bool same01 = inv0 == inv1, same0s = inv0 == invs;  // equal scales: cast once, store again
+#pragma unroll
+      for (int c = 0; c < NCHUNK; ++c) {
+        const uint2 v0 = hdmoe_q_8(cur[c], inv0);
+        r0[c * 64 + lane] = v0;
+        r0[ROW16 + c * 64 + lane] = same01 ? v0 : hdmoe_q_8(cur[c], inv1);
+        if (q.xq_shared != nullptr)
+          q.xq_shared[(size_t)t * ROW16 + c * 64 + lane] = same0s ? v0 : hdmoe_q_8(cur[c], invs);
+      }
+    }
 #pragma unroll
     for (int c = 0; c < NCHUNK; ++c) cur[c] = nxt[c];
   }
 }
 
 // Any D that is a multiple of 8: Wg is re-read through the cache hierarchy.
-template <int E>
+template <int E, bool QUANT>
 __global__ __launch_bounds__(WAVES_PER_BLOCK * 64) void gate_top2_generic_kernel(
     const uint4* __restrict__ x, const uint4* __restrict__ wg, int T, int D, int32_t* __restrict__ idx,
-    uint16_t* __restrict__ wout) {
+    uint16_t* __restrict__ wout, GateQuant q) {
   const int lane = threadIdx.x & 63;
   const int wave = blockIdx.x * WAVES_PER_BLOCK + (threadIdx.x >> 6);
   const int nwaves = gridDim.x * WAVES_PER_BLOCK;
@@ -163,12 +191,24 @@ __global__ __launch_bounds__(WAVES_PER_BLOCK * 64) void gate_top2_generic_kernel
 #pragma unroll
       for (int e = 0; e < E; ++e) logit[e] = dot8(xv, wg[(size_t)e * row16 + u], logit[e]);
     }
-    finish_token<E>(logit, lane, t, idx, wout);
+    int i0, i1;
+    finish_token<E>(logit, lane, t, idx, wout, i0, i1);
+    if constexpr (QUANT) {
+      const float inv0 = hdmoe_q_inv_scale(q.scale_in.p[i0]), inv1 = hdmoe_q_inv_scale(q.scale_in.p[i1]);
+      const float invs = hdmoe_q_inv_scale(q.shared_scale);
+      for (int u = lane; u < row16; u += 64) {
+        const uint4 xv = x[(size_t)t * row16 + u];
+        q.xq_routed[(size_t)(2 * t) * row16 + u] = hdmoe_q_8(xv, inv0);
+        q.xq_routed[(size_t)(2 * t + 1) * row16 + u] = hdmoe_q_8(xv, inv1);
+        if (q.xq_shared != nullptr) q.xq_shared[(size_t)t * row16 + u] = hdmoe_q_8(xv, invs);
+      }
+    }
   }
 }
 
 template <int E>
-int launch_gate(const void* x, const void* wg, int T, int D, int32_t* idx, void* w, hipStream_t s) {
+int launch_gate(const void* x, const void* wg, int T, int D, int32_t* idx, void* w, const GateQuant* quant,
+                hipStream_t s, const char* what) {
   // about 4 tokens per wave amortise the register-resident weight slice and still give 8 waves per CU at T = 8192
   int blocks = (T + WAVES_PER_BLOCK * 4 - 1) / (WAVES_PER_BLOCK * 4);
   if (blocks < 1) blocks = 1;
@@ -177,12 +217,31 @@ int launch_gate(const void* x, const void* wg, int T, int D, int32_t* idx, void*
   const uint4* xp = static_cast<const uint4*>(x);
   const uint4* wp = static_cast<const uint4*>(wg);
   uint16_t* wo = static_cast<uint16_t*>(w);
+  GateQuant q;
+  memset(&q, 0, sizeof(q));
+  if (quant) q = *quant;
+  constexpr int ER = E <= 4 ? E : 4;  // the register kernel is only instantiated for up to 4 experts
   if (E <= 4 && D == 2560) {
-    hipLaunchKernelGGL((gate_top2_reg_kernel<(E <= 4 ? E : 4), 5>), grid, block, 0, s, xp, wp, T, idx, wo);
+    if (quant) hipLaunchKernelGGL((gate_top2_reg_kernel<ER, 5, true>), grid, block, 0, s, xp, wp, T, idx, wo, q);
+    else hipLaunchKernelGGL((gate_top2_reg_kernel<ER, 5, false>), grid, block, 0, s, xp, wp, T, idx, wo, q);
   } else {
-    hipLaunchKernelGGL((gate_top2_generic_kernel<E>), grid, block, 0, s, xp, wp, T, D, idx, wo);
+    if (quant) hipLaunchKernelGGL((gate_top2_generic_kernel<E, true>), grid, block, 0, s, xp, wp, T, D, idx, wo, q);
+    else hipLaunchKernelGGL((gate_top2_generic_kernel<E, false>), grid, block, 0, s, xp, wp, T, D, idx, wo, q);
   }
-  return hdmoe_check_launch("hdmoe_gate_top2");
+  return hdmoe_check_launch(what);
+}
+
+int dispatch_gate(const void* x_bf16, const void* gate_w_bf16, int T, int D, int E, int32_t* topk_idx,
+                  void* topk_weight_bf16, const GateQuant* quant, hipStream_t s, const char* what) {
+  switch (E) {
+#define HDMOE_GATE_CASE(n) \
+  case n: return launch_gate<n>(x_bf16, gate_w_bf16, T, D, topk_idx, topk_weight_bf16, quant, s, what);
+    HDMOE_GATE_CASE(2) HDMOE_GATE_CASE(3) HDMOE_GATE_CASE(4) HDMOE_GATE_CASE(5) HDMOE_GATE_CASE(6)
+    HDMOE_GATE_CASE(7) HDMOE_GATE_CASE(8) HDMOE_GATE_CASE(9) HDMOE_GATE_CASE(10) HDMOE_GATE_CASE(11)
+    HDMOE_GATE_CASE(12) HDMOE_GATE_CASE(13) HDMOE_GATE_CASE(14) HDMOE_GATE_CASE(15) HDMOE_GATE_CASE(16)
+#undef HDMOE_GATE_CASE
+    default: return hdmoe_fail(HDMOE_E_SHAPE, "%s: E=%d not in 2..16", what, E);
+  }
 }
 
 // ---- LayerNorm (no affine) + adaLN modulation in front of the feed-forward -----------------------------
@@ -300,15 +359,21 @@ extern "C" int hdmoe_gate_top2(const void* x_bf16, const void* gate_w_bf16, int 
   if (T < 0 || D <= 0 || D % 8 != 0)
     return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_gate_top2: T=%d D=%d (D must be a positive multiple of 8)", T, D);
   if (T == 0) return HDMOE_OK;
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  switch (E) {
-#define HDMOE_GATE_CASE(n) case n: return launch_gate<n>(x_bf16, gate_w_bf16, T, D, topk_idx, topk_weight_bf16, s);
-    HDMOE_GATE_CASE(2) HDMOE_GATE_CASE(3) HDMOE_GATE_CASE(4) HDMOE_GATE_CASE(5) HDMOE_GATE_CASE(6)
-    HDMOE_GATE_CASE(7) HDMOE_GATE_CASE(8) HDMOE_GATE_CASE(9) HDMOE_GATE_CASE(10) HDMOE_GATE_CASE(11)
-    HDMOE_GATE_CASE(12) HDMOE_GATE_CASE(13) HDMOE_GATE_CASE(14) HDMOE_GATE_CASE(15) HDMOE_GATE_CASE(16)
-#undef HDMOE_GATE_CASE
-    default: return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_gate_top2: E=%d not in 2..16", E);
-  }
+  return dispatch_gate(x_bf16, gate_w_bf16, T, D, E, topk_idx, topk_weight_bf16, nullptr,
+                       static_cast<hipStream_t>(stream), "hdmoe_gate_top2");
+}
+
+// The gate of the one-call layer with fp8 experts: routing plus the token's three fp8 rows in one pass over x.
+int hdmoe_launch_gate_quant(const void* x_bf16, const void* gate_w_bf16, int T, int D, int E, int32_t* topk_idx,
+                            void* topk_weight_bf16, const float* const* scale_input, const float* shared_scale,
+                            void* xq_routed, void* xq_shared, hipStream_t s, const char* what) {
+  GateQuant q;
+  memset(&q, 0, sizeof(q));
+  for (int e = 0; e < E && e < HDMOE_MAX_EXPERTS; ++e) q.scale_in.p[e] = scale_input[e];
+  q.shared_scale = shared_scale;
+  q.xq_routed = static_cast<uint2*>(xq_routed);
+  q.xq_shared = static_cast<uint2*>(xq_shared);
+  return dispatch_gate(x_bf16, gate_w_bf16, T, D, E, topk_idx, topk_weight_bf16, &q, s, what);
 }
 
 extern "C" int hdmoe_ln_modulate_bf16(const void* x_bf16, const void* scale_bf16, const void* shift_bf16, int T, int D,

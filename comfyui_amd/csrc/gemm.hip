@@ -58,6 +58,8 @@ enum Mode { FP8_SWIGLU = 0, FP8_PLAIN = 1, BF16_SWIGLU = 2, BF16_PLAIN = 3, BF16
 
 struct GemmGroup {
   const uint8_t* a;     // activations; row indices below are relative to this base
+  const int32_t* gather;  // NULL: row r of the group is row r of a; else it is row gather[r] of a (a_rows rows)
+  int a_rows;
   const uint8_t* b0;    // plain: W [N,K]; swiglu: w1 [H,K]
   const uint8_t* b1;    // swiglu: w3 [H,K]
   const float* sb0;     // scale_weight of b0 (fp8)
@@ -173,16 +175,32 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
   __amdgpu_buffer_rsrc_t src_a = make_rsrc(nullptr, 0), src_b0 = src_a, src_b1 = src_a;
   int src_voff[4] = {0, 0, 0, 0};
   int src_voff_b[2] = {0, 0};
-  auto set_src = [&](const Tile& d) {
+  // Row indices of a gathered token operand: loaded one tile ahead (load_gather), consumed by set_src.
+  auto load_gather = [&](const Tile& d, int (&gi)[4]) {
     const GemmGroup& gg = args.g[d.g];
-    src_a = make_rsrc(gg.a + (size_t)d.row0 * d.kbytes, (uint32_t)d.rows_here * (uint32_t)d.kbytes);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int r = j * 64 + ld_row;
+      gi[j] = (gg.gather != nullptr && r < d.rows_here) ? gg.gather[d.row0 + r] : -1;
+    }
+  };
+  auto set_src = [&](const Tile& d, const int (&gi)[4]) {
+    const GemmGroup& gg = args.g[d.g];
+    if (gg.gather != nullptr) {
+      // rows past the segment end get an offset beyond the buffer and read as zero
+      src_a = make_rsrc(gg.a, (uint32_t)gg.a_rows * (uint32_t)d.kbytes);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) src_voff[j] = gi[j] >= 0 ? gi[j] * d.kbytes + ld_chunk * 16 : (int)0x80000000u;
+    } else {
+      src_a = make_rsrc(gg.a + (size_t)d.row0 * d.kbytes, (uint32_t)d.rows_here * (uint32_t)d.kbytes);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) src_voff[j] = (j * 64 + ld_row) * d.kbytes + ld_chunk * 16;
+    }
     const uint8_t* b_half0 = gg.b0 + (size_t)d.n0 * d.kbytes;
     const uint8_t* b_half1 = SWIGLU ? gg.b1 + (size_t)d.n0 * d.kbytes : gg.b0 + (size_t)(d.n0 + 32) * d.kbytes;
     const uint32_t b_rows = SWIGLU ? BN / 2 : BN - 32;
     src_b0 = make_rsrc(b_half0, b_rows * (uint32_t)d.kbytes);
     src_b1 = make_rsrc(b_half1, b_rows * (uint32_t)d.kbytes);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) src_voff[j] = (j * 64 + ld_row) * d.kbytes + ld_chunk * 16;
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       const int r = j * 64 + ld_row;  // row within the 128-row LDS half
@@ -455,11 +473,15 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
   // current one, so its latency hides behind the stores.
   Tile cur = decode(0);
   if (cur.g < 0) return;
-  set_src(cur);
+  int gi_cur[4], gi_nxt[4] = {-1, -1, -1, -1};
+  load_gather(cur, gi_cur);
+  set_src(cur, gi_cur);
   issue_loads(0, 0);
   for (int i = 0; cur.g >= 0; ++i) {
     const int KT = cur.kbytes / BK;
     load_scales(cur);
+    const Tile nxt = decode(i + 1);
+    if (nxt.g >= 0) load_gather(nxt, gi_nxt);  // lands during the K loop
 #pragma unroll
     for (int a2 = 0; a2 < 2; ++a2)
 #pragma unroll
@@ -483,12 +505,11 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
     const int my_rows = __builtin_amdgcn_readfirstlane(cur.rows_here) - wt * 128;  // rows of the tile in this wave's half
     if (my_rows >= 97) k_loop(std::true_type{}, 4);
     else k_loop(std::false_type{}, my_rows <= 0 ? 0 : (my_rows + 31) / 32);
-    const Tile nxt = decode(i + 1);
     // Every wave is done reading both stages: stage 0 can take the next tile's first K step, stage 1 the
     // staged outputs of this one (it is not loaded into again before the barrier of that K step).
     __syncthreads();
     if (nxt.g >= 0) {
-      set_src(nxt);
+      set_src(nxt, gi_nxt);
       issue_loads(0, 0);
     }
     epilogue(cur);
@@ -529,13 +550,19 @@ int check_dtype(int weight_dtype, const char* what) {
 
 // Shared by hdmoe_grouped_swiglu / hdmoe_grouped_down / hdmoe_linear / hdmoe_moe_ffn.
 // groups: n_dyn experts with device-side segments, optionally one static group (the shared expert).
+// gather_dyn (optional): the routed rows are not materialised in segment order; row r of the segments is row
+// gather_dyn[r] of a_dyn, which holds gather_rows rows.
 int hdmoe_launch_ffn_gemm(bool swiglu, int weight_dtype, const uint8_t* a_dyn, const int32_t* offsets, int rows_dyn,
                           int n_dyn, const hdmoe_ffn_weights* experts, uint8_t* out_dyn, const uint8_t* a_static,
                           int rows_static, const hdmoe_ffn_weights* shared, uint8_t* out_static, int K_dyn, int N_dyn,
-                          int K_static, int N_static, hipStream_t s, const char* what) {
+                          int K_static, int N_static, hipStream_t s, const char* what,
+                          const int32_t* gather_dyn = nullptr, int gather_rows = 0) {
   const int eb = elem_bytes(weight_dtype);
   const bool fp8 = weight_dtype == HDMOE_W_E4M3FN;
   const int feat_per_tile = swiglu ? BN / 2 : BN;
+  if (gather_dyn != nullptr && (unsigned long long)gather_rows * K_dyn * eb >= (1ull << 31))
+    return hdmoe_fail(HDMOE_E_SHAPE, "%s: %d gathered rows of %d bytes exceed the 2 GiB offset range", what, gather_rows,
+                      K_dyn * eb);
   GemmArgs args;
   memset(&args, 0, sizeof(args));
   args.offsets = offsets;
@@ -545,6 +572,8 @@ int hdmoe_launch_ffn_gemm(bool swiglu, int weight_dtype, const uint8_t* a_dyn, c
     GemmGroup& gg = args.g[G];
     const hdmoe_ffn_weights& w = experts[e];
     gg.a = a_dyn;
+    gg.gather = gather_dyn;
+    gg.a_rows = gather_rows;
     gg.out = out_dyn;
     gg.row_begin = -1;
     gg.dyn = e;

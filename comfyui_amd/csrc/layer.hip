@@ -7,11 +7,15 @@
 int hdmoe_launch_ffn_gemm(bool swiglu, int weight_dtype, const uint8_t* a_dyn, const int32_t* offsets, int rows_dyn,
                           int n_dyn, const hdmoe_ffn_weights* experts, uint8_t* out_dyn, const uint8_t* a_static,
                           int rows_static, const hdmoe_ffn_weights* shared, uint8_t* out_static, int K_dyn, int N_dyn,
-                          int K_static, int N_static, hipStream_t s, const char* what);
+                          int K_static, int N_static, hipStream_t s, const char* what,
+                          const int32_t* gather_dyn = nullptr, int gather_rows = 0);
 int hdmoe_check_gemm_shape(const char* what, int weight_dtype, long rows, int K, int N, int feat_per_tile);
 int hdmoe_launch_quant_dispatch(const void* x_bf16, const int32_t* perm, const int32_t* offsets, int T, int D, int E,
                                 const float* const* scale_input, const float* shared_scale, bool with_shared,
                                 void* a_fp8, hipStream_t s, const char* what);
+int hdmoe_launch_gate_quant(const void* x_bf16, const void* gate_w_bf16, int T, int D, int E, int32_t* topk_idx,
+                            void* topk_weight_bf16, const float* const* scale_input, const float* shared_scale,
+                            void* xq_routed, void* xq_shared, hipStream_t s, const char* what);
 int hdmoe_launch_combine(const void* y_sorted_bf16, const int32_t* inv_perm, const void* topk_weight_bf16,
                          const void* shared_bf16, const void* gate_bf16, const void* residual_bf16, int tokens_per_batch,
                          int T, int D, void* out_bf16, hipStream_t s, const char* what);
@@ -118,7 +122,7 @@ extern "C" int hdmoe_moe_ffn(const hdmoe_layer_args* p, hdmoe_stream_t stream) {
   int ev = 0;
   hipError_t ev_err = hipSuccess;
   auto mark = [&]() {
-    if (p->stage_events) {
+    if (p->stage_events && p->stage_events[ev] != nullptr) {
       const hipError_t e = hipEventRecord(static_cast<hipEvent_t>(p->stage_events[ev]), s);
       if (e != hipSuccess && ev_err == hipSuccess) ev_err = e;
     }
@@ -134,7 +138,18 @@ extern "C" int hdmoe_moe_ffn(const hdmoe_layer_args* p, hdmoe_stream_t stream) {
       return rc;
     xin = normed;
   }
-  if (int rc = hdmoe_gate_top2(xin, p->gate_w, T, D, E, idx, tw, stream)) return rc;
+  // fp8 experts: the gate kernel also casts each token to e4m3fn for its two experts (rows 2t, 2t+1 of a_routed,
+  // i.e. in flat slot order) and for the shared expert while it holds the row; the gate/up GEMM then reads the
+  // routed rows through the permutation instead of from a permuted copy.
+  if (fp8) {
+    const float* sin[HDMOE_MAX_EXPERTS];
+    for (int e = 0; e < E; ++e) sin[e] = p->experts[e].scale_in1;
+    if (int rc = hdmoe_launch_gate_quant(xin, p->gate_w, T, D, E, idx, tw, sin, Hs > 0 ? p->shared->scale_in1 : nullptr,
+                                         a_routed, Hs > 0 ? a_shared : nullptr, s, "hdmoe_moe_ffn (gate + quantise)"))
+      return rc;
+  } else {
+    if (int rc = hdmoe_gate_top2(xin, p->gate_w, T, D, E, idx, tw, stream)) return rc;
+  }
   mark();
   if (int rc = hdmoe_dispatch(idx, T, E, counts, offsets, perm, inv_perm, ws + l.dispatch_ws,
                               hdmoe_dispatch_workspace_bytes(T, E), stream))
@@ -143,12 +158,6 @@ extern "C" int hdmoe_moe_ffn(const hdmoe_layer_args* p, hdmoe_stream_t stream) {
 
   const uint8_t* a_static = nullptr;
   if (fp8) {
-    const float* sin[HDMOE_MAX_EXPERTS];
-    for (int e = 0; e < E; ++e) sin[e] = p->experts[e].scale_in1;
-    // routed rows and the shared expert's token-order copy in one launch ([2T,D] then [T,D] of the same buffer)
-    if (int rc = hdmoe_launch_quant_dispatch(xin, perm, offsets, T, D, E, sin, Hs > 0 ? p->shared->scale_in1 : nullptr,
-                                             Hs > 0, a_routed, s, "hdmoe_moe_ffn (quantise)"))
-      return rc;
     if (Hs > 0) a_static = a_shared;
   } else {
     if (int rc = hdmoe_permute_bf16(xin, perm, T, D, a_routed, stream)) return rc;
@@ -158,7 +167,8 @@ extern "C" int hdmoe_moe_ffn(const hdmoe_layer_args* p, hdmoe_stream_t stream) {
   mark();
   // gate/up projections + SiLU*mul, routed experts and shared expert in one launch
   if (int rc = hdmoe_launch_ffn_gemm(true, wd, a_routed, offsets, (int)n, E, p->experts, h_routed, a_static,
-                                     Hs > 0 ? T : 0, p->shared, h_shared, D, H, D, Hs, s, "hdmoe_moe_ffn (gate/up)"))
+                                     Hs > 0 ? T : 0, p->shared, h_shared, D, H, D, Hs, s, "hdmoe_moe_ffn (gate/up)",
+                                     fp8 ? perm : nullptr, (int)n))
     return rc;
   mark();
   // down projections, both in one launch

@@ -220,7 +220,9 @@ typedef struct hdmoe_layer_args {
   void* topk_weight;  /* [T,2] bf16 */
   /* optional timing hook (may be NULL): HDMOE_NUM_STAGE_EVENTS hipEvent_t created by the caller.
    * Event i is recorded on `stream` before stage i and event i+1 after it; stages in order:
-   * gate, dispatch, quantise/permute, gate-up GEMM, down GEMM, combine. */
+   * gate (with fp8 experts it also casts the activations), dispatch, permute (bf16 experts only), gate-up GEMM,
+   * down GEMM, combine. NULL entries of the array are skipped (each recorded event costs a few microseconds
+   * on the stream). */
   void** stage_events;
   /* optional block fusion (all three NULL = the plain layer). When set, x is the un-normalised token stream and
    * out = x + mod_gate * FFN( LayerNorm(x, ln_eps) * (1 + mod_scale) + mod_shift ); the normalised tokens live in
