@@ -160,3 +160,51 @@ def test_production_row_counts_are_ragged(dev):
         picks.append(perm[rows].long() // 2)
     subset = torch.unique(torch.cat(picks))
     check_layer(sd, x, "fp8", y, idx, w, 4, token_subset=subset)
+
+
+@pytest.mark.parametrize("dim,E,scaled", [(2560, 4, True), (512, 4, True), (512, 8, False), (2560, 2, True)])
+def test_layer_casts_activations_in_the_gate_kernel_bit_exactly(dev, dim, E, scaled):
+    """With fp8 experts the one-call layer leaves, in its workspace, row 2t+s = e4m3fn(x[t] * bf16(1/scale_input of
+    the expert in slot s)) and the shared expert's token-order copy: compared with torch's own casts bit for bit,
+    with different scale_input values per expert (or none: clamp rule)."""
+    import ctypes
+    from comfyui_amd import functional as HF
+    from comfyui_amd import _lib
+    T = 333
+    hidden_arg = 1024
+    master, g = synth.make_weights(5, dim=dim, hidden_arg=hidden_arg, num_experts=E)
+    sd = synth.to_state_dict(master, "fp8", scale_input=scaled)
+    scales = {}
+    if scaled:
+        for i, k in enumerate(sorted(k for k in sd if k.endswith("w1.scale_input"))):
+            v = torch.tensor(0.5 + 0.173 * i, dtype=torch.float32)          # not powers of two
+            sd[k] = v
+            sd[k.replace("w1.", "w3.")] = v.clone()
+            scales[k.rsplit(".w1.", 1)[0]] = v
+    x = (synth.make_input(g, T, dim=dim) * 3).to(BF16)
+    m = synth.build_module({k: v.to(dev) for k, v in sd.items()}, "fp8", dev, dim=dim, hidden_arg=hidden_arg,
+                           num_experts=E, scale_input=scaled)
+    x2 = x.reshape(T, dim).to(dev)
+    wdt, experts, shared, keep = m._collect(x2)
+    H, Hs = m.experts[0].w1.weight.shape[0], m.shared_experts.w1.weight.shape[0]
+    lay = HF.layer_layout(T, dim, H, Hs, E, _lib.W_E4M3FN)
+    ws = torch.zeros(lay.total, dtype=torch.uint8, device=dev)
+    _, idx, _ = HF.moe_ffn(x2, m.gate.weight, experts, shared, H, Hs, wdt, workspace=ws, want_routing=True)
+    torch.cuda.synchronize()
+    a = ws[lay.a:lay.a + 3 * T * dim].cpu().view(3 * T, dim)
+    idx = idx.cpu()
+    xc = x.reshape(T, dim)
+
+    def cast(rows, s):
+        if s is None:
+            return torch.clamp(rows, min=-448, max=448).to(torch.float8_e4m3fn).view(torch.uint8)
+        return (rows * (1.0 / s).to(BF16)).to(torch.float8_e4m3fn).view(torch.uint8)
+
+    for slot in range(2):
+        for e in range(E):
+            sel = (idx[:, slot] == e).nonzero().flatten()
+            if sel.numel():
+                want = cast(xc[sel], scales.get(f"experts.{e}") if scaled else None)
+                assert torch.equal(a[2 * sel + slot], want), (slot, e)
+    want = cast(xc, scales.get("shared_experts") if scaled else None)
+    assert torch.equal(a[2 * T:], want)
