@@ -35,7 +35,7 @@ PEAK_HBM_GBPS = 8000.0      # MI355X HBM3E
 # L2-side traffic of the dominant kernel per launch (bytes fetched + written), from the two rocprofv3 --pmc runs
 # summarised in profiles/bench_cfg3_pmc.txt (FETCH_SIZE x 2.000 and WRITE_SIZE x 1.000 after calibration against a
 # plain 256 MiB copy). Only known for the workload that was profiled.
-MEASURED_TRAFFIC_BYTES = {"cfg3": 1272.8e6 + 142.6e6}
+MEASURED_TRAFFIC_BYTES = {"cfg3": 1290.2e6 + 142.6e6}
 
 
 class HipEvents:
@@ -276,9 +276,10 @@ def main():
     gemm2_tflops = T * fl["down"] / (stage_ms["gemm_down"] * 1e-3) / 1e12
     eb = 1 if fp8 else 2
     gate_bytes = T * D * 2 + E * D * 2 + T * 2 * (4 + 2)
-    # dispatch as built: index sort (read 2T ids twice, write perm + inv_perm) plus the materialised permuted
-    # activation copy for the routed experts and the token-order copy for the shared expert
-    dispatch_bytes = 2 * (2 * T * 4) + 2 * (2 * T * 4) + (2 * T * D * 2 + 2 * T * D * eb) + (T * D * 2 + T * D * eb if fp8 else 0)
+    # dispatch as built: index sort (read 2T ids twice, write perm + inv_perm). fp8: the gate kernel also writes the
+    # token's three e4m3fn rows (two routed slots + shared expert), and nothing is permuted; bf16: the routed rows are
+    # materialised in expert order (read + write 2T rows).
+    dispatch_bytes = 2 * (2 * T * 4) + 2 * (2 * T * 4) + (3 * T * D if fp8 else 2 * (2 * T * D * 2))
     gd_ms = stage_ms["gate"] + stage_ms["dispatch"] + stage_ms["quant_permute"]
     combine_bytes = 2 * T * D * 2 + T * D * 2 + T * D * 2 + T * 2 * 2 + 2 * T * 4
 
