@@ -47,7 +47,8 @@ def test_gate_exact_ties_go_to_lower_index(dev):
     assert w0.cpu().float().tolist() == [[0.25, 0.25]] * 3
 
 
-@pytest.mark.parametrize("T,E", [(1, 4), (5, 4), (1024, 4), (1025, 4), (8192, 4), (3000, 8), (700, 16)])
+@pytest.mark.parametrize("T,E", [(1, 4), (5, 4), (1024, 4), (1025, 4), (8192, 4), (3000, 8), (700, 16), (8191, 2),
+                                 (8193, 6), (20000, 15), (32768, 4), (32769, 4), (40000, 8), (33000, 16)])
 def test_dispatch_bit_exact(dev, T, E):
     g = torch.Generator().manual_seed(T + E)
     first = torch.randint(0, E, (T,), generator=g)
