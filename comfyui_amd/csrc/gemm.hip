@@ -43,13 +43,19 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 
-constexpr int BM = 256;        // tokens per block tile
 constexpr int BN = 256;        // weight rows per block tile
 constexpr int BK = 128;        // K bytes per stage
-constexpr int TILE_BYTES = 256 * BK;
-constexpr int STAGE_BYTES = 2 * TILE_BYTES;
 constexpr int STAGES = 2;
-constexpr int SMEM_BYTES = STAGES * STAGE_BYTES;
+// Tokens per block tile: 2 wave rows x TT MFMA tiles of 32 tokens. TT = 4 (256 tokens) everywhere; the fp8 kernels
+// also exist with TT = 5 (320 tokens: 10 % fewer operand bytes per MAC and fewer tiles), which the launcher picks
+// when its tile count fills the chip as well.
+constexpr int MAX_SLABS = 5;  // 64-row slabs of the largest token tile (arrays of dependent size in lambda
+                              // signatures make the host pass drop the kernel stubs)
+template <int TT>
+struct TileCfg {
+  static constexpr int BM = 64 * TT;                      // tokens per block tile
+  static constexpr int SMEM = STAGES * (BM + 256) * 128;  // dynamic LDS of a block
+};
 constexpr int GROUP_M = 4;     // m-tiles per raster band
 constexpr int NTHREADS = 512;
 constexpr int MAX_GROUPS = HDMOE_MAX_EXPERTS + 1;
@@ -93,11 +99,16 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
-template <int MODE>
+template <int MODE, int TT>
 __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs args) {
   constexpr bool FP8 = (MODE == FP8_SWIGLU || MODE == FP8_PLAIN);
   constexpr bool SWIGLU = (MODE == FP8_SWIGLU || MODE == BF16_SWIGLU);
   constexpr bool BIAS = (MODE == BF16_PLAIN_BIAS);  // Linear with bias and optional GELU (bf16 weights)
+  constexpr int WAVE_TOK = 32 * TT;        // tokens per wave row
+  constexpr int BM = 2 * WAVE_TOK;         // tokens per block tile
+  constexpr int A_SLABS = BM / 64;         // 64-row slabs of the token tile
+  constexpr int A_BYTES = BM * BK;         // token tile of one K step in LDS; the weight tile follows it
+  constexpr int STAGE_BYTES = (BM + BN) * BK;
   constexpr int FEAT_PER_TILE = SWIGLU ? BN / 2 : BN;  // output features per block tile
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
 
@@ -173,28 +184,28 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
   // Plain: wave column wq multiplies LDS rows wq*32..+32 of both halves, and its 64 output features should be
   // contiguous in memory, so LDS row (h, wq, i) holds weight row n0 + wq*64 + h*32 + i.
   __amdgpu_buffer_rsrc_t src_a = make_rsrc(nullptr, 0), src_b0 = src_a, src_b1 = src_a;
-  int src_voff[4] = {0, 0, 0, 0};
+  int src_voff[MAX_SLABS] = {};
   int src_voff_b[2] = {0, 0};
   // Row indices of a gathered token operand: loaded one tile ahead (load_gather), consumed by set_src.
-  auto load_gather = [&](const Tile& d, int (&gi)[4]) {
+  auto load_gather = [&](const Tile& d, int (&gi)[MAX_SLABS]) {
     const GemmGroup& gg = args.g[d.g];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < A_SLABS; ++j) {
       const int r = j * 64 + ld_row;
       gi[j] = (gg.gather != nullptr && r < d.rows_here) ? gg.gather[d.row0 + r] : -1;
     }
   };
-  auto set_src = [&](const Tile& d, const int (&gi)[4]) {
+  auto set_src = [&](const Tile& d, const int (&gi)[MAX_SLABS]) {
     const GemmGroup& gg = args.g[d.g];
     if (gg.gather != nullptr) {
       // rows past the segment end get an offset beyond the buffer and read as zero
       src_a = make_rsrc(gg.a, (uint32_t)gg.a_rows * (uint32_t)d.kbytes);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) src_voff[j] = gi[j] >= 0 ? gi[j] * d.kbytes + ld_chunk * 16 : (int)0x80000000u;
+      for (int j = 0; j < A_SLABS; ++j) src_voff[j] = gi[j] >= 0 ? gi[j] * d.kbytes + ld_chunk * 16 : (int)0x80000000u;
     } else {
       src_a = make_rsrc(gg.a + (size_t)d.row0 * d.kbytes, (uint32_t)d.rows_here * (uint32_t)d.kbytes);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) src_voff[j] = (j * 64 + ld_row) * d.kbytes + ld_chunk * 16;
+      for (int j = 0; j < A_SLABS; ++j) src_voff[j] = (j * 64 + ld_row) * d.kbytes + ld_chunk * 16;
     }
     const uint8_t* b_half0 = gg.b0 + (size_t)d.n0 * d.kbytes;
     const uint8_t* b_half1 = SWIGLU ? gg.b1 + (size_t)d.n0 * d.kbytes : gg.b0 + (size_t)(d.n0 + 32) * d.kbytes;
@@ -209,10 +220,10 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
   };
   auto issue_loads = [&](int stage, int kt) {
     uint8_t* sa = smem + stage * STAGE_BYTES;
-    uint8_t* sb = sa + TILE_BYTES;
+    uint8_t* sb = sa + A_BYTES;
     const int k0 = kt * BK;
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < A_SLABS; ++j)
       __builtin_amdgcn_raw_ptr_buffer_load_lds(src_a, (lds_ptr_t)(sa + ld_lds + j * 64 * BK), 16, src_voff[j], k0, 0, 0);
 #pragma unroll
     for (int j = 0; j < 2; ++j)
@@ -227,10 +238,10 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
   const int fr_row = lane & 31;
   const int fr_grp = lane >> 5;
   const int fr_swz = swz(fr_row);  // tile origins are multiples of 32 rows, so f() only sees fr_row
-  const int a_base = (wt * 128 + fr_row) * BK;               // token operand, + tt*32*BK
-  const int b_base = TILE_BYTES + (wq * 32 + fr_row) * BK;   // weight operand, + ft*128*BK
+  const int a_base = (wt * WAVE_TOK + fr_row) * BK;          // token operand, + tt*32*BK
+  const int b_base = A_BYTES + (wq * 32 + fr_row) * BK;      // weight operand, + ft*128*BK
 
-  v16f acc[2][4];
+  v16f acc[2][TT];
   // n_tt: how many of this wave's four 32-token blocks hold rows of the tile (4 except in the last, partial
   // m-tile of a segment); the others are neither read from LDS nor multiplied.
   auto compute = [&](int stage, auto full_c, int n_tt) {
@@ -241,38 +252,50 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
       for (int ks = 0; ks < 2; ++ks) {
         const int c0 = ((ks * 4 + fr_grp * 2) ^ fr_swz) * 16;
         const int c1 = c0 ^ 16;
-        v8i fa[4], fb[2];
-#pragma unroll
-        for (int tt = 0; tt < 4; ++tt) {
-          if (!FULL && tt >= n_tt) continue;
-          const uint8_t* p = st + a_base + tt * 32 * BK;
+        auto ld = [&](const uint8_t* p) -> v8i {
           const v4i lo = *reinterpret_cast<const v4i*>(p + c0);
           const v4i hi = *reinterpret_cast<const v4i*>(p + c1);
-          fa[tt] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-        }
+          return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        };
         if (!FULL && n_tt == 0) continue;
+        v8i fb[2];
 #pragma unroll
-        for (int ft = 0; ft < 2; ++ft) {
-          const uint8_t* p = st + b_base + ft * 128 * BK;
-          const v4i lo = *reinterpret_cast<const v4i*>(p + c0);
-          const v4i hi = *reinterpret_cast<const v4i*>(p + c1);
-          fb[ft] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-        }
+        for (int ft = 0; ft < 2; ++ft) fb[ft] = ld(st + b_base + ft * 128 * BK);
+        if constexpr (TT <= 4) {
+          // all token fragments of the slice at once
+          v8i fa[TT];
 #pragma unroll
-        for (int ft = 0; ft < 2; ++ft)
-#pragma unroll
-          for (int tt = 0; tt < 4; ++tt) {
+          for (int tt = 0; tt < TT; ++tt) {
             if (!FULL && tt >= n_tt) continue;
-            acc[ft][tt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[ft], fa[tt], acc[ft][tt], 0, 0, 0, 0, 0, 0);
+            fa[tt] = ld(st + a_base + tt * 32 * BK);
           }
+#pragma unroll
+          for (int ft = 0; ft < 2; ++ft)
+#pragma unroll
+            for (int tt = 0; tt < TT; ++tt) {
+              if (!FULL && tt >= n_tt) continue;
+              acc[ft][tt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[ft], fa[tt], acc[ft][tt], 0, 0, 0, 0, 0, 0);
+            }
+        } else {
+          // taller tiles: one token fragment ahead of the MFMAs instead of all of them (registers)
+          v8i fa_cur = ld(st + a_base), fa_nxt = fa_cur;
+#pragma unroll
+          for (int tt = 0; tt < TT; ++tt) {
+            if (!FULL && tt >= n_tt) continue;
+            if (tt + 1 < TT && (FULL || tt + 1 < n_tt)) fa_nxt = ld(st + a_base + (tt + 1) * 32 * BK);
+            acc[0][tt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[0], fa_cur, acc[0][tt], 0, 0, 0, 0, 0, 0);
+            acc[1][tt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[1], fa_cur, acc[1][tt], 0, 0, 0, 0, 0, 0);
+            fa_cur = fa_nxt;
+          }
+        }
       }
     } else {
 #pragma unroll
       for (int ks = 0; ks < 4; ++ks) {
         const int c0 = ((ks * 2 + fr_grp) ^ fr_swz) * 16;
-        v8bf fa[4], fb[2];
+        v8bf fa[TT], fb[2];
 #pragma unroll
-        for (int tt = 0; tt < 4; ++tt) {
+        for (int tt = 0; tt < TT; ++tt) {
           if (!FULL && tt >= n_tt) continue;
           fa[tt] = *reinterpret_cast<const v8bf*>(st + a_base + tt * 32 * BK + c0);
         }
@@ -283,7 +306,7 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
 #pragma unroll
         for (int ft = 0; ft < 2; ++ft)
 #pragma unroll
-          for (int tt = 0; tt < 4; ++tt) {
+          for (int tt = 0; tt < TT; ++tt) {
             if (!FULL && tt >= n_tt) continue;
             acc[ft][tt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[ft], fa[tt], acc[ft][tt], 0, 0, 0);
           }
@@ -355,8 +378,8 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
       auto swiglu_tile = [&](auto next_mode) {
         constexpr int NEXT = decltype(next_mode)::value;  // 0 clamp, 1 unit scale, 2 general scale
 #pragma unroll
-        for (int tt = 0; tt < 4; ++tt) {
-          const int tok = wt * 128 + tt * 32 + tok32;
+        for (int tt = 0; tt < TT; ++tt) {
+          const int tok = wt * WAVE_TOK + tt * 32 + tok32;
           uint8_t* const row = stg + tok * ROWB;
 #pragma unroll
           for (int q = 0; q < 4; ++q) {
@@ -411,8 +434,8 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
       constexpr int ROWS_PER_PASS = 64 / LANES_PER_ROW;
       const int c = lane % LANES_PER_ROW;
 #pragma unroll
-      for (int p = 0; p < 32 / ROWS_PER_PASS; ++p) {
-        const int r = wave * 32 + p * ROWS_PER_PASS + lane / LANES_PER_ROW;
+      for (int p = 0; p < (BM / 8) / ROWS_PER_PASS; ++p) {
+        const int r = wave * (BM / 8) + p * ROWS_PER_PASS + lane / LANES_PER_ROW;
         const v4i v = *reinterpret_cast<const v4i*>(stg + r * ROWB + ((c ^ (r & 7)) << 4));
         __builtin_amdgcn_raw_buffer_store_b128(v, ro, r * ldo + d.n0 * EB + c * 16, 0, 0);
       }
@@ -424,7 +447,7 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
       uint8_t* const mine = stg + wave * 8192;
       const int rd_row = lane >> 3, rd_c = lane & 7;
 #pragma unroll
-      for (int tt = 0; tt < 4; ++tt) {
+      for (int tt = 0; tt < TT; ++tt) {
         uint8_t* const buf = mine + (tt & 1) * 4096;
         wave_sync();  // the reads of two rounds ago are ahead of these writes
 #pragma unroll
@@ -461,7 +484,7 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
         for (int p = 0; p < 4; ++p) {
           const int r = p * 8 + rd_row;
           const v4i v = *reinterpret_cast<const v4i*>(buf + r * 128 + ((rd_c ^ rd_row) << 4));
-          __builtin_amdgcn_raw_buffer_store_b128(v, ro, (wt * 128 + tt * 32 + r) * ldo + (d.n0 + wq * 64) * 2 + rd_c * 16, 0, 0);
+          __builtin_amdgcn_raw_buffer_store_b128(v, ro, (wt * WAVE_TOK + tt * 32 + r) * ldo + (d.n0 + wq * 64) * 2 + rd_c * 16, 0, 0);
         }
       }
     }
@@ -473,7 +496,9 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
   // current one, so its latency hides behind the stores.
   Tile cur = decode(0);
   if (cur.g < 0) return;
-  int gi_cur[4], gi_nxt[4] = {-1, -1, -1, -1};
+  int gi_cur[MAX_SLABS], gi_nxt[MAX_SLABS];
+#pragma unroll
+  for (int j = 0; j < A_SLABS; ++j) gi_nxt[j] = -1;
   load_gather(cur, gi_cur);
   set_src(cur, gi_cur);
   issue_loads(0, 0);
@@ -485,7 +510,7 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
 #pragma unroll
     for (int a2 = 0; a2 < 2; ++a2)
 #pragma unroll
-      for (int b2 = 0; b2 < 4; ++b2)
+      for (int b2 = 0; b2 < TT; ++b2)
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[a2][b2][r] = 0.0f;
     auto k_loop = [&](auto full_c, int n_tt) {
@@ -502,8 +527,8 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
         }
       }
     };
-    const int my_rows = __builtin_amdgcn_readfirstlane(cur.rows_here) - wt * 128;  // rows of the tile in this wave's half
-    if (my_rows >= 97) k_loop(std::true_type{}, 4);
+    const int my_rows = __builtin_amdgcn_readfirstlane(cur.rows_here) - wt * WAVE_TOK;  // rows of the tile in this wave's half
+    if (my_rows > 32 * (TT - 1)) k_loop(std::true_type{}, TT);
     else k_loop(std::false_type{}, my_rows <= 0 ? 0 : (my_rows + 31) / 32);
     // Every wave is done reading both stages: stage 0 can take the next tile's first K step, stage 1 the
     // staged outputs of this one (it is not loaded into again before the barrier of that K step).
@@ -517,7 +542,7 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
   }
 }
 
-template <int MODE>
+template <int MODE, int TT = 4>
 int launch_grouped(const GemmArgs& args, int tile_bound, hipStream_t s, const char* what) {
   // The opt-in for more than 64 KiB of dynamic LDS is a per-device function attribute: remembered per device
   // and instantiation (a race between two threads sets it twice, which is harmless).
@@ -525,8 +550,8 @@ int launch_grouped(const GemmArgs& args, int tile_bound, hipStream_t s, const ch
   int device = 0;
   if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) device = -1;
   if (device < 0 || !attr_set[device]) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&grouped_gemm_kernel<MODE>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES);
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&grouped_gemm_kernel<MODE, TT>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, TileCfg<TT>::SMEM);
     if (e != hipSuccess) return hdmoe_fail(HDMOE_E_LAUNCH, "%s: hipFuncSetAttribute: %s", what, hipGetErrorString(e));
     if (device >= 0) attr_set[device] = true;
   }
@@ -534,7 +559,7 @@ int launch_grouped(const GemmArgs& args, int tile_bound, hipStream_t s, const ch
   // persistent blocks: one per CU (128 KiB of LDS allow no second one), a multiple of the XCD count
   int grid = (tile_bound + HDMOE_NUM_XCD - 1) / HDMOE_NUM_XCD * HDMOE_NUM_XCD;
   if (grid > HDMOE_NUM_CU) grid = HDMOE_NUM_CU;
-  hipLaunchKernelGGL((grouped_gemm_kernel<MODE>), dim3(grid), dim3(NTHREADS), SMEM_BYTES, s, args);
+  hipLaunchKernelGGL((grouped_gemm_kernel<MODE, TT>), dim3(grid), dim3(NTHREADS), TileCfg<TT>::SMEM, s, args);
   return hdmoe_check_launch(what);
 }
 
@@ -560,6 +585,17 @@ int hdmoe_launch_ffn_gemm(bool swiglu, int weight_dtype, const uint8_t* a_dyn, c
   const int eb = elem_bytes(weight_dtype);
   const bool fp8 = weight_dtype == HDMOE_W_E4M3FN;
   const int feat_per_tile = swiglu ? BN / 2 : BN;
+  // Tile height. Expected tiles with evenly loaded experts, static round-robin over the CUs, and a fixed cost per tile
+  // of about one 32-token block: rounds x (TT + 1). The taller tile wins when it does not add a round.
+  auto expected_cost = [&](int tt) {
+    const int bm = 64 * tt;
+    long tiles = 0;
+    if (n_dyn > 0) tiles += (long)n_dyn * ((rows_dyn / n_dyn + bm - 1) / bm) * (N_dyn / feat_per_tile);
+    if (shared != nullptr && rows_static > 0) tiles += (long)((rows_static + bm - 1) / bm) * (N_static / feat_per_tile);
+    return ((tiles + HDMOE_NUM_CU - 1) / HDMOE_NUM_CU) * (tt + 1);
+  };
+  const bool tall = fp8 && expected_cost(5) < expected_cost(4);
+  const int BM = tall ? TileCfg<5>::BM : TileCfg<4>::BM;  // tokens per block tile of the kernel that will run
   if (gather_dyn != nullptr && (unsigned long long)gather_rows * K_dyn * eb >= (1ull << 31))
     return hdmoe_fail(HDMOE_E_SHAPE, "%s: %d gathered rows of %d bytes exceed the 2 GiB offset range", what, gather_rows,
                       K_dyn * eb);
@@ -612,6 +648,8 @@ int hdmoe_launch_ffn_gemm(bool swiglu, int weight_dtype, const uint8_t* a_dyn, c
     ++G;
   }
   args.G = G;
+  if (fp8 && tall) return swiglu ? launch_grouped<FP8_SWIGLU, 5>(args, tile_bound, s, what)
+                                 : launch_grouped<FP8_PLAIN, 5>(args, tile_bound, s, what);
   if (fp8) return swiglu ? launch_grouped<FP8_SWIGLU>(args, tile_bound, s, what)
                          : launch_grouped<FP8_PLAIN>(args, tile_bound, s, what);
   return swiglu ? launch_grouped<BF16_SWIGLU>(args, tile_bound, s, what)
@@ -645,6 +683,7 @@ int hdmoe_launch_linear_groups(const uint8_t* a_dyn, const int32_t* offsets, int
     gg.dyn = e;
     if (!gg.b0) return hdmoe_fail(HDMOE_E_NULL, "%s: expert %d has a NULL weight", what, e);
   }
+  constexpr int BM = TileCfg<4>::BM;
   if (n_dyn > 0) tile_bound += (rows_dyn / BM + n_dyn) * (N / BN);
   if (shared != nullptr && rows_static > 0) {
     GemmGroup& gg = args.g[G];

@@ -122,8 +122,9 @@ def test_quant_permute(dev):
         assert torch.equal(got[lo:hi].view(torch.uint8), want.view(torch.uint8))
 
 
+# the last two shapes make the launcher pick the 320-token tile for the plain fp8 kernel (fewer rounds over the CUs)
 @pytest.mark.parametrize("rows,K,N", [(256, 128, 256), (1, 2560, 256), (300, 2560, 512), (513, 6912, 2560),
-                                      (1000, 384, 768)])
+                                      (1000, 384, 768), (1280, 256, 16384), (1301, 384, 16384)])
 def test_linear_fp8(dev, rows, K, N):
     g = torch.Generator().manual_seed(rows + K + N)
     a = torch.randn((rows, K), generator=g).to(FP8)
