@@ -35,7 +35,7 @@ PEAK_HBM_GBPS = 8000.0      # MI355X HBM3E
 # L2-side traffic of the dominant kernel per launch (bytes fetched + written), from the two rocprofv3 --pmc runs
 # summarised in profiles/bench_cfg3_pmc.txt (FETCH_SIZE x 2.000 and WRITE_SIZE x 1.000 after calibration against a
 # plain 256 MiB copy). Only known for the workload that was profiled.
-MEASURED_TRAFFIC_BYTES = {"cfg3": 1290.2e6 + 142.6e6}
+MEASURED_TRAFFIC_BYTES = {"cfg3": 1088.7e6 + 145.8e6}
 
 
 class HipEvents:
@@ -323,7 +323,7 @@ def main():
         "stage_ms": stage_ms,
         "gemm_down_tflops": gemm2_tflops,
         "roofline": {
-            "kernel": "grouped_gemm_kernel<FP8_SWIGLU>" if fp8 else "grouped_gemm_kernel<BF16_SWIGLU>",
+            "kernel": "grouped_gemm_kernel<FP8_SWIGLU, TT> (TT = 5 at 8192 tokens)" if fp8 else "grouped_gemm_kernel<BF16_SWIGLU>",
             "bound": "mfma",
             "achieved": gemm1_tflops,
             "peak": peak,
