@@ -19,7 +19,7 @@ __device__ __forceinline__ float bf16_hi(uint32_t u) { return __uint_as_float(u 
 __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) { return hdmoe_dev_pack_bf16(lo, hi); }
 __device__ __forceinline__ float round_bf16(float f) { return hdmoe_dev_round_bf16(f); }
 __device__ __forceinline__ uint2 quant8(const uint4& v, float inv) { return hdmoe_q_8(v, inv); }
-__device__ __forceinline__ float inv_scale(const float* s) { return hdmoe_q_inv_scale(s); }
+__device__ __forceinline__ float inv_scale(const float* s) { return hdmoe_q_uniform(hdmoe_q_inv_scale(s)); }
 
 __global__ __launch_bounds__(THREADS) void quant_rows_kernel(const uint4* __restrict__ x, long rows, int row16,
                                                              const float* scale_in, uint2* __restrict__ out) {

@@ -58,15 +58,35 @@ __device__ __forceinline__ float dot8(const uint4& a, const uint4& b, float acc)
   return acc;
 }
 
+// Sum over the wave in the fixed butterfly order v[l] + v[l ^ off], off = 32, 16, 8, 4, 2, 1, every lane ending
+// with the total. No LDS traffic: the halves and the 16-lane rows are exchanged with the lane-swap instructions,
+// the rest with DPP. After the first two steps the values repeat every 16 lanes, so the rotate by 8 inside a row
+// is the xor-8 partner, and once they repeat every 8 lanes the rotate by 4 is the xor-4 partner; fp32 addition is
+// commutative, so each lane forms exactly the sum the plain xor shuffle would.
+__device__ __forceinline__ float wave_sum(float v) {
+  uint32_t b = __float_as_uint(v);
+  auto h = __builtin_amdgcn_permlane32_swap(b, b, false, false);
+  v = __uint_as_float(h[0]) + __uint_as_float(h[1]);
+  b = __float_as_uint(v);
+  auto r = __builtin_amdgcn_permlane16_swap(b, b, false, false);
+  v = __uint_as_float(r[0]) + __uint_as_float(r[1]);
+  int x = __float_as_int(v);
+  v = v + __int_as_float(__builtin_amdgcn_update_dpp(x, x, 0x128, 0xf, 0xf, false));  // row_ror:8
+  x = __float_as_int(v);
+  v = v + __int_as_float(__builtin_amdgcn_update_dpp(x, x, 0x124, 0xf, 0xf, false));  // row_ror:4
+  x = __float_as_int(v);
+  v = v + __int_as_float(__builtin_amdgcn_update_dpp(x, x, 0x4e, 0xf, 0xf, false));   // quad_perm:[2,3,0,1]
+  x = __float_as_int(v);
+  v = v + __int_as_float(__builtin_amdgcn_update_dpp(x, x, 0xb1, 0xf, 0xf, false));   // quad_perm:[1,0,3,2]
+  return v;
+}
+
 template <int E>
 __device__ __forceinline__ void finish_token(float (&logit)[E], int lane, int t, int32_t* idx,
                                              uint16_t* wout, int& first, int& second) {
 #pragma unroll
   for (int e = 0; e < E; ++e) {
-    float v = logit[e];
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) v = v + __shfl_xor(v, off, 64);
-    logit[e] = hdmoe_round_bf16(v);  // F.linear output is a bf16 tensor
+    logit[e] = hdmoe_round_bf16(wave_sum(logit[e]));  // F.linear output is a bf16 tensor
   }
   float mx = logit[0];
 #pragma unroll
@@ -130,6 +150,14 @@ __global__ __launch_bounds__(WAVES_PER_BLOCK * 64) void gate_top2_reg_kernel(
 
   int t = wave;
   if (t >= T) return;
+  // the 1/scale_input of every expert, read once: a load that depends on the routing inside the token loop
+  // would make every token wait for its predecessor's stores (loads and stores retire in order)
+  float inv_e[E], invs = -1.0f;
+  if constexpr (QUANT) {
+#pragma unroll
+    for (int e = 0; e < E; ++e) inv_e[e] = hdmoe_q_inv_scale(q.scale_in.p[e]);
+    invs = hdmoe_q_uniform(hdmoe_q_inv_scale(q.shared_scale));
+  }
   uint4 cur[NCHUNK], nxt[NCHUNK];
 #pragma unroll
   for (int c = 0; c < NCHUNK; ++c) cur[c] = x[(size_t)t * ROW16 + c * 64 + lane];
@@ -155,8 +183,14 @@ __global__ __launch_bounds__(WAVES_PER_BLOCK * 64) void gate_top2_reg_kernel(
     int i0, i1;
     finish_token<E>(logit, lane, t, idx, wout, i0, i1);
     if constexpr (QUANT) {
-      const float inv0 = hdmoe_q_inv_scale(q.scale_in.p[i0]), inv1 = hdmoe_q_inv_scale(q.scale_in.p[i1]);
-      const float invs = hdmoe_q_inv_scale(q.shared_scale);
+      float inv0 = inv_e[0], inv1 = inv_e[0];
+#pragma unroll
+      for (int e = 1; e < E; ++e) {
+        inv0 = i0 == e ? inv_e[e] : inv0;
+        inv1 = i1 == e ? inv_e[e] : inv1;
+      }
+      inv0 = hdmoe_q_uniform(inv0);
+      inv1 = hdmoe_q_uniform(inv1);
       uint2* r0 = q.xq_routed + (size_t)(2 * t) * ROW16;
       const bool same01 = inv0 == inv1, same0s = inv0 == invs;  // equal scales: cast once, store again
 #pragma unroll
@@ -194,8 +228,9 @@ __global__ __launch_bounds__(WAVES_PER_BLOCK * 64) void gate_top2_generic_kernel
     int i0, i1;
     finish_token<E>(logit, lane, t, idx, wout, i0, i1);
     if constexpr (QUANT) {
-      const float inv0 = hdmoe_q_inv_scale(q.scale_in.p[i0]), inv1 = hdmoe_q_inv_scale(q.scale_in.p[i1]);
-      const float invs = hdmoe_q_inv_scale(q.shared_scale);
+      const float inv0 = hdmoe_q_uniform(hdmoe_q_inv_scale(q.scale_in.p[i0]));
+      const float inv1 = hdmoe_q_uniform(hdmoe_q_inv_scale(q.scale_in.p[i1]));
+      const float invs = hdmoe_q_uniform(hdmoe_q_inv_scale(q.shared_scale));
       for (int u = lane; u < row16; u += 64) {
         const uint4 xv = x[(size_t)t * row16 + u];
         q.xq_routed[(size_t)(2 * t) * row16 + u] = hdmoe_q_8(xv, inv0);
@@ -210,7 +245,10 @@ template <int E>
 int launch_gate(const void* x, const void* wg, int T, int D, int32_t* idx, void* w, const GateQuant* quant,
                 hipStream_t s, const char* what) {
   // about 4 tokens per wave amortise the register-resident weight slice and still give 8 waves per CU at T = 8192
-  int blocks = (T + WAVES_PER_BLOCK * 4 - 1) / (WAVES_PER_BLOCK * 4);
+#ifndef GATE_TPW
+#define GATE_TPW 4
+#endif
+  int blocks = (T + WAVES_PER_BLOCK * GATE_TPW - 1) / (WAVES_PER_BLOCK * GATE_TPW);
   if (blocks < 1) blocks = 1;
   if (blocks > HDMOE_NUM_CU * 8) blocks = HDMOE_NUM_CU * 8;
   dim3 grid(blocks), block(WAVES_PER_BLOCK * 64);
@@ -250,12 +288,6 @@ int dispatch_gate(const void* x_bf16, const void* gate_w_bf16, int T, int D, int
 // as the gate kernel; mean and variance are two passes over the registers with the same fixed fp32 order
 // (per-lane ascending elements, then the xor butterfly), so the CPU checker can restate it bit for bit.
 // The root is __builtin_sqrtf, which hipcc rounds correctly; __fsqrt_rn is the approximate native root here.
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int off = 32; off >= 1; off >>= 1) v = v + __shfl_xor(v, off, 64);
-  return v;
-}
-
 __device__ __forceinline__ void unpack8(const uint4& a, float (&f)[8]) {
   f[0] = bf16_lo(a.x); f[1] = bf16_hi(a.x); f[2] = bf16_lo(a.y); f[3] = bf16_hi(a.y);
   f[4] = bf16_lo(a.z); f[5] = bf16_hi(a.z); f[6] = bf16_lo(a.w); f[7] = bf16_hi(a.w);

@@ -9,7 +9,13 @@ struct HdmoeScalePtrs {
 };
 
 #if defined(__HIPCC__)
-// inv < 0 selects the scale_input-is-None rule (clamp to +-448, scale 1).
+// All helpers take inv = (1.0 / scale_input).to(bfloat16), or a negative value for the scale_input-is-None rule
+// (clamp to +-448, scale 1). inv must be the same in every lane of the wave; pass it through hdmoe_q_uniform
+// once so that the branches on it are scalar.
+__device__ __forceinline__ float hdmoe_q_uniform(float inv) {
+  return __uint_as_float(__builtin_amdgcn_readfirstlane(__float_as_uint(inv)));
+}
+
 __device__ __forceinline__ float hdmoe_q_pre(float v, float inv) {
   if (inv < 0.0f) return v < -448.0f ? -448.0f : (v > 448.0f ? 448.0f : v);
   return hdmoe_dev_round_bf16(v * inv);  // bf16 tensor times bf16 scalar, rounded to bf16
@@ -21,12 +27,49 @@ __device__ __forceinline__ uint32_t hdmoe_q_2(uint32_t u, float inv) {
                                hdmoe_q_pre(__uint_as_float(u & 0xffff0000u), inv));
 }
 
-// eight bf16 values -> eight e4m3fn bytes
+// eight bf16 values -> eight e4m3fn bytes. A scale of exactly 1 skips the multiply (x * 1 rounded to bf16 is x);
+// the rule "beyond the rounding midpoint above 448 -> NaN" is checked once for the eight values (largest
+// magnitude as an integer compare, which also catches NaN inputs, whose cast is sign | 0x7F either way) and
+// patched per byte only when it fires.
 __device__ __forceinline__ uint2 hdmoe_q_8(const uint4& v, float inv) {
-  uint2 o;
-  o.x = hdmoe_q_2(v.x, inv) | (hdmoe_q_2(v.y, inv) << 16);
-  o.y = hdmoe_q_2(v.z, inv) | (hdmoe_q_2(v.w, inv) << 16);
-  return o;
+  const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+  float f[8];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    f[2 * j] = __uint_as_float(w[j] << 16);
+    f[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+  }
+  if (inv < 0.0f) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) f[j] = f[j] < -448.0f ? -448.0f : (f[j] > 448.0f ? 448.0f : f[j]);
+  } else if (inv != 1.0f) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint32_t p = hdmoe_dev_pack_bf16(f[2 * j] * inv, f[2 * j + 1] * inv);
+      f[2 * j] = __uint_as_float(p << 16);
+      f[2 * j + 1] = __uint_as_float(p & 0xffff0000u);
+    }
+  }
+  uint32_t o[2];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    int p = __builtin_amdgcn_cvt_pk_fp8_f32(f[4 * h], f[4 * h + 1], 0, false);
+    o[h] = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(f[4 * h + 2], f[4 * h + 3], p, true);
+  }
+  if (!(inv < 0.0f)) {
+    uint32_t m = 0;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const uint32_t a = __float_as_uint(f[j]) & 0x7fffffffu;
+      m = a > m ? a : m;
+    }
+    if (m > 0x43e80000u) {  // some |value| > 464 (or NaN)
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        if ((__float_as_uint(f[j]) & 0x7fffffffu) > 0x43e80000u) o[j >> 2] |= 0x7fu << (8 * (j & 3));
+    }
+  }
+  return make_uint2(o[0], o[1]);
 }
 
 // (1.0 / scale_input).to(bfloat16) as fp32; NULL pointer -> clamp rule marker

@@ -16,6 +16,7 @@ otherwise it composes the same HIP stages per expert through the Linear modules,
 needs the per-expert row counts on the host (one sync, as the reference's mask indexing).
 Inputs must be bf16 HIP tensors: there is no CPU path.
 """
+import weakref
 from typing import Optional
 
 import torch
@@ -32,15 +33,17 @@ _scale_cache = {}
 
 
 def _scale_value(p):
-    """Host copy of an fp32 scalar Parameter, cached on (identity, version, address): read once per parameter
-    object, so steady-state forwards do not synchronise."""
-    key = (id(p), p._version, p.data_ptr())
-    v = _scale_cache.get(key)
-    if v is None:
-        if len(_scale_cache) > 4096:
-            _scale_cache.clear()
-        v = float(p.detach().float().cpu())
-        _scale_cache[key] = v
+    """Host copy of an fp32 scalar Parameter, read once per (parameter object, version, address), so steady-state
+    forwards do not synchronise. The entry keeps a weak reference to the tensor it was read from: an id or an
+    address alone can be reused by a different tensor after the first one is freed."""
+    key = id(p)
+    hit = _scale_cache.get(key)
+    if hit is not None and hit[0]() is p and hit[1] == p._version and hit[2] == p.data_ptr():
+        return hit[3]
+    if len(_scale_cache) > 4096:
+        _scale_cache.clear()
+    v = float(p.detach().float().cpu())
+    _scale_cache[key] = (weakref.ref(p), p._version, p.data_ptr(), v)
     return v
 
 

@@ -108,10 +108,13 @@ class CastWeightBiasOp:
 
 
 def _linear_bf16(input, weight, bias):
-    if bias is not None:
-        raise NotImplementedError("comfyui_amd Linear: bias is not part of the MoE feed-forward path")
     shape = input.shape
-    out = HF.linear(input.reshape(-1, shape[-1]).contiguous(), weight.contiguous())
+    x2 = input.reshape(-1, shape[-1]).contiguous()
+    if bias is not None:
+        # the bias is added to the fp32 accumulator before the one rounding to bf16, like F.linear's fused epilogue
+        _, out = HF.grouped_linear(x2[:0], None, [], a_static=x2, shared=(weight.contiguous(), bias.contiguous()))
+    else:
+        out = HF.linear(x2, weight.contiguous())
     return out.reshape(*shape[:-1], weight.shape[0])
 
 

@@ -52,6 +52,26 @@ def test_plain_and_manual_cast_linear(dev):
     assert lin2.weight.device.type == "cpu"
 
 
+def test_linear_with_bias(dev):
+    """operations.Linear with a bias (comfy/ops.py:103-115): bias joins the fp32 accumulator, one rounding."""
+    from comfyui_amd import ops
+    g = torch.Generator().manual_seed(5)
+    w = (torch.randn((512, 256), generator=g) * 0.05).to(BF16)
+    b = torch.randn((512,), generator=g).to(BF16)
+    x = torch.randn((2, 77, 256), generator=g).to(BF16)
+    ref = O.linear_bias(x, w, b)
+    for cls, wdev, wdtype in ((ops.disable_weight_init, dev, BF16), (ops.manual_cast, "cpu", torch.float32)):
+        lin = cls.Linear(256, 512, bias=True, dtype=wdtype, device=wdev)
+        with torch.no_grad():
+            lin.weight.copy_(w)
+            lin.bias.copy_(b)
+        y = lin(x.to(dev))
+        assert y.shape == (2, 77, 512) and y.dtype == BF16
+        close(y.cpu(), ref, 3e-3)
+        # at most one bf16 step (summation order): |y| < 8 here, so a step is at most 2^-5
+        assert float((y.cpu().float() - ref.float()).abs().max()) <= 2.0 ** -5
+
+
 def test_scaled_fp8_linear_with_fp8_matmul(dev):
     from comfyui_amd import ops
     cls = ops.scaled_fp8_ops(fp8_matrix_mult=True, scale_input=True, override_dtype=FP8)

@@ -150,3 +150,18 @@ def test_product_never_imports_the_oracle():
                 text = open(os.path.join(dirpath, f)).read()
                 assert not re.search(r"^\s*(from|import)\s+oracle\b", text, flags=re.M), f
                 assert "libhdmoe_oracle" not in text and "moe_ref" not in text, f
+
+
+def test_scale_cache_is_not_fooled_by_a_reused_id_or_address():
+    """The host copy of a scale is cached per parameter object; an entry left by a freed tensor whose id and address
+    a new tensor happens to reuse must not be served for the new one."""
+    import weakref
+    from comfyui_amd import hidream
+    old = torch.nn.Parameter(torch.tensor(3.0), requires_grad=False)
+    new = torch.nn.Parameter(torch.tensor(0.25), requires_grad=False)
+    hidream._scale_cache[id(new)] = (weakref.ref(old), new._version, new.data_ptr(), 3.0)
+    assert hidream._scale_value(new) == 0.25
+    assert hidream._scale_value(new) == 0.25          # now served from the refreshed entry
+    with torch.no_grad():
+        new.fill_(0.5)                                 # in-place update bumps the version
+    assert hidream._scale_value(new) == 0.5
