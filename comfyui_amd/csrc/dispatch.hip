@@ -3,7 +3,7 @@
 // (/root/reference/comfy/ldm/hidream/model.py:313-318), which pick, for expert i,
 // the flat slots p = 2t+s with topk_idx[p] == i in ascending p.
 //
-// Two launches over chunks of CHUNK flat slots:
+// Two launches over chunks of 256 flat slots (2048 above 2^16 slots):
 //   count:   per-chunk expert histogram from wave ballots        -> chunk_counts[chunk][E]
 //   scatter: every block sums the histograms of the chunks before it (and all of
 //            them for the global counts/offsets), then ranks its own slots with
@@ -17,12 +17,21 @@ namespace {
 
 constexpr int THREADS = 256;
 constexpr int WAVES = THREADS / 64;
-constexpr int ITEMS = 8;
-constexpr int CHUNK = THREADS * ITEMS;  // flat slots per block
+// A block handles THREADS * ITEMS flat slots. Few items per block keep the serial part of a block short (this
+// stage is latency bound at the sizes of one layer); many items bound the number of per-chunk histograms every
+// block has to sum at very large T.
+#ifndef DISPATCH_SMALL_ITEMS
+#define DISPATCH_SMALL_ITEMS 1
+#endif
+constexpr int ITEMS_SMALL = DISPATCH_SMALL_ITEMS, ITEMS_LARGE = 8;
+constexpr int SMALL_MAX_SLOTS = 1 << 16;
+inline int items_for(size_t n) { return n <= (size_t)SMALL_MAX_SLOTS ? ITEMS_SMALL : ITEMS_LARGE; }
 
+template <int ITEMS>
 __global__ __launch_bounds__(THREADS) void dispatch_count_kernel(const int32_t* __restrict__ flat, int n,
                                                                  int E, int32_t* __restrict__ chunk_counts) {
   __shared__ int32_t wave_cnt[WAVES][HDMOE_MAX_EXPERTS];
+  constexpr int CHUNK = THREADS * ITEMS;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int base = blockIdx.x * CHUNK;
   int32_t cnt = 0;  // lane e (< E) of each wave accumulates the wave's count for expert e
@@ -43,6 +52,7 @@ __global__ __launch_bounds__(THREADS) void dispatch_count_kernel(const int32_t* 
   }
 }
 
+template <int ITEMS>
 __global__ __launch_bounds__(THREADS) void dispatch_scatter_kernel(
     const int32_t* __restrict__ flat, int n, int E, int nchunks, const int32_t* __restrict__ chunk_counts,
     int32_t* __restrict__ counts, int32_t* __restrict__ offsets, int32_t* __restrict__ perm,
@@ -79,6 +89,7 @@ __global__ __launch_bounds__(THREADS) void dispatch_scatter_kernel(
   }
   __syncthreads();
 
+  constexpr int CHUNK = THREADS * ITEMS;
   const int base = blockIdx.x * CHUNK;
   const unsigned long long lt = (1ull << lane) - 1ull;
   for (int it = 0; it < ITEMS; ++it) {
@@ -115,7 +126,8 @@ __global__ __launch_bounds__(THREADS) void dispatch_scatter_kernel(
 extern "C" size_t hdmoe_dispatch_workspace_bytes(int T, int E) {
   if (T < 0 || E < 1) return 0;
   const size_t n = (size_t)T * HDMOE_TOPK;
-  const size_t nchunks = (n + CHUNK - 1) / CHUNK;
+  const size_t chunk = (size_t)THREADS * items_for(n);
+  const size_t nchunks = (n + chunk - 1) / chunk;
   return hdmoe_align_up((nchunks > 0 ? nchunks : 1) * (size_t)E * sizeof(int32_t), 256);
 }
 
@@ -137,11 +149,19 @@ extern "C" int hdmoe_dispatch(const int32_t* topk_idx, int T, int E, int32_t* co
                       workspace_bytes, hdmoe_dispatch_workspace_bytes(T, E));
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int n = T * HDMOE_TOPK;
-  int nchunks = (n + CHUNK - 1) / CHUNK;
+  const int items = items_for((size_t)n);
+  const int chunk = THREADS * items;
+  int nchunks = (n + chunk - 1) / chunk;
   if (nchunks < 1) nchunks = 1;  // T == 0 still writes counts = 0 and offsets = 0
   int32_t* cc = static_cast<int32_t*>(workspace);
-  hipLaunchKernelGGL(dispatch_count_kernel, dim3(nchunks), dim3(THREADS), 0, s, topk_idx, n, E, cc);
-  hipLaunchKernelGGL(dispatch_scatter_kernel, dim3(nchunks), dim3(THREADS), 0, s, topk_idx, n, E, nchunks, cc,
-                     counts, offsets, perm, inv_perm);
+  if (items == ITEMS_SMALL) {
+    hipLaunchKernelGGL(dispatch_count_kernel<ITEMS_SMALL>, dim3(nchunks), dim3(THREADS), 0, s, topk_idx, n, E, cc);
+    hipLaunchKernelGGL(dispatch_scatter_kernel<ITEMS_SMALL>, dim3(nchunks), dim3(THREADS), 0, s, topk_idx, n, E,
+                       nchunks, cc, counts, offsets, perm, inv_perm);
+  } else {
+    hipLaunchKernelGGL(dispatch_count_kernel<ITEMS_LARGE>, dim3(nchunks), dim3(THREADS), 0, s, topk_idx, n, E, cc);
+    hipLaunchKernelGGL(dispatch_scatter_kernel<ITEMS_LARGE>, dim3(nchunks), dim3(THREADS), 0, s, topk_idx, n, E,
+                       nchunks, cc, counts, offsets, perm, inv_perm);
+  }
   return hdmoe_check_launch("hdmoe_dispatch");
 }

@@ -411,7 +411,7 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
             const int byte = (wq * 32 + q * 8 + hi32 * 4) * EB;  // position of the 4 features in the staged row
             uint8_t* const dst = row + ((((byte >> 4) ^ (tok32 & 7)) << 4) | (byte & 15));
             if constexpr (FP8) {
-              *reinterpret_cast<uint32_t*>(dst) = hdmoe_dev_pack_e4m3fn(m[0], m[1]) | (hdmoe_dev_pack_e4m3fn(m[2], m[3]) << 16);
+              *reinterpret_cast<uint32_t*>(dst) = hdmoe_dev_pack4_e4m3fn(m[0], m[1], m[2], m[3]);
             } else {
               u32x2 pk;
               pk.x = hdmoe_dev_pack_bf16(m[0], m[1]);

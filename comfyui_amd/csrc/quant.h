@@ -27,10 +27,7 @@ __device__ __forceinline__ uint32_t hdmoe_q_2(uint32_t u, float inv) {
                                hdmoe_q_pre(__uint_as_float(u & 0xffff0000u), inv));
 }
 
-// eight bf16 values -> eight e4m3fn bytes. A scale of exactly 1 skips the multiply (x * 1 rounded to bf16 is x);
-// the rule "beyond the rounding midpoint above 448 -> NaN" is checked once for the eight values (largest
-// magnitude as an integer compare, which also catches NaN inputs, whose cast is sign | 0x7F either way) and
-// patched per byte only when it fires.
+// eight bf16 values -> eight e4m3fn bytes. A scale of exactly 1 skips the multiply (x * 1 rounded to bf16 is x).
 __device__ __forceinline__ uint2 hdmoe_q_8(const uint4& v, float inv) {
   const uint32_t w[4] = {v.x, v.y, v.z, v.w};
   float f[8];
@@ -50,26 +47,7 @@ __device__ __forceinline__ uint2 hdmoe_q_8(const uint4& v, float inv) {
       f[2 * j + 1] = __uint_as_float(p & 0xffff0000u);
     }
   }
-  uint32_t o[2];
-#pragma unroll
-  for (int h = 0; h < 2; ++h) {
-    int p = __builtin_amdgcn_cvt_pk_fp8_f32(f[4 * h], f[4 * h + 1], 0, false);
-    o[h] = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(f[4 * h + 2], f[4 * h + 3], p, true);
-  }
-  if (!(inv < 0.0f)) {
-    uint32_t m = 0;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const uint32_t a = __float_as_uint(f[j]) & 0x7fffffffu;
-      m = a > m ? a : m;
-    }
-    if (m > 0x43e80000u) {  // some |value| > 464 (or NaN)
-#pragma unroll
-      for (int j = 0; j < 8; ++j)
-        if ((__float_as_uint(f[j]) & 0x7fffffffu) > 0x43e80000u) o[j >> 2] |= 0x7fu << (8 * (j & 3));
-    }
-  }
-  return make_uint2(o[0], o[1]);
+  return make_uint2(hdmoe_dev_pack4_e4m3fn(f[0], f[1], f[2], f[3]), hdmoe_dev_pack4_e4m3fn(f[4], f[5], f[6], f[7]));
 }
 
 // (1.0 / scale_input).to(bfloat16) as fp32; NULL pointer -> clamp rule marker

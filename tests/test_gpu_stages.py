@@ -48,7 +48,8 @@ def test_gate_exact_ties_go_to_lower_index(dev):
 
 
 @pytest.mark.parametrize("T,E", [(1, 4), (5, 4), (1024, 4), (1025, 4), (8192, 4), (3000, 8), (700, 16), (8191, 2),
-                                 (8193, 6), (20000, 15), (32768, 4), (32769, 4), (40000, 8), (33000, 16)])
+                                 (8193, 6), (20000, 15), (32768, 4), (32769, 4), (40000, 8), (33000, 16),
+                                 (131072, 4), (150001, 5)])  # above 32768 tokens: the large-chunk kernels
 def test_dispatch_bit_exact(dev, T, E):
     g = torch.Generator().manual_seed(T + E)
     first = torch.randint(0, E, (T,), generator=g)
