@@ -87,6 +87,7 @@ struct GemmArgs {
   const int32_t* offsets;  // segment bounds of the dynamic groups, n_offsets + 1 entries
   int n_offsets;
   int G;
+  int spread;  // 0: one tile list cut in eighths; 1 / -1: every group cut in eighths, groups walked up / down
 };
 
 __device__ __forceinline__ int swz(int row) { return ((row >> 1) & 7) ^ ((row & 1) << 2); }
@@ -140,19 +141,37 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
   struct Tile { int g, row0, rows_here, n0, kbytes; };
   auto decode = [&](int i) -> Tile {
     Tile d = {-1, 0, 0, 0, 0};
-    const int in_xcd = slot + i * nslots;
-    int L = xcd * per_xcd + in_xcd;
-    if (in_xcd >= per_xcd || L >= total) return d;
-    int g = 0, rb = 0, re = 0, mtiles = 0, ntiles = 0;
-    for (; g < args.G; ++g) {
-      seg(args.g[g], rb, re);
-      mtiles = (re - rb + BM - 1) / BM;
-      ntiles = args.g[g].n_out / FEAT_PER_TILE;
-      const int tiles = mtiles * ntiles;
-      if (L < tiles) break;
-      L -= tiles;
+    int in_xcd = slot + i * nslots;
+    int L = 0, g = 0, rb = 0, re = 0, mtiles = 0, ntiles = 0;
+    if (args.spread != 0) {
+      // Groups whose tiles differ in length (the K of the shared expert's down projection is about half the
+      // routed experts'): every XCD takes its eighth of every group, longest tiles first, so each block gets
+      // the same mix and the blocks end together.
+      int k = 0;
+      for (; k < args.G; ++k) {
+        g = args.spread > 0 ? k : args.G - 1 - k;
+        seg(args.g[g], rb, re);
+        mtiles = (re - rb + BM - 1) / BM;
+        ntiles = args.g[g].n_out / FEAT_PER_TILE;
+        const long long tiles = (long long)mtiles * ntiles;
+        const int lo = (int)(xcd * tiles / HDMOE_NUM_XCD), hi = (int)((xcd + 1) * tiles / HDMOE_NUM_XCD);
+        if (in_xcd < hi - lo) { L = lo + in_xcd; break; }
+        in_xcd -= hi - lo;
+      }
+      if (k >= args.G) return d;
+    } else {
+      L = xcd * per_xcd + in_xcd;
+      if (in_xcd >= per_xcd || L >= total) return d;
+      for (; g < args.G; ++g) {
+        seg(args.g[g], rb, re);
+        mtiles = (re - rb + BM - 1) / BM;
+        ntiles = args.g[g].n_out / FEAT_PER_TILE;
+        const int tiles = mtiles * ntiles;
+        if (L < tiles) break;
+        L -= tiles;
+      }
+      if (g >= args.G) return d;
     }
-    if (g >= args.G) return d;
     // bands of GROUP_M m-tiles; a short remainder joins the last band, so that the cheap partial m-tile at the
     // end of a segment is interleaved with full ones instead of forming a run of its own
     const int nbands = max(1, (mtiles + GROUP_M / 2) / GROUP_M);
@@ -648,6 +667,8 @@ int hdmoe_launch_ffn_gemm(bool swiglu, int weight_dtype, const uint8_t* a_dyn, c
     ++G;
   }
   args.G = G;
+  // tiles of the static group are shorter or longer than the experts' when the two K differ (down projection)
+  if (n_dyn > 0 && shared != nullptr && rows_static > 0 && K_static != K_dyn) args.spread = K_static < K_dyn ? 1 : -1;
   if (fp8 && tall) return swiglu ? launch_grouped<FP8_SWIGLU, 5>(args, tile_bound, s, what)
                                  : launch_grouped<FP8_PLAIN, 5>(args, tile_bound, s, what);
   if (fp8) return swiglu ? launch_grouped<FP8_SWIGLU>(args, tile_bound, s, what)
