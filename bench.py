@@ -35,7 +35,7 @@ PEAK_HBM_GBPS = 8000.0      # MI355X HBM3E
 # L2-side traffic of the dominant kernel per launch (bytes fetched + written), from the two rocprofv3 --pmc runs
 # summarised in profiles/bench_cfg3_pmc.txt (FETCH_SIZE x 2.000 and WRITE_SIZE x 1.000 after calibration against a
 # plain 256 MiB copy). Only known for the workload that was profiled.
-MEASURED_TRAFFIC_BYTES = {"cfg3": 1088.7e6 + 145.8e6}
+MEASURED_TRAFFIC_BYTES = {"cfg3": 1084.5e6 + 145.8e6}
 
 
 class HipEvents:
