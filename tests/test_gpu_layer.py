@@ -68,6 +68,35 @@ def test_small_layers(dev, weights, dim, tokens, batch):
     check_layer(sd, x, weights, y, idx, w, 4)
 
 
+@pytest.mark.parametrize("weights", ["fp8", "bf16"])
+def test_shared_expert_wider_than_the_routed_ones(dev, weights):
+    """The down GEMM hands out its tiles group by group when the groups' K differ, longest tiles first; here the
+    shared expert is the long one (hidden 3072 vs 1536), the opposite of HiDream's shapes."""
+    from comfyui_amd import hidream, ops
+    from comfyui_amd import functional as HF
+    dim, E, T = 512, 4, 900
+    g = torch.Generator().manual_seed(77)
+    master = {}
+    for prefix, h in [("shared_experts.", 3072)] + [(f"experts.{e}.", 1536) for e in range(E)]:
+        master[prefix + "w1.weight"] = torch.randn((h, dim), generator=g) * 0.02
+        master[prefix + "w2.weight"] = torch.randn((dim, h), generator=g) * 0.02
+        master[prefix + "w3.weight"] = torch.randn((h, dim), generator=g) * 0.02
+    master["gate.weight"] = torch.randn((E, dim), generator=g) / dim ** 0.5
+    sd = synth.to_state_dict(master, weights)
+    x = synth.make_input(g, T, dim=dim)
+    operations = (ops.disable_weight_init if weights == "bf16"
+                  else ops.scaled_fp8_ops(fp8_matrix_mult=True, scale_input=True, override_dtype=torch.float8_e4m3fn))
+    m = hidream.MOEFeedForwardSwiGLU(dim, 4 * dim, E, 2, dtype=BF16, device=dev, operations=operations)
+    m.shared_experts = hidream.FeedForwardSwiGLU(dim, 4608, dtype=BF16, device=dev, operations=operations)
+    assert m.shared_experts.w1.weight.shape[0] == 3072 and m.experts[0].w1.weight.shape[0] == 1536
+    m.load_state_dict({k: v.to(dev) for k, v in sd.items()}, strict=False)
+    xd = x.to(dev)
+    y = m.eval()(xd)
+    idx, w = HF.gate_top2(xd.reshape(-1, dim), m.gate.weight.to(BF16))
+    torch.cuda.synchronize()
+    check_layer(sd, x, weights, y.cpu(), idx.cpu(), w.cpu(), E)
+
+
 def test_fp8_nontrivial_scale_inputs(dev):
     # per-Linear scale_input values: w1/w3 of an expert share one, experts differ
     dim = 512
