@@ -183,3 +183,47 @@ def test_silu_mul(dev):
     diff = (got.float() - want.float()).abs()
     assert bool((diff <= want.float().abs() * 2 ** -6 + 1e-30).all())
     assert float((got.view(torch.int16) != want.view(torch.int16)).float().mean()) < 0.01
+
+
+@pytest.mark.parametrize("rows,next_scale", [(300, 1.0), (333, 0.5), (64, None)])
+def test_swiglu_epilogue_cast_overflows_to_nan_like_torch(dev, rows, next_scale):
+    """The gate/up GEMM casts silu(w1 x) * w3 x to e4m3fn for the w2 Linear (ops.py:337-343): beyond the rounding
+    midpoint above 448 the reference's cast gives NaN (no saturation), with scale_input None it clamps first.
+    Integer-valued operands and power-of-two scales make the fp32 sums exact in any order, so the only freedom left
+    is the last bit of silu: values agree within one e4m3 step and NaN positions agree away from the threshold."""
+    from comfyui_amd import functional as HF
+    D, H = 128, 256
+    g = torch.Generator().manual_seed(rows)
+    a = torch.randint(-3, 4, (rows, D), generator=g).float()
+    w1 = torch.randint(-3, 4, (H, D), generator=g).float()
+    w3 = torch.randint(-3, 4, (H, D), generator=g).float()
+    one = torch.ones((), dtype=torch.float32)
+    s1, s3 = torch.tensor(0.5), torch.tensor(1.0)
+    sn = None if next_scale is None else torch.tensor(float(next_scale))
+    scales = dict(scale_w1=s1.to(dev), scale_w3=s3.to(dev), scale_in1=one.to(dev))
+    if sn is not None:
+        scales["scale_in2"] = sn.to(dev)
+    w1d, w3d = w1.to(FP8).to(dev), w3.to(FP8).to(dev)
+    fw = HF.make_ffn_weights(w1d, w1d, w3d, scales)      # w2 is not read by this stage
+    offsets = torch.tensor([0, rows], dtype=torch.int32, device=dev)
+    h = HF.grouped_swiglu(a.to(FP8).to(dev), offsets, [fw], H).cpu()
+    h1 = ((a @ w1.t()) * s1).to(BF16)
+    h3 = ((a @ w3.t()) * s3).to(BF16)
+    m = torch.nn.functional.silu(h1) * h3                  # bf16 tensors: each op rounds to bf16
+    if sn is None:
+        pre = torch.clamp(m, min=-448, max=448)
+    else:
+        pre = m * (1.0 / sn).to(BF16)
+    want = pre.to(FP8)
+    got_f, want_f = h.float(), want.float()
+    if sn is not None:
+        assert int(want_f.isnan().sum()) > 1000                        # the overflow case is exercised
+    else:
+        assert int((m.float().abs() > 464).sum()) > 1000               # the clamp has something to do
+        assert not bool(got_f.isnan().any()) and float(got_f.abs().max()) == 448.0
+    near = (pre.float().abs() > 440) & (pre.float().abs() < 490)      # one bf16 step around 464 decides NaN or 448
+    assert torch.equal(got_f.isnan() & ~near, want_f.isnan() & ~near)
+    ok = ~got_f.isnan() & ~want_f.isnan()
+    step = torch.maximum(want_f.abs(), torch.tensor(2.0 ** -6)) * 2.0 ** -3 * 1.001   # one e4m3 step at that magnitude
+    assert bool(((got_f - want_f).abs()[ok] <= step[ok]).all())
+    assert float((got_f[ok] == want_f[ok]).float().mean()) > 0.99
