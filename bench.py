@@ -142,8 +142,8 @@ def aux_kernels(dev, module, x):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="cfg3", choices=["cfg1", "cfg2", "cfg3", "cfg5-256", "cfg5-4096", "cfg3-branch", "cfg4"])
     ap.add_argument("--layers", type=int, default=48, help="cfg4 only: number of stacked layers")
     ap.add_argument("--cpu-sample-tokens", type=int, default=8192)
