@@ -83,6 +83,8 @@ SIGNATURES = {
     "hdmoe_grouped_down": (c_int, [c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                                    ctypes.POINTER(FfnWeights), c_void_p, c_void_p]),
     "hdmoe_linear": (c_int, [c_int, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "hdmoe_linear_bias": (c_int, [c_int, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                  c_void_p]),
     "hdmoe_silu_mul_bf16": (c_int, [c_void_p, c_void_p, c_int64, c_void_p, c_void_p]),
     "hdmoe_scale_to_bf16": (c_int, [c_int, c_void_p, c_int64, c_void_p, c_void_p, c_void_p]),
     "hdmoe_grouped_linear": (c_int, [c_void_p, c_void_p, c_int, c_int, ctypes.POINTER(LinearWeights), c_void_p, c_void_p,

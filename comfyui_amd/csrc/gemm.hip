@@ -60,7 +60,7 @@ constexpr int GROUP_M = 4;     // m-tiles per raster band
 constexpr int NTHREADS = 512;
 constexpr int MAX_GROUPS = HDMOE_MAX_EXPERTS + 1;
 
-enum Mode { FP8_SWIGLU = 0, FP8_PLAIN = 1, BF16_SWIGLU = 2, BF16_PLAIN = 3, BF16_PLAIN_BIAS = 4 };
+enum Mode { FP8_SWIGLU = 0, FP8_PLAIN = 1, BF16_SWIGLU = 2, BF16_PLAIN = 3, BF16_PLAIN_BIAS = 4, FP8_PLAIN_BIAS = 5 };
 
 struct GemmGroup {
   const uint8_t* a;     // activations; row indices below are relative to this base
@@ -102,9 +102,9 @@ typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
 template <int MODE, int TT>
 __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs args) {
-  constexpr bool FP8 = (MODE == FP8_SWIGLU || MODE == FP8_PLAIN);
+  constexpr bool FP8 = (MODE == FP8_SWIGLU || MODE == FP8_PLAIN || MODE == FP8_PLAIN_BIAS);
   constexpr bool SWIGLU = (MODE == FP8_SWIGLU || MODE == BF16_SWIGLU);
-  constexpr bool BIAS = (MODE == BF16_PLAIN_BIAS);  // Linear with bias and optional GELU (bf16 weights)
+  constexpr bool BIAS = (MODE == BF16_PLAIN_BIAS || MODE == FP8_PLAIN_BIAS);  // Linear with bias and optional GELU
   constexpr int WAVE_TOK = 32 * TT;        // tokens per wave row
   constexpr int BM = 2 * WAVE_TOK;         // tokens per block tile
   constexpr int A_SLABS = BM / 64;         // 64-row slabs of the token tile
@@ -476,12 +476,23 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
             u32x2 pk;
             if constexpr (BIAS) {
               // F.linear with bias: bf16(acc + bias); then F.gelu (erf form) of that bf16 tensor, rounded again
-              // (/root/reference/comfy/ldm/hunyuan3dv2_1/hunyuandit.py:14-26, 44-50)
+              // (/root/reference/comfy/ldm/hunyuan3dv2_1/hunyuandit.py:14-26, 44-50). fp8: the scaled-mm epilogue
+              // bf16(acc * scale_input * scale_weight + bias) of fp8_linear (/root/reference/comfy/ops.py:345-346).
               const u32x2 bq = ep_bias[ft][q];
-              float v[4] = {acc[ft][tt][q * 4 + 0] + __uint_as_float(bq.x << 16),
-                            acc[ft][tt][q * 4 + 1] + __uint_as_float(bq.x & 0xffff0000u),
-                            acc[ft][tt][q * 4 + 2] + __uint_as_float(bq.y << 16),
-                            acc[ft][tt][q * 4 + 3] + __uint_as_float(bq.y & 0xffff0000u)};
+              float v[4] = {acc[ft][tt][q * 4 + 0], acc[ft][tt][q * 4 + 1], acc[ft][tt][q * 4 + 2], acc[ft][tt][q * 4 + 3]};
+              {
+                // product rounded to fp32 before the bias is added (no fused multiply-add), the order the CPU
+                // checker and torch's own scaled matrix multiply on the CPU use
+#pragma clang fp contract(off)
+                if constexpr (FP8) {
+#pragma unroll
+                  for (int i = 0; i < 4; ++i) v[i] = v[i] * sc;
+                }
+                v[0] = v[0] + __uint_as_float(bq.x << 16);
+                v[1] = v[1] + __uint_as_float(bq.x & 0xffff0000u);
+                v[2] = v[2] + __uint_as_float(bq.y << 16);
+                v[3] = v[3] + __uint_as_float(bq.y & 0xffff0000u);
+              }
               if (gg.act == 1) {
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
@@ -721,6 +732,31 @@ int hdmoe_launch_linear_groups(const uint8_t* a_dyn, const int32_t* offsets, int
   return launch_grouped<BF16_PLAIN_BIAS>(args, tile_bound, s, what);
 }
 
+// One Linear with an optional bias over all rows of `a` (either weight type): a single static group.
+int hdmoe_launch_linear_bias(int weight_dtype, const uint8_t* a, int rows, int K, int N, const uint8_t* w,
+                             const float* scale_w, const float* scale_in, const uint16_t* bias, uint8_t* out,
+                             hipStream_t s, const char* what) {
+  const bool fp8 = weight_dtype == HDMOE_W_E4M3FN;
+  GemmArgs args;
+  memset(&args, 0, sizeof(args));
+  GemmGroup& gg = args.g[0];
+  gg.a = a;
+  gg.out = out;
+  gg.row_begin = 0;
+  gg.row_end = rows;
+  gg.n_out = N;
+  gg.kbytes = K * elem_bytes(weight_dtype);
+  gg.b0 = w;
+  gg.sb0 = scale_w;
+  gg.s_in = scale_in;
+  gg.bias = bias;
+  gg.act = HDMOE_ACT_NONE;
+  args.G = 1;
+  const int tile_bound = ((rows + TileCfg<4>::BM - 1) / TileCfg<4>::BM) * (N / BN);
+  return fp8 ? launch_grouped<FP8_PLAIN_BIAS>(args, tile_bound, s, what)
+             : launch_grouped<BF16_PLAIN_BIAS>(args, tile_bound, s, what);
+}
+
 // Size rules shared by the entry points: K bytes per row must be a multiple of the
 // 128-byte K step; total bytes of each operand must fit the 32-bit buffer range.
 int hdmoe_check_gemm_shape(const char* what, int weight_dtype, long rows, int K, int N, int feat_per_tile) {
@@ -779,6 +815,23 @@ extern "C" int hdmoe_linear(int weight_dtype, const void* a, int rows, int K, in
   return hdmoe_launch_ffn_gemm(false, weight_dtype, nullptr, nullptr, 0, 0, nullptr, nullptr,
                                static_cast<const uint8_t*>(a), rows, &fw, static_cast<uint8_t*>(out_bf16), 0, 0, K, N,
                                static_cast<hipStream_t>(stream), "hdmoe_linear");
+}
+
+extern "C" int hdmoe_linear_bias(int weight_dtype, const void* a, int rows, int K, int N, const void* w,
+                                 const float* scale_w_dev, const float* scale_in_dev, const void* bias_bf16,
+                                 void* out_bf16, hdmoe_stream_t stream) {
+  if (bias_bf16 == nullptr)
+    return hdmoe_linear(weight_dtype, a, rows, K, N, w, scale_w_dev, scale_in_dev, out_bf16, stream);
+  HDMOE_REQUIRE_PTR(a);
+  HDMOE_REQUIRE_PTR(w);
+  HDMOE_REQUIRE_PTR(out_bf16);
+  if (int rc = hdmoe_check_gemm_shape("hdmoe_linear_bias", weight_dtype, rows, K, N, BN)) return rc;
+  if (weight_dtype == HDMOE_W_E4M3FN) HDMOE_REQUIRE_PTR(scale_w_dev);
+  if (rows == 0) return HDMOE_OK;
+  return hdmoe_launch_linear_bias(weight_dtype, static_cast<const uint8_t*>(a), rows, K, N,
+                                  static_cast<const uint8_t*>(w), scale_w_dev, scale_in_dev,
+                                  static_cast<const uint16_t*>(bias_bf16), static_cast<uint8_t*>(out_bf16),
+                                  static_cast<hipStream_t>(stream), "hdmoe_linear_bias");
 }
 
 extern "C" int hdmoe_grouped_linear(const void* a_bf16, const int32_t* offsets, int rows_total, int E,

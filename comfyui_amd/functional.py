@@ -104,8 +104,9 @@ def permute_bf16(x2d, perm):
     return out
 
 
-def linear(a2d, weight, scale_weight=None, scale_input=None):
-    """a2d [rows,K] (fp8 for fp8 weights, bf16 for bf16 weights) x weight [N,K]^T -> bf16 [rows,N]."""
+def linear(a2d, weight, scale_weight=None, scale_input=None, bias=None):
+    """a2d [rows,K] (fp8 for fp8 weights, bf16 for bf16 weights) x weight [N,K]^T (+ bias [N] bf16) -> bf16 [rows,N];
+    the bias joins the fp32 result before the one rounding."""
     code = weight_dtype_code(weight.dtype)
     _need_hip(a2d, "linear activations", weight.dtype)
     _need_hip(weight, "linear weight")
@@ -113,10 +114,14 @@ def linear(a2d, weight, scale_weight=None, scale_input=None):
     N = weight.shape[0]
     if weight.shape[1] != K:
         raise ValueError(f"linear: activations [{rows},{K}] do not match weight {tuple(weight.shape)}")
+    if bias is not None:
+        _need_hip(bias, "linear bias", BF16)
+        if bias.shape != (N,) or not bias.is_contiguous():
+            raise ValueError(f"linear: bias {tuple(bias.shape)} does not match {N} output features")
     out = torch.empty((rows, N), dtype=BF16, device=a2d.device)
-    check(lib.hdmoe_linear(code, ptr(a2d), rows, K, N, ptr(weight),
-                           _scale_ptr(scale_weight, a2d.device, "scale_weight"),
-                           _scale_ptr(scale_input, a2d.device, "scale_input"), ptr(out), _stream(a2d)))
+    check(lib.hdmoe_linear_bias(code, ptr(a2d), rows, K, N, ptr(weight),
+                                _scale_ptr(scale_weight, a2d.device, "scale_weight"),
+                                _scale_ptr(scale_input, a2d.device, "scale_input"), ptr(bias), ptr(out), _stream(a2d)))
     return out
 
 

@@ -110,11 +110,8 @@ class CastWeightBiasOp:
 def _linear_bf16(input, weight, bias):
     shape = input.shape
     x2 = input.reshape(-1, shape[-1]).contiguous()
-    if bias is not None:
-        # the bias is added to the fp32 accumulator before the one rounding to bf16, like F.linear's fused epilogue
-        _, out = HF.grouped_linear(x2[:0], None, [], a_static=x2, shared=(weight.contiguous(), bias.contiguous()))
-    else:
-        out = HF.linear(x2, weight.contiguous())
+    # a bias is added to the fp32 accumulator before the one rounding to bf16, like F.linear's fused epilogue
+    out = HF.linear(x2, weight.contiguous(), bias=None if bias is None else bias.contiguous())
     return out.reshape(*shape[:-1], weight.shape[0])
 
 
@@ -161,8 +158,6 @@ def fp8_linear(self, input):
     if input.dtype != BF16:
         raise TypeError(f"fp8_linear on the HIP path takes bfloat16 activations, got {input.dtype}")
     weight, bias = cast_bias_weight(self, input, dtype=FP8, bias_dtype=input.dtype)
-    if bias is not None:
-        raise NotImplementedError("comfyui_amd fp8_linear: bias is not part of the MoE feed-forward path")
     dev = input.device
     scale_weight = self.scale_weight
     scale_weight = _one(dev) if scale_weight is None else scale_weight.to(dev)
@@ -171,7 +166,8 @@ def fp8_linear(self, input):
         scale_input = scale_input.to(dev)
     x2 = input.reshape(-1, input.shape[-1]).contiguous()
     xq = HF.quant_fp8(x2, scale_input)
-    out = HF.linear(xq, weight.contiguous(), scale_weight, scale_input)
+    out = HF.linear(xq, weight.contiguous(), scale_weight, scale_input,
+                    bias=None if bias is None else bias.contiguous())
     return out.reshape(*input.shape[:-1], weight.shape[0])
 
 

@@ -33,7 +33,7 @@
 extern "C" {
 #endif
 
-#define HDMOE_VERSION 104
+#define HDMOE_VERSION 105
 
 #define HDMOE_OK 0
 #define HDMOE_E_NULL (-1)      /* required pointer is NULL */
@@ -134,6 +134,15 @@ int hdmoe_grouped_down(int weight_dtype, const void* h, const int32_t* offsets, 
 int hdmoe_linear(int weight_dtype, const void* a, int rows, int K, int N, const void* w,
                  const float* scale_w_dev, const float* scale_in_dev, void* out_bf16,
                  hdmoe_stream_t stream);
+
+/* The same Linear with a bias (bias_bf16 [N]; NULL = hdmoe_linear): the bias joins the fp32 result before the one
+ * rounding, as F.linear does (ops.py:107-115) and as the scaled matrix multiply of fp8_linear does with its bias
+ * argument (ops.py:345-346):
+ *   fp8:  out = bf16( (a_fp8 . w_fp8^T) * scale_in * scale_w + bias )
+ *   bf16: out = bf16( a_bf16 . w_bf16^T + bias ) */
+int hdmoe_linear_bias(int weight_dtype, const void* a, int rows, int K, int N, const void* w,
+                      const float* scale_w_dev, const float* scale_in_dev, const void* bias_bf16,
+                      void* out_bf16, hdmoe_stream_t stream);
 
 /* Elementwise middle of model.py:238 for the unfused path: out = bf16(bf16(silu(a)) * b). */
 int hdmoe_silu_mul_bf16(const void* a_bf16, const void* b_bf16, int64_t n, void* out_bf16,

@@ -158,13 +158,14 @@ def combine_c(y_sorted_bf16, inv_perm, w_bf16, shared_bf16):
 # ------------------------------------------------------------------------ linear
 
 class LinearParams:
-    """One reference Linear without bias: weight [out,in] (bf16/fp32, or float8_e4m3fn with
-    scale_weight and optional scale_input fp32 scalars, ops.py:388-397)."""
+    """One reference Linear: weight [out,in] (bf16/fp32, or float8_e4m3fn with scale_weight and optional
+    scale_input fp32 scalars, ops.py:388-397) and an optional bias [out]."""
 
-    def __init__(self, weight, scale_weight=None, scale_input=None):
+    def __init__(self, weight, scale_weight=None, scale_input=None, bias=None):
         self.weight = weight
         self.scale_weight = scale_weight
         self.scale_input = scale_input
+        self.bias = bias
 
 
 def oracle_params(state_dict, num_experts):
@@ -186,15 +187,22 @@ def linear(x, p, mode):
     mode "fp8mm":  fp8_linear (ops.py:314-358): quantise x (x * (1/scale_input).to(x.dtype) -> e4m3fn,
                    or clamp +-448 when scale_input is None), fp8 x fp8 products accumulated in fp32,
                    times scale_input*scale_weight, rounded to x.dtype. Products of two e4m3 values are
-                   exact in fp32, so an fp32 matmul of the decoded operands is the same contraction."""
+                   exact in fp32, so an fp32 matmul of the decoded operands is the same contraction.
+                   A bias (cast to x.dtype, ops.py:329) goes into the scaled matrix multiply (ops.py:345-346),
+                   which adds it to the scaled fp32 result before the one rounding (checked against
+                   torch._scaled_mm itself in the tests).
+    Modes "plain" and "upcast" with a bias: F.linear's own bias argument."""
+    bias = getattr(p, "bias", None)
+    if bias is not None:
+        bias = bias.to(x.dtype)
     if mode == "plain":
-        return F.linear(x, p.weight.to(x.dtype), None)
+        return F.linear(x, p.weight.to(x.dtype), bias)
     if mode == "upcast":
         w = p.weight.to(x.dtype)
         s = p.scale_weight.to(x.dtype)
         if w.numel() < x.numel():
-            return F.linear(x, w * s, None)
-        return F.linear(x * s, w, None)
+            return F.linear(x, w * s, bias)
+        return F.linear(x * s, w, bias)
     if mode == "fp8mm":
         assert p.weight.dtype == torch.float8_e4m3fn
         if p.scale_input is None:
@@ -204,7 +212,10 @@ def linear(x, p, mode):
             s_in = p.scale_input.to(torch.float32)
             xq = (x * (1.0 / s_in).to(x.dtype)).to(torch.float8_e4m3fn)
         acc = xq.to(torch.float32) @ p.weight.to(torch.float32).t()
-        return (acc * (s_in * p.scale_weight.to(torch.float32))).to(x.dtype)
+        acc = acc * (s_in * p.scale_weight.to(torch.float32))
+        if bias is not None:
+            acc = acc + bias.to(torch.float32)
+        return acc.to(x.dtype)
     raise ValueError(mode)
 
 

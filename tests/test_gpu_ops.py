@@ -72,6 +72,41 @@ def test_linear_with_bias(dev):
         assert float((y.cpu().float() - ref.float()).abs().max()) <= 2.0 ** -5
 
 
+@pytest.mark.parametrize("s_in", [1.0, 0.37, None])
+def test_fp8_linear_with_bias(dev, s_in):
+    """fp8_linear with a bias (ops.py:329, 345-346), as the attention projections of a scaled-fp8 checkpoint have."""
+    from comfyui_amd import ops
+    cls = ops.scaled_fp8_ops(fp8_matrix_mult=True, scale_input=s_in is not None, override_dtype=FP8)
+    K, N = 256, 512
+    g = torch.Generator().manual_seed(11)
+    w8, sw = synth.quantize_per_tensor(torch.randn((N, K), generator=g) * 0.02)
+    lin = cls.Linear(K, N, bias=True, dtype=BF16, device=dev)
+    assert lin.bias.dtype == FP8          # the class stores every parameter in the override dtype (ops.py:383-386)
+    bias = torch.randn((N,), generator=g).to(FP8).to(BF16)     # what such a parameter can hold, cast as ops.py:329 does
+    lin.weight = torch.nn.Parameter(w8.to(dev), requires_grad=False)
+    with torch.no_grad():
+        lin.bias.copy_(bias)
+        lin.scale_weight.copy_(sw)
+        if s_in is not None:
+            lin.scale_input.fill_(s_in)
+    x = torch.randn((3, 50, K), generator=g).to(BF16)
+    ref = O.linear(x, O.LinearParams(w8, sw, None if s_in is None else torch.tensor(s_in), bias), "fp8mm")
+    xd = x.to(dev)
+    y = lin(xd)
+    assert torch.equal(xd.cpu(), x)                      # the caller's tensor is not clamped in place
+    assert y.shape == (3, 50, N) and y.dtype == BF16
+    close(y.cpu(), ref, 3e-3)
+    # integer-valued operands make the fp32 sums exact in any order: bit-exact, bias placement included
+    xi = torch.randint(-4, 5, (2, 33, K), generator=g).to(BF16)
+    wi = torch.randint(-4, 5, (N, K), generator=g).float()
+    lin.weight = torch.nn.Parameter(wi.to(FP8).to(dev), requires_grad=False)
+    with torch.no_grad():
+        lin.scale_weight.fill_(0.3)
+    ref_i = O.linear(xi, O.LinearParams(wi.to(FP8), torch.tensor(0.3), None if s_in is None else torch.tensor(s_in), bias),
+                     "fp8mm")
+    assert torch.equal(lin(xi.to(dev)).cpu().view(torch.int16), ref_i.view(torch.int16))
+
+
 def test_scaled_fp8_linear_with_fp8_matmul(dev):
     from comfyui_amd import ops
     cls = ops.scaled_fp8_ops(fp8_matrix_mult=True, scale_input=True, override_dtype=FP8)

@@ -32,6 +32,27 @@ def test_fp8mm_linear_equals_torch_scaled_mm():
     assert float(O.linear(x1, p, "fp8mm")[0, 0]) == (1.5 * 0.5 - 2.0 * 0.25) * 2.0
 
 
+def test_fp8mm_linear_with_bias_equals_torch_scaled_mm():
+    """The bias of fp8_linear goes into the scaled matrix multiply (ops.py:345-346): torch's own CPU kernel adds it
+    to the scaled fp32 result before the one rounding; rounding the product first would differ on ~30 % of outputs."""
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn((40, 128), generator=g).to(BF16)
+    w8, sw = O.quantize_weight_per_tensor(torch.randn((64, 128), generator=g) * 0.05)
+    bias = (torch.randn((64,), generator=g) * 3).to(BF16)
+    si = torch.tensor(0.37, dtype=torch.float32)
+    got = O.linear(x, O.LinearParams(w8, sw, si, bias), "fp8mm")
+    xq = (x * (1.0 / si).to(BF16)).to(FP8)
+    try:
+        ref = torch._scaled_mm(xq, w8.t(), out_dtype=BF16, bias=bias, scale_a=si, scale_b=sw)
+    except Exception as e:
+        pytest.skip(f"torch._scaled_mm unavailable on CPU: {e}")
+    assert torch.equal(got.view(torch.int16), ref.view(torch.int16))
+    rounded_first = (O.linear(x, O.LinearParams(w8, sw, si), "fp8mm") + bias).to(BF16)
+    assert float((rounded_first != ref).float().mean()) > 0.05      # the other order is distinguishable
+    no_bias = O.linear(x, O.LinearParams(w8, sw, si), "fp8mm")
+    assert not torch.equal(no_bias, got)                              # a dropped bias is detected
+
+
 def test_fp8mm_without_scale_input_clamps():
     x = torch.tensor([[1000.0, -1000.0, 3.0, 0.0] + [0.0] * 12], dtype=BF16)
     w = torch.zeros((16, 16)); w[0, 0] = w[0, 1] = w[0, 2] = 1.0
