@@ -123,6 +123,61 @@ __device__ __forceinline__ void finish_token(float (&logit)[E], int lane, int t,
   }
 }
 
+__device__ __forceinline__ void unpack8(const uint4& a, float (&f)[8]) {
+  f[0] = bf16_lo(a.x); f[1] = bf16_hi(a.x); f[2] = bf16_lo(a.y); f[3] = bf16_hi(a.y);
+  f[4] = bf16_lo(a.z); f[5] = bf16_hi(a.z); f[6] = bf16_lo(a.w); f[7] = bf16_hi(a.w);
+}
+
+__device__ __forceinline__ void round2(float& a, float& b) {
+  const uint32_t p = hdmoe_dev_pack_bf16(a, b);
+  a = __uint_as_float(p << 16);
+  b = __uint_as_float(p & 0xffff0000u);
+}
+
+__device__ __forceinline__ uint4 modulate8(const uint4& xv, const uint4& sc, const uint4& sh, float mean, float rstd) {
+  float x[8], a[8], b[8];
+  unpack8(xv, x);
+  unpack8(sc, a);
+  unpack8(sh, b);
+  uint32_t o[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    // two elements at a time: one packed conversion (v_cvt_pk_bf16_f32, round to nearest even) per rounding point
+    float n0 = (x[2 * j] - mean) * rstd, n1 = (x[2 * j + 1] - mean) * rstd;  // LayerNorm output as a bf16 tensor
+    round2(n0, n1);
+    float m0 = 1.0f + a[2 * j], m1 = 1.0f + a[2 * j + 1];                    // (1 + scale)
+    round2(m0, m1);
+    float p0 = n0 * m0, p1 = n1 * m1;                                        // n * (1 + scale)
+    round2(p0, p1);
+    o[j] = hdmoe_dev_pack_bf16(p0 + b[2 * j], p1 + b[2 * j + 1]);            // + shift
+  }
+  return make_uint4(o[0], o[1], o[2], o[3]);
+}
+
+// LayerNorm statistics of a row held in registers (NCHUNK x 8 elements per lane): the two passes and the fixed
+// fp32 order documented at the LayerNorm kernel below.
+template <int NCHUNK>
+__device__ __forceinline__ void ln_stats(const uint4 (&v)[NCHUNK], float fD, float eps, float& mean, float& rstd) {
+  float s = 0.0f;
+#pragma unroll
+  for (int c = 0; c < NCHUNK; ++c) {
+    float f[8];
+    unpack8(v[c], f);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) s = s + f[j];
+  }
+  mean = __fdiv_rn(wave_sum(s), fD);
+  float s2 = 0.0f;
+#pragma unroll
+  for (int c = 0; c < NCHUNK; ++c) {
+    float f[8];
+    unpack8(v[c], f);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) { const float d = f[j] - mean; s2 = __builtin_fmaf(d, d, s2); }
+  }
+  rstd = __fdiv_rn(1.0f, __builtin_sqrtf(__fdiv_rn(wave_sum(s2), fD) + eps));
+}
+
 // D == NCHUNK * 512: the lane's Wg slice lives in registers.
 // Optional second output of both kernels (QUANT): the token's fp8 rows for the expert GEMMs, cast while the row
 // is at hand. Row 2t+s of xq_routed is x[t] cast with the scale_input of the expert in slot s, row t of xq_shared
@@ -132,10 +187,16 @@ struct GateQuant {
   const float* shared_scale;
   uint2* xq_routed;           // [2T, D] e4m3fn
   uint2* xq_shared;           // [T, D] e4m3fn or NULL
+  // LN variant of the register kernel: the row is LayerNorm(x) * (1 + scale[b]) + shift[b] (as ln_modulate_kernel
+  // computes it, bit for bit), b = token / tokens_per_batch; the normalised tokens are never written as bf16
+  const uint4* mod_scale;     // [batch, D] bf16
+  const uint4* mod_shift;
+  int tokens_per_batch;
+  float ln_eps;
 };
 
-template <int E, int NCHUNK, bool QUANT>
-__global__ __launch_bounds__(WAVES_PER_BLOCK * 64) void gate_top2_reg_kernel(
+template <int E, int NCHUNK, bool QUANT, bool LN = false>
+__global__ __launch_bounds__(WAVES_PER_BLOCK * 64, LN ? 2 : 1) void gate_top2_reg_kernel(
     const uint4* __restrict__ x, const uint4* __restrict__ wg, int T, int32_t* __restrict__ idx,
     uint16_t* __restrict__ wout, GateQuant q) {
   const int lane = threadIdx.x & 63;
@@ -166,6 +227,14 @@ __global__ __launch_bounds__(WAVES_PER_BLOCK * 64) void gate_top2_reg_kernel(
     if (tn < T) {
 #pragma unroll
       for (int c = 0; c < NCHUNK; ++c) nxt[c] = x[(size_t)tn * ROW16 + c * 64 + lane];
+    }
+    if constexpr (LN) {
+      float mean, rstd;
+      ln_stats<NCHUNK>(cur, (float)(NCHUNK * 512), q.ln_eps, mean, rstd);
+      const size_t brow = (size_t)(t / q.tokens_per_batch) * ROW16;
+#pragma unroll
+      for (int c = 0; c < NCHUNK; ++c)
+        cur[c] = modulate8(cur[c], q.mod_scale[brow + c * 64 + lane], q.mod_shift[brow + c * 64 + lane], mean, rstd);
     }
     float logit[E];
 #pragma unroll
@@ -260,9 +329,12 @@ int launch_gate(const void* x, const void* wg, int T, int D, int32_t* idx, void*
   if (quant) q = *quant;
   constexpr int ER = E <= 4 ? E : 4;  // the register kernel is only instantiated for up to 4 experts
   if (E <= 4 && D == 2560) {
-    if (quant) hipLaunchKernelGGL((gate_top2_reg_kernel<ER, 5, true>), grid, block, 0, s, xp, wp, T, idx, wo, q);
+    if (quant && q.mod_scale != nullptr)
+      hipLaunchKernelGGL((gate_top2_reg_kernel<ER, 5, true, true>), grid, block, 0, s, xp, wp, T, idx, wo, q);
+    else if (quant) hipLaunchKernelGGL((gate_top2_reg_kernel<ER, 5, true>), grid, block, 0, s, xp, wp, T, idx, wo, q);
     else hipLaunchKernelGGL((gate_top2_reg_kernel<ER, 5, false>), grid, block, 0, s, xp, wp, T, idx, wo, q);
   } else {
+    if (q.mod_scale != nullptr) return hdmoe_fail(HDMOE_E_SHAPE, "%s: the LayerNorm variant needs D = 2560 and E <= 4", what);
     if (quant) hipLaunchKernelGGL((gate_top2_generic_kernel<E, true>), grid, block, 0, s, xp, wp, T, D, idx, wo, q);
     else hipLaunchKernelGGL((gate_top2_generic_kernel<E, false>), grid, block, 0, s, xp, wp, T, D, idx, wo, q);
   }
@@ -288,37 +360,6 @@ int dispatch_gate(const void* x_bf16, const void* gate_w_bf16, int T, int D, int
 // as the gate kernel; mean and variance are two passes over the registers with the same fixed fp32 order
 // (per-lane ascending elements, then the xor butterfly), so the CPU checker can restate it bit for bit.
 // The root is __builtin_sqrtf, which hipcc rounds correctly; __fsqrt_rn is the approximate native root here.
-__device__ __forceinline__ void unpack8(const uint4& a, float (&f)[8]) {
-  f[0] = bf16_lo(a.x); f[1] = bf16_hi(a.x); f[2] = bf16_lo(a.y); f[3] = bf16_hi(a.y);
-  f[4] = bf16_lo(a.z); f[5] = bf16_hi(a.z); f[6] = bf16_lo(a.w); f[7] = bf16_hi(a.w);
-}
-
-__device__ __forceinline__ void round2(float& a, float& b) {
-  const uint32_t p = hdmoe_dev_pack_bf16(a, b);
-  a = __uint_as_float(p << 16);
-  b = __uint_as_float(p & 0xffff0000u);
-}
-
-__device__ __forceinline__ uint4 modulate8(const uint4& xv, const uint4& sc, const uint4& sh, float mean, float rstd) {
-  float x[8], a[8], b[8];
-  unpack8(xv, x);
-  unpack8(sc, a);
-  unpack8(sh, b);
-  uint32_t o[4];
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    // two elements at a time: one packed conversion (v_cvt_pk_bf16_f32, round to nearest even) per rounding point
-    float n0 = (x[2 * j] - mean) * rstd, n1 = (x[2 * j + 1] - mean) * rstd;  // LayerNorm output as a bf16 tensor
-    round2(n0, n1);
-    float m0 = 1.0f + a[2 * j], m1 = 1.0f + a[2 * j + 1];                    // (1 + scale)
-    round2(m0, m1);
-    float p0 = n0 * m0, p1 = n1 * m1;                                        // n * (1 + scale)
-    round2(p0, p1);
-    o[j] = hdmoe_dev_pack_bf16(p0 + b[2 * j], p1 + b[2 * j + 1]);            // + shift
-  }
-  return make_uint4(o[0], o[1], o[2], o[3]);
-}
-
 template <int NCHUNK>  // NCHUNK * 512 == D: row held in registers; 0: any D % 8 == 0, row re-read from cache
 __global__ __launch_bounds__(WAVES_PER_BLOCK * 64) void ln_modulate_kernel(
     const uint4* __restrict__ x, const uint4* __restrict__ scale, const uint4* __restrict__ shift, int T, int D,
@@ -335,24 +376,8 @@ __global__ __launch_bounds__(WAVES_PER_BLOCK * 64) void ln_modulate_kernel(
       uint4 v[NCHUNK];
 #pragma unroll
       for (int c = 0; c < NCHUNK; ++c) v[c] = xr[c * 64 + lane];
-      float s = 0.0f;
-#pragma unroll
-      for (int c = 0; c < NCHUNK; ++c) {
-        float f[8];
-        unpack8(v[c], f);
-#pragma unroll
-        for (int j = 0; j < 8; ++j) s = s + f[j];
-      }
-      const float mean = __fdiv_rn(wave_sum(s), fD);
-      float s2 = 0.0f;
-#pragma unroll
-      for (int c = 0; c < NCHUNK; ++c) {
-        float f[8];
-        unpack8(v[c], f);
-#pragma unroll
-        for (int j = 0; j < 8; ++j) { const float d = f[j] - mean; s2 = __builtin_fmaf(d, d, s2); }
-      }
-      const float rstd = __fdiv_rn(1.0f, __builtin_sqrtf(__fdiv_rn(wave_sum(s2), fD) + eps));
+      float mean, rstd;
+      ln_stats<NCHUNK>(v, fD, eps, mean, rstd);
 #pragma unroll
       for (int c = 0; c < NCHUNK; ++c)
         out[(size_t)t * row16 + c * 64 + lane] =
@@ -396,11 +421,22 @@ extern "C" int hdmoe_gate_top2(const void* x_bf16, const void* gate_w_bf16, int 
 }
 
 // The gate of the one-call layer with fp8 experts: routing plus the token's three fp8 rows in one pass over x.
+// Whether the gate + cast kernel can also do the block's LayerNorm + modulation in front of it.
+bool hdmoe_gate_quant_takes_ln(int D, int E) { return D == 2560 && E <= 4; }
+
 int hdmoe_launch_gate_quant(const void* x_bf16, const void* gate_w_bf16, int T, int D, int E, int32_t* topk_idx,
                             void* topk_weight_bf16, const float* const* scale_input, const float* shared_scale,
-                            void* xq_routed, void* xq_shared, hipStream_t s, const char* what) {
+                            void* xq_routed, void* xq_shared, hipStream_t s, const char* what,
+                            const void* mod_scale = nullptr, const void* mod_shift = nullptr, int tokens_per_batch = 0,
+                            float ln_eps = 0.0f) {
   GateQuant q;
   memset(&q, 0, sizeof(q));
+  if (mod_scale != nullptr) {
+    q.mod_scale = static_cast<const uint4*>(mod_scale);
+    q.mod_shift = static_cast<const uint4*>(mod_shift);
+    q.tokens_per_batch = tokens_per_batch;
+    q.ln_eps = ln_eps;
+  }
   for (int e = 0; e < E && e < HDMOE_MAX_EXPERTS; ++e) q.scale_in.p[e] = scale_input[e];
   q.shared_scale = shared_scale;
   q.xq_routed = static_cast<uint2*>(xq_routed);

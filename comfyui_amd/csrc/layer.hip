@@ -15,7 +15,10 @@ int hdmoe_launch_quant_dispatch(const void* x_bf16, const int32_t* perm, const i
                                 void* a_fp8, hipStream_t s, const char* what);
 int hdmoe_launch_gate_quant(const void* x_bf16, const void* gate_w_bf16, int T, int D, int E, int32_t* topk_idx,
                             void* topk_weight_bf16, const float* const* scale_input, const float* shared_scale,
-                            void* xq_routed, void* xq_shared, hipStream_t s, const char* what);
+                            void* xq_routed, void* xq_shared, hipStream_t s, const char* what,
+                            const void* mod_scale = nullptr, const void* mod_shift = nullptr, int tokens_per_batch = 0,
+                            float ln_eps = 0.0f);
+bool hdmoe_gate_quant_takes_ln(int D, int E);
 int hdmoe_launch_combine(const void* y_sorted_bf16, const int32_t* inv_perm, const void* topk_weight_bf16,
                          const void* shared_bf16, const void* gate_bf16, const void* residual_bf16, int tokens_per_batch,
                          int T, int D, void* out_bf16, hipStream_t s, const char* what);
@@ -131,7 +134,10 @@ extern "C" int hdmoe_moe_ffn(const hdmoe_layer_args* p, hdmoe_stream_t stream) {
   // the tokens the feed-forward sees: x itself, or LayerNorm(x) * (1 + scale) + shift (timed with the gate stage)
   const void* xin = p->x;
   mark();
-  if (fused_block) {
+  // fp8 experts at the register kernel's shape: LayerNorm + modulation happen inside the gate + cast kernel and
+  // the normalised tokens are never written as bf16
+  const bool ln_in_gate = fused_block && fp8 && hdmoe_gate_quant_takes_ln(D, E);
+  if (fused_block && !ln_in_gate) {
     void* normed = ws + l.normed;
     if (int rc = hdmoe_ln_modulate_bf16(p->x, p->mod_scale, p->mod_shift, T, D, p->tokens_per_batch, p->ln_eps, normed,
                                         stream))
@@ -145,7 +151,9 @@ extern "C" int hdmoe_moe_ffn(const hdmoe_layer_args* p, hdmoe_stream_t stream) {
     const float* sin[HDMOE_MAX_EXPERTS];
     for (int e = 0; e < E; ++e) sin[e] = p->experts[e].scale_in1;
     if (int rc = hdmoe_launch_gate_quant(xin, p->gate_w, T, D, E, idx, tw, sin, Hs > 0 ? p->shared->scale_in1 : nullptr,
-                                         a_routed, Hs > 0 ? a_shared : nullptr, s, "hdmoe_moe_ffn (gate + quantise)"))
+                                         a_routed, Hs > 0 ? a_shared : nullptr, s, "hdmoe_moe_ffn (gate + quantise)",
+                                         ln_in_gate ? p->mod_scale : nullptr, ln_in_gate ? p->mod_shift : nullptr,
+                                         p->tokens_per_batch, p->ln_eps))
       return rc;
   } else {
     if (int rc = hdmoe_gate_top2(xin, p->gate_w, T, D, E, idx, tw, stream)) return rc;

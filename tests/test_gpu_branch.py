@@ -121,6 +121,26 @@ def test_branch_equals_its_three_stages(dev, weights):
         assert d["rel_rms"] < 1e-2, d
 
 
+@pytest.mark.parametrize("B,S,E", [(3, 77, 4), (1, 1, 4), (2, 129, 2), (5, 13, 3)])
+def test_branch_with_layernorm_inside_the_gate_kernel(dev, B, S, E):
+    """At width 2560 with up to four fp8 experts the LayerNorm + modulation run inside the gate + cast kernel: the
+    branch must still equal its three stages bit for bit (ragged token counts, several batch rows, 2..4 experts)."""
+    from comfyui_amd import functional as HF
+    dim, hidden_arg = 2560, 1024
+    master, g = synth.make_weights(B * 100 + S, dim=dim, hidden_arg=hidden_arg, num_experts=E)
+    sd = synth.to_state_dict(master, "fp8")
+    for i, k in enumerate(sorted(k for k in sd if k.endswith("w1.scale_input"))):
+        v = torch.tensor(0.5 + 0.25 * (i % 3), dtype=torch.float32)      # experts cast with different scales
+        sd[k] = v
+        sd[k.replace("w1.", "w3.")] = v.clone()
+    m = synth.build_module({k: v.to(dev) for k, v in sd.items()}, "fp8", dev, dim=dim, hidden_arg=hidden_arg,
+                           num_experts=E)
+    x, shift, scale, gate = (t.to(dev) for t in make(B, S, dim, seed=S, mean=0.3, spread=1.7))
+    fused = m.forward_branch(x, shift, scale, gate)
+    n = HF.ln_modulate(x.reshape(-1, dim), scale, shift, S).view(B, S, dim)
+    assert torch.equal(bits(fused), bits(gate * m(n) + x))
+
+
 def test_branch_at_headline_size_properties(dev):
     """cfg3 shape (8192 tokens, fp8): gate = 0 is the identity, the fused branch equals its stages bit for bit,
     and the normalised tokens match torch's own layer_norm on the device to one bf16 step."""
