@@ -403,6 +403,7 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
 #pragma unroll
           for (int q = 0; q < 4; ++q) {
             float m[4];
+            uint32_t pm[2];  // the same four values as packed bf16 pairs (fp8 cast without unpacking them again)
 #pragma unroll
             for (int i = 0; i < 4; i += 2) {
               // two elements at a time: one packed conversion rounds both to bf16
@@ -414,11 +415,15 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
               float sb = h1b * __builtin_amdgcn_rcpf(1.0f + __expf(-h1b));
               round2_bf16(sa, sb);
               float ma = sa * h3a, mb = sb * h3b;                                              // silu(.) * w3(x)
-              round2_bf16(ma, mb);
+              if constexpr (FP8 && NEXT == 1) {
+                pm[i / 2] = hdmoe_dev_pack_bf16(ma, mb);  // the rounding to bf16; cast from the packed pair below
+              } else {
+                round2_bf16(ma, mb);
+              }
               if constexpr (FP8 && NEXT == 2) {
                 ma *= inv_next;
                 mb *= inv_next;
-                round2_bf16(ma, mb);
+                pm[i / 2] = hdmoe_dev_pack_bf16(ma, mb);
               }
               if constexpr (FP8 && NEXT == 0) {
                 ma = ma < -448.0f ? -448.0f : (ma > 448.0f ? 448.0f : ma);
@@ -429,7 +434,9 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
             }
             const int byte = (wq * 32 + q * 8 + hi32 * 4) * EB;  // position of the 4 features in the staged row
             uint8_t* const dst = row + ((((byte >> 4) ^ (tok32 & 7)) << 4) | (byte & 15));
-            if constexpr (FP8) {
+            if constexpr (FP8 && NEXT != 0) {
+              *reinterpret_cast<uint32_t*>(dst) = hdmoe_dev_pack4_e4m3fn_bf16(pm[0], pm[1]);
+            } else if constexpr (FP8) {
               *reinterpret_cast<uint32_t*>(dst) = hdmoe_dev_pack4_e4m3fn(m[0], m[1], m[2], m[3]);
             } else {
               u32x2 pk;

@@ -111,6 +111,17 @@ __device__ __forceinline__ uint32_t hdmoe_dev_pack_e4m3fn(float a, float b) {
   return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false) & 0xffffu;
 }
 
+// e4m3fn bytes of four bf16 values given as two packed words (p01 = values 0 and 1, value 0 in the low half):
+// v_cvt_scalef32_pk_fp8_bf16 with a scale of 1 converts a bf16 pair without unpacking it and follows the same
+// no-saturation rule (checked over every bf16 pattern on the device).
+typedef short hdmoe_i16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t hdmoe_dev_pack4_e4m3fn_bf16(uint32_t p01, uint32_t p23) {
+  hdmoe_i16x2 r = {0, 0};
+  r = __builtin_amdgcn_cvt_scalef32_pk_fp8_bf16(r, *reinterpret_cast<hdmoe_bf16x2*>(&p01), 1.0f, false);
+  r = __builtin_amdgcn_cvt_scalef32_pk_fp8_bf16(r, *reinterpret_cast<hdmoe_bf16x2*>(&p23), 1.0f, true);
+  return *reinterpret_cast<uint32_t*>(&r);
+}
+
 // e4m3fn bytes of (a, b, c, d), a in the lowest byte
 __device__ __forceinline__ uint32_t hdmoe_dev_pack4_e4m3fn(float a, float b, float c, float d) {
   const int lo = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);

@@ -27,9 +27,11 @@ __device__ __forceinline__ uint32_t hdmoe_q_2(uint32_t u, float inv) {
                                hdmoe_q_pre(__uint_as_float(u & 0xffff0000u), inv));
 }
 
-// eight bf16 values -> eight e4m3fn bytes. A scale of exactly 1 skips the multiply (x * 1 rounded to bf16 is x).
+// eight bf16 values -> eight e4m3fn bytes. A scale of exactly 1 casts the packed pairs as they are (x * 1 rounded
+// to bf16 is x); otherwise the products are rounded to bf16 as packed pairs and cast from those.
 __device__ __forceinline__ uint2 hdmoe_q_8(const uint4& v, float inv) {
   const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+  if (inv == 1.0f) return make_uint2(hdmoe_dev_pack4_e4m3fn_bf16(w[0], w[1]), hdmoe_dev_pack4_e4m3fn_bf16(w[2], w[3]));
   float f[8];
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
@@ -39,15 +41,12 @@ __device__ __forceinline__ uint2 hdmoe_q_8(const uint4& v, float inv) {
   if (inv < 0.0f) {
 #pragma unroll
     for (int j = 0; j < 8; ++j) f[j] = f[j] < -448.0f ? -448.0f : (f[j] > 448.0f ? 448.0f : f[j]);
-  } else if (inv != 1.0f) {
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const uint32_t p = hdmoe_dev_pack_bf16(f[2 * j] * inv, f[2 * j + 1] * inv);
-      f[2 * j] = __uint_as_float(p << 16);
-      f[2 * j + 1] = __uint_as_float(p & 0xffff0000u);
-    }
+    return make_uint2(hdmoe_dev_pack4_e4m3fn(f[0], f[1], f[2], f[3]), hdmoe_dev_pack4_e4m3fn(f[4], f[5], f[6], f[7]));
   }
-  return make_uint2(hdmoe_dev_pack4_e4m3fn(f[0], f[1], f[2], f[3]), hdmoe_dev_pack4_e4m3fn(f[4], f[5], f[6], f[7]));
+  uint32_t p[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) p[j] = hdmoe_dev_pack_bf16(f[2 * j] * inv, f[2 * j + 1] * inv);
+  return make_uint2(hdmoe_dev_pack4_e4m3fn_bf16(p[0], p[1]), hdmoe_dev_pack4_e4m3fn_bf16(p[2], p[3]));
 }
 
 // (1.0 / scale_input).to(bfloat16) as fp32; NULL pointer -> clamp rule marker
