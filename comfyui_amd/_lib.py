@@ -74,6 +74,8 @@ SIGNATURES = {
     "hdmoe_dispatch_workspace_bytes": (c_size_t, [c_int, c_int]),
     "hdmoe_dispatch": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t,
                                c_void_p]),
+    "hdmoe_dispatch_static_max_tokens": (c_int, [c_int]),
+    "hdmoe_dispatch_static": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "hdmoe_quant_fp8": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_void_p, c_void_p]),
     "hdmoe_quant_permute_fp8": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                                         ctypes.POINTER(c_void_p), c_void_p, c_void_p]),

@@ -11,6 +11,8 @@
 //            writes perm / inv_perm.
 // No atomics, so the result does not depend on scheduling.
 // Traffic: 2T*4 bytes read twice, 2*2T*4 bytes written.
+#include <mutex>
+
 #include "common.h"
 
 namespace {
@@ -20,10 +22,7 @@ constexpr int WAVES = THREADS / 64;
 // A block handles THREADS * ITEMS flat slots. Few items per block keep the serial part of a block short (this
 // stage is latency bound at the sizes of one layer); many items bound the number of per-chunk histograms every
 // block has to sum at very large T.
-#ifndef DISPATCH_SMALL_ITEMS
-#define DISPATCH_SMALL_ITEMS 1
-#endif
-constexpr int ITEMS_SMALL = DISPATCH_SMALL_ITEMS, ITEMS_LARGE = 8;
+constexpr int ITEMS_SMALL = 1, ITEMS_LARGE = 8;
 constexpr int SMALL_MAX_SLOTS = 1 << 16;
 inline int items_for(size_t n) { return n <= (size_t)SMALL_MAX_SLOTS ? ITEMS_SMALL : ITEMS_LARGE; }
 
@@ -131,29 +130,16 @@ extern "C" size_t hdmoe_dispatch_workspace_bytes(int T, int E) {
   return hdmoe_align_up((nchunks > 0 ? nchunks : 1) * (size_t)E * sizeof(int32_t), 256);
 }
 
-extern "C" int hdmoe_dispatch(const int32_t* topk_idx, int T, int E, int32_t* counts, int32_t* offsets,
-                              int32_t* perm, int32_t* inv_perm, void* workspace, size_t workspace_bytes,
-                              hdmoe_stream_t stream) {
-  HDMOE_REQUIRE_PTR(topk_idx);
-  HDMOE_REQUIRE_PTR(counts);
-  HDMOE_REQUIRE_PTR(offsets);
-  HDMOE_REQUIRE_PTR(perm);
-  HDMOE_REQUIRE_PTR(inv_perm);
-  HDMOE_REQUIRE_PTR(workspace);
-  if (T < 0 || E < 1 || E > HDMOE_MAX_EXPERTS)
-    return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_dispatch: T=%d E=%d (1 <= E <= %d)", T, E, HDMOE_MAX_EXPERTS);
-  if ((size_t)T * HDMOE_TOPK > (size_t)INT32_MAX)
-    return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_dispatch: T=%d too large", T);
-  if (workspace_bytes < hdmoe_dispatch_workspace_bytes(T, E) || (reinterpret_cast<uintptr_t>(workspace) & 3))
-    return hdmoe_fail(HDMOE_E_WORKSPACE, "hdmoe_dispatch: workspace %zu bytes, need %zu (4-byte aligned)",
-                      workspace_bytes, hdmoe_dispatch_workspace_bytes(T, E));
-  hipStream_t s = static_cast<hipStream_t>(stream);
+namespace {
+
+// Shared by the two entry points: argument checks and the two launches; cc holds the per-chunk histograms.
+int dispatch_enqueue(const char* what, const int32_t* topk_idx, int T, int E, int32_t* counts, int32_t* offsets,
+                     int32_t* perm, int32_t* inv_perm, int32_t* cc, hipStream_t s) {
   const int n = T * HDMOE_TOPK;
   const int items = items_for((size_t)n);
   const int chunk = THREADS * items;
   int nchunks = (n + chunk - 1) / chunk;
   if (nchunks < 1) nchunks = 1;  // T == 0 still writes counts = 0 and offsets = 0
-  int32_t* cc = static_cast<int32_t*>(workspace);
   if (items == ITEMS_SMALL) {
     hipLaunchKernelGGL(dispatch_count_kernel<ITEMS_SMALL>, dim3(nchunks), dim3(THREADS), 0, s, topk_idx, n, E, cc);
     hipLaunchKernelGGL(dispatch_scatter_kernel<ITEMS_SMALL>, dim3(nchunks), dim3(THREADS), 0, s, topk_idx, n, E,
@@ -163,5 +149,98 @@ extern "C" int hdmoe_dispatch(const int32_t* topk_idx, int T, int E, int32_t* co
     hipLaunchKernelGGL(dispatch_scatter_kernel<ITEMS_LARGE>, dim3(nchunks), dim3(THREADS), 0, s, topk_idx, n, E,
                        nchunks, cc, counts, offsets, perm, inv_perm);
   }
-  return hdmoe_check_launch("hdmoe_dispatch");
+  return hdmoe_check_launch(what);
+}
+
+int dispatch_check_sizes(const char* what, int T, int E) {
+  if (T < 0 || E < 1 || E > HDMOE_MAX_EXPERTS)
+    return hdmoe_fail(HDMOE_E_SHAPE, "%s: T=%d E=%d (1 <= E <= %d)", what, T, E, HDMOE_MAX_EXPERTS);
+  if ((size_t)T * HDMOE_TOPK > (size_t)INT32_MAX) return hdmoe_fail(HDMOE_E_SHAPE, "%s: T=%d too large", what, T);
+  return HDMOE_OK;
+}
+
+}  // namespace
+
+extern "C" int hdmoe_dispatch(const int32_t* topk_idx, int T, int E, int32_t* counts, int32_t* offsets,
+                              int32_t* perm, int32_t* inv_perm, void* workspace, size_t workspace_bytes,
+                              hdmoe_stream_t stream) {
+  HDMOE_REQUIRE_PTR(topk_idx);
+  HDMOE_REQUIRE_PTR(counts);
+  HDMOE_REQUIRE_PTR(offsets);
+  HDMOE_REQUIRE_PTR(perm);
+  HDMOE_REQUIRE_PTR(inv_perm);
+  HDMOE_REQUIRE_PTR(workspace);
+  if (int rc = dispatch_check_sizes("hdmoe_dispatch", T, E)) return rc;
+  if (workspace_bytes < hdmoe_dispatch_workspace_bytes(T, E) || (reinterpret_cast<uintptr_t>(workspace) & 3))
+    return hdmoe_fail(HDMOE_E_WORKSPACE, "hdmoe_dispatch: workspace %zu bytes, need %zu (4-byte aligned)",
+                      workspace_bytes, hdmoe_dispatch_workspace_bytes(T, E));
+  return dispatch_enqueue("hdmoe_dispatch", topk_idx, T, E, counts, offsets, perm, inv_perm,
+                          static_cast<int32_t*>(workspace), static_cast<hipStream_t>(stream));
+}
+
+// ---- the same dispatch for callers that cannot allocate ------------------------------------------------------
+// The per-chunk histograms live in a device array that is part of the library image (every GPU the library runs
+// on holds its own copy until the process ends). Host code must not use the array's name as an address: the
+// device address is asked for once per device and kept.
+namespace {
+
+constexpr size_t STATIC_SCRATCH_BYTES = 64 * 1024;
+static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];
+
+constexpr int MAX_DEVICES = 64;
+std::mutex scratch_mutex;
+void* scratch_dev_ptr[MAX_DEVICES] = {};
+
+// Device address of `scratch` on the current device (looked up on the first call per device), nullptr on failure.
+void* scratch_address(const char* what, int* rc) {
+  int device = -1;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess || device < 0 || device >= MAX_DEVICES) {
+    *rc = hdmoe_fail(HDMOE_E_LAUNCH, "%s: hipGetDevice: %s (device %d)", what, hipGetErrorString(e), device);
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(scratch_mutex);
+  if (scratch_dev_ptr[device] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || p == nullptr) {
+      *rc = hdmoe_fail(HDMOE_E_LAUNCH, "%s: hipGetSymbolAddress: %s", what, hipGetErrorString(e));
+      return nullptr;
+    }
+    scratch_dev_ptr[device] = p;
+  }
+  return scratch_dev_ptr[device];
+}
+
+}  // namespace
+
+extern "C" int hdmoe_dispatch_static_max_tokens(int E) {
+  if (E < 1 || E > HDMOE_MAX_EXPERTS) return 0;
+  // chunks of THREADS * ITEMS_LARGE flat slots above SMALL_MAX_SLOTS; E counters per chunk
+  const size_t max_chunks = STATIC_SCRATCH_BYTES / (sizeof(int32_t) * (size_t)E);
+  const size_t tokens = max_chunks * (size_t)(THREADS * ITEMS_LARGE) / HDMOE_TOPK;
+  return tokens > (size_t)(INT32_MAX / HDMOE_TOPK) ? INT32_MAX / HDMOE_TOPK : (int)tokens;
+}
+
+extern "C" int hdmoe_dispatch_static(const int32_t* topk_idx, int T, int E, int32_t* counts, int32_t* offsets,
+                                     int32_t* perm, int32_t* inv_perm, hdmoe_stream_t stream) {
+  HDMOE_REQUIRE_PTR(topk_idx);
+  HDMOE_REQUIRE_PTR(counts);
+  HDMOE_REQUIRE_PTR(offsets);
+  HDMOE_REQUIRE_PTR(perm);
+  HDMOE_REQUIRE_PTR(inv_perm);
+  if (int rc = dispatch_check_sizes("hdmoe_dispatch_static", T, E)) return rc;
+  const size_t need = hdmoe_dispatch_workspace_bytes(T, E);
+  if (need > STATIC_SCRATCH_BYTES)
+    return hdmoe_fail(HDMOE_E_WORKSPACE,
+                      "hdmoe_dispatch_static: T=%d E=%d needs %zu bytes of histograms, the built-in buffer holds %zu "
+                      "(at most %d tokens for this E); use hdmoe_dispatch with a workspace",
+                      T, E, need, STATIC_SCRATCH_BYTES, hdmoe_dispatch_static_max_tokens(E));
+  int rc = HDMOE_OK;
+  void* cc = scratch_address("hdmoe_dispatch_static", &rc);
+  if (cc == nullptr) return rc;
+  // every chunk histogram the scatter kernel reads is written by the count kernel of the same call: nothing of
+  // the previous call's contents is used, so nothing has to be cleared
+  return dispatch_enqueue("hdmoe_dispatch_static", topk_idx, T, E, counts, offsets, perm, inv_perm,
+                          static_cast<int32_t*>(cc), static_cast<hipStream_t>(stream));
 }

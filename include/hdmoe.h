@@ -33,7 +33,7 @@
 extern "C" {
 #endif
 
-#define HDMOE_VERSION 105
+#define HDMOE_VERSION 106
 
 #define HDMOE_OK 0
 #define HDMOE_E_NULL (-1)      /* required pointer is NULL */
@@ -74,6 +74,18 @@ size_t hdmoe_dispatch_workspace_bytes(int T, int E);
 int hdmoe_dispatch(const int32_t* topk_idx, int T, int E, int32_t* counts, int32_t* offsets,
                    int32_t* perm, int32_t* inv_perm, void* workspace, size_t workspace_bytes,
                    hdmoe_stream_t stream);
+
+/* The same dispatch for callers that cannot allocate device memory or carry a workspace (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc). It has no counterpart in the reference. The
+ * per-chunk histograms that hdmoe_dispatch keeps in its workspace live in a 64 KiB device array inside the library
+ * image instead (one copy per GPU, held until the process ends); the call allocates nothing. T is limited to
+ * hdmoe_dispatch_static_max_tokens(E) (1 048 576 tokens at E = 16, more for fewer experts, capped by the int32 slot
+ * range); beyond that the call returns HDMOE_E_WORKSPACE and enqueues nothing. All calls on one GPU share the array:
+ * two calls whose kernels may overlap on the same GPU (different streams) race; calls on one stream do not. The
+ * first call on a device looks the array's device address up (hipGetSymbolAddress, no allocation). */
+int hdmoe_dispatch_static_max_tokens(int E);
+int hdmoe_dispatch_static(const int32_t* topk_idx, int T, int E, int32_t* counts, int32_t* offsets,
+                          int32_t* perm, int32_t* inv_perm, hdmoe_stream_t stream);
 
 /* Activation quantisation of fp8_linear, comfy/ops.py:337-343:
  * out = e4m3fn( bf16( x * bf16(1/scale_input) ) ), no saturation (|v| > 464 -> NaN);

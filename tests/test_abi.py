@@ -112,3 +112,22 @@ def test_layer_layout_is_consistent():
         assert lay.y - lay.h >= (2 * T * H + T * Hs) * eb
         assert lay.total - lay.y >= (2 * T + (T if Hs else 0)) * D * 2
     assert _lib.lib.hdmoe_layer_workspace_bytes(8, 256, 768, 512, 99, 1) == 0
+
+
+def test_static_dispatch_rejects_sizes_beyond_its_buffer():
+    from comfyui_amd import _lib
+    L = _lib.lib
+    for E in (1, 4, 16):
+        limit = L.hdmoe_dispatch_static_max_tokens(E)
+        assert limit >= 1 << 20
+        assert L.hdmoe_dispatch_workspace_bytes(limit, E) <= 64 * 1024
+    limit = L.hdmoe_dispatch_static_max_tokens(16)
+    assert L.hdmoe_dispatch_workspace_bytes(limit + 2048, 16) > 64 * 1024
+    # nothing is enqueued for a refused size, so the buffers may be tiny
+    t = torch.zeros(64, dtype=torch.int32)
+    p = t.data_ptr()
+    rc = L.hdmoe_dispatch_static(p, limit + 2048, 16, p, p, p, p, None)
+    assert rc == _lib.E_WORKSPACE
+    assert b"at most" in L.hdmoe_last_error()
+    assert L.hdmoe_dispatch_static(p, 8, 17, p, p, p, p, None) == _lib.E_SHAPE
+    assert L.hdmoe_dispatch_static(None, 8, 4, p, p, p, p, None) == _lib.E_NULL
