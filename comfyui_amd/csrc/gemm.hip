@@ -100,6 +100,71 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
+// ---- fp8 K loop in assembly ---------------------------------------------------------------------
+// The fragment registers of the fp8 K loop are fixed and its slices are written in assembly: the schedule below
+// depends on every fragment being refilled in place right after its last use, which the register allocator does
+// not do (it rotates registers and then spills the loop-invariant addresses, whose reloads wait on vmcnt and
+// with it on the global->LDS loads in flight).
+//   weight fragments  fb0 v[200:207]  fb1 v[208:215]        token fragments  fa(t) v[216+8t : 223+8t]
+// One slice (64 K bytes) = part A (weight half 0 against every token block) + part B (weight half 1). LDS
+// requests in flight at the start of a slice, oldest first: fb0, fa0 .. fa(TT-1), fb1 (two ds_read_b128 each);
+// LDS returns in order, so part A waits with lgkmcnt(2*(TT-t)) in front of MFMA t. Part B refills fb0 first,
+// then fa(t) behind the MFMA that last reads it, then fb1: every fragment is requested TT or more MFMAs (320+
+// cycles of matrix pipe) before its first use.
+#define HDMOE_FB0 "v[200:207]"
+#define HDMOE_FB1 "v[208:215]"
+#define HDMOE_FA0 "v[216:223]"
+#define HDMOE_FA1 "v[224:231]"
+#define HDMOE_FA2 "v[232:239]"
+#define HDMOE_FA3 "v[240:247]"
+#define HDMOE_FA4 "v[248:255]"
+#define HDMOE_MF(C, A, B) "v_mfma_f32_32x32x64_f8f6f4 %[" C "], " A ", " B ", %[" C "]\n"
+#define HDMOE_MZ(C, A, B) "v_mfma_f32_32x32x64_f8f6f4 %[" C "], " A ", " B ", 0\n"
+#define HDMOE_RD(LO, HI, A0, A1, OFF) \
+  "ds_read_b128 " LO ", %[" A0 "] offset:%[" OFF "]\nds_read_b128 " HI ", %[" A1 "] offset:%[" OFF "]\n"
+#define HDMOE_RD_FB0 HDMOE_RD("v[200:203]", "v[204:207]", "w0", "w1", "ob0")
+#define HDMOE_RD_FB1 HDMOE_RD("v[208:211]", "v[212:215]", "w0", "w1", "ob1")
+#define HDMOE_RD_FA0 HDMOE_RD("v[216:219]", "v[220:223]", "t0", "t1", "oa0")
+#define HDMOE_RD_FA1 HDMOE_RD("v[224:227]", "v[228:231]", "t0", "t1", "oa1")
+#define HDMOE_RD_FA2 HDMOE_RD("v[232:235]", "v[236:239]", "t0", "t1", "oa2")
+#define HDMOE_RD_FA3 HDMOE_RD("v[240:243]", "v[244:247]", "t0", "t1", "oa3")
+#define HDMOE_RD_FA4 HDMOE_RD("v[248:251]", "v[252:255]", "t0", "t1", "oa4")
+// part A: M = HDMOE_MF (accumulate) or HDMOE_MZ (first slice of a tile: C = 0)
+#define HDMOE_PART_A4(M)                                                                                   \
+  "s_waitcnt lgkmcnt(8)\n" M("c0", HDMOE_FB0, HDMOE_FA0) "s_waitcnt lgkmcnt(6)\n" M("c1", HDMOE_FB0, HDMOE_FA1) \
+  "s_waitcnt lgkmcnt(4)\n" M("c2", HDMOE_FB0, HDMOE_FA2) "s_waitcnt lgkmcnt(2)\n" M("c3", HDMOE_FB0, HDMOE_FA3)
+#define HDMOE_PART_A5(M)                                                                                    \
+  "s_waitcnt lgkmcnt(10)\n" M("c0", HDMOE_FB0, HDMOE_FA0) "s_waitcnt lgkmcnt(8)\n" M("c1", HDMOE_FB0, HDMOE_FA1) \
+  "s_waitcnt lgkmcnt(6)\n" M("c2", HDMOE_FB0, HDMOE_FA2) "s_waitcnt lgkmcnt(4)\n" M("c3", HDMOE_FB0, HDMOE_FA3)  \
+  "s_waitcnt lgkmcnt(2)\n" M("c4", HDMOE_FB0, HDMOE_FA4)
+// part B with the refills for the next slice
+#define HDMOE_PART_B4(M)                                                                        \
+  HDMOE_RD_FB0 "s_waitcnt lgkmcnt(2)\n" M("d0", HDMOE_FB1, HDMOE_FA0) HDMOE_RD_FA0               \
+  M("d1", HDMOE_FB1, HDMOE_FA1) HDMOE_RD_FA1 M("d2", HDMOE_FB1, HDMOE_FA2) HDMOE_RD_FA2          \
+  M("d3", HDMOE_FB1, HDMOE_FA3) HDMOE_RD_FA3 HDMOE_RD_FB1
+#define HDMOE_PART_B5(M)                                                                        \
+  HDMOE_RD_FB0 "s_waitcnt lgkmcnt(2)\n" M("d0", HDMOE_FB1, HDMOE_FA0) HDMOE_RD_FA0               \
+  M("d1", HDMOE_FB1, HDMOE_FA1) HDMOE_RD_FA1 M("d2", HDMOE_FB1, HDMOE_FA2) HDMOE_RD_FA2          \
+  M("d3", HDMOE_FB1, HDMOE_FA3) HDMOE_RD_FA3 M("d4", HDMOE_FB1, HDMOE_FA4) HDMOE_RD_FA4 HDMOE_RD_FB1
+// part B of the last slice of a tile: no refills; the trailing wait states cover the distance the hardware wants
+// between the last MFMA and the first VALU read of an accumulator (the compiler cannot see into the block)
+#define HDMOE_PART_B4_LAST                                                                                  \
+  "s_waitcnt lgkmcnt(0)\n" HDMOE_MF("d0", HDMOE_FB1, HDMOE_FA0) HDMOE_MF("d1", HDMOE_FB1, HDMOE_FA1)        \
+  HDMOE_MF("d2", HDMOE_FB1, HDMOE_FA2) HDMOE_MF("d3", HDMOE_FB1, HDMOE_FA3) "s_nop 15\ns_nop 7\n"
+#define HDMOE_PART_B5_LAST                                                                                  \
+  "s_waitcnt lgkmcnt(0)\n" HDMOE_MF("d0", HDMOE_FB1, HDMOE_FA0) HDMOE_MF("d1", HDMOE_FB1, HDMOE_FA1)        \
+  HDMOE_MF("d2", HDMOE_FB1, HDMOE_FA2) HDMOE_MF("d3", HDMOE_FB1, HDMOE_FA3)                                 \
+  HDMOE_MF("d4", HDMOE_FB1, HDMOE_FA4) "s_nop 15\ns_nop 7\n"
+// part B whose refills depend on a wave-uniform flag (the last slice of a tile has nothing to refill): both forms in
+// one block, so that the accumulators pass through the same statement either way
+#define HDMOE_PART_B4_SEL \
+  "s_cmp_lg_u32 %[more], 0\ns_cbranch_scc0 1f\n" HDMOE_PART_B4(HDMOE_MF) "s_branch 2f\n1:\n" HDMOE_PART_B4_LAST "2:\n"
+#define HDMOE_PART_B5_SEL \
+  "s_cmp_lg_u32 %[more], 0\ns_cbranch_scc0 1f\n" HDMOE_PART_B5(HDMOE_MF) "s_branch 2f\n1:\n" HDMOE_PART_B5_LAST "2:\n"
+// the first fragments of a tile, in the order the waits of part A assume
+#define HDMOE_FILL4 HDMOE_RD_FB0 HDMOE_RD_FA0 HDMOE_RD_FA1 HDMOE_RD_FA2 HDMOE_RD_FA3 HDMOE_RD_FB1
+#define HDMOE_FILL5 HDMOE_RD_FB0 HDMOE_RD_FA0 HDMOE_RD_FA1 HDMOE_RD_FA2 HDMOE_RD_FA3 HDMOE_RD_FA4 HDMOE_RD_FB1
+
 template <int MODE, int TT>
 __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs args) {
   constexpr bool FP8 = (MODE == FP8_SWIGLU || MODE == FP8_PLAIN || MODE == FP8_PLAIN_BIAS);
@@ -111,6 +176,12 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
   constexpr int A_BYTES = BM * BK;         // token tile of one K step in LDS; the weight tile follows it
   constexpr int STAGE_BYTES = (BM + BN) * BK;
   constexpr int FEAT_PER_TILE = SWIGLU ? BN / 2 : BN;  // output features per block tile
+  // LDS layout of the two stages. bf16: stage after stage, [A0 | B0 | A1 | B1]. fp8: [A0 | A1 | B0 | B1], so that
+  // every fragment read of the K loop is one of eight per-lane base addresses plus an immediate below 64 KiB.
+  constexpr int B_BYTES = BN * BK;
+  constexpr int A_OFF1 = FP8 ? A_BYTES : STAGE_BYTES;
+  constexpr int B_OFF0 = FP8 ? 2 * A_BYTES : A_BYTES;
+  constexpr int B_OFF1 = FP8 ? 2 * A_BYTES + B_BYTES : STAGE_BYTES + A_BYTES;
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
 
   const int tid = threadIdx.x;
@@ -237,19 +308,25 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
       src_voff_b[j] = (SWIGLU ? r : (r >> 5) * 64 + (r & 31)) * d.kbytes + ld_chunk * 16;
     }
   };
+  // K steps of the tile being loaded; a step at or past it (padding) is fetched as zeros. Step 0 of a tile is
+  // requested before the tile becomes current, so the count is never below 1.
+  int kt_real = 1;
   auto issue_loads = [&](int stage, int kt) {
-    uint8_t* sa = smem + stage * STAGE_BYTES;
-    uint8_t* sb = sa + A_BYTES;
+    uint8_t* sa = smem + (stage ? A_OFF1 : 0);
+    uint8_t* sb = smem + (stage ? B_OFF1 : B_OFF0);
     const int k0 = kt * BK;
+    const __amdgpu_buffer_rsrc_t empty = make_rsrc(nullptr, 0);
+    const bool pad = kt >= kt_real;
+    const __amdgpu_buffer_rsrc_t ra = pad ? empty : src_a, rb0 = pad ? empty : src_b0, rb1 = pad ? empty : src_b1;
 #pragma unroll
     for (int j = 0; j < A_SLABS; ++j)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(src_a, (lds_ptr_t)(sa + ld_lds + j * 64 * BK), 16, src_voff[j], k0, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, (lds_ptr_t)(sa + ld_lds + j * 64 * BK), 16, src_voff[j], k0, 0, 0);
 #pragma unroll
     for (int j = 0; j < 2; ++j)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(src_b0, (lds_ptr_t)(sb + ld_lds + j * 64 * BK), 16, src_voff_b[j], k0, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rb0, (lds_ptr_t)(sb + ld_lds + j * 64 * BK), 16, src_voff_b[j], k0, 0, 0);
 #pragma unroll
     for (int j = 0; j < 2; ++j)
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(src_b1, (lds_ptr_t)(sb + ld_lds + (j + 2) * 64 * BK), 16, src_voff_b[j], k0, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rb1, (lds_ptr_t)(sb + ld_lds + (j + 2) * 64 * BK), 16, src_voff_b[j], k0, 0, 0);
   };
 
   // ---- LDS -> MFMA fragment addressing -------------------------------------------
@@ -257,58 +334,17 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
   const int fr_row = lane & 31;
   const int fr_grp = lane >> 5;
   const int fr_swz = swz(fr_row);  // tile origins are multiples of 32 rows, so f() only sees fr_row
-  const int a_base = (wt * WAVE_TOK + fr_row) * BK;          // token operand, + tt*32*BK
-  const int b_base = A_BYTES + (wq * 32 + fr_row) * BK;      // weight operand, + ft*128*BK
+  const int a_base = (wt * WAVE_TOK + fr_row) * BK;          // token operand within its stage, + tt*32*BK
+  const int b_base = (wq * 32 + fr_row) * BK;                // weight operand within its stage, + ft*128*BK
 
   v16f acc[2][TT];
   // n_tt: how many of this wave's four 32-token blocks hold rows of the tile (4 except in the last, partial
   // m-tile of a segment); the others are neither read from LDS nor multiplied.
-  auto compute = [&](int stage, auto full_c, int n_tt) {
+  [[maybe_unused]] auto compute = [&](int stage, auto full_c, int n_tt) {
     constexpr bool FULL = decltype(full_c)::value;
-    const uint8_t* st = smem + stage * STAGE_BYTES;
-    if constexpr (FP8) {
-#pragma unroll
-      for (int ks = 0; ks < 2; ++ks) {
-        const int c0 = ((ks * 4 + fr_grp * 2) ^ fr_swz) * 16;
-        const int c1 = c0 ^ 16;
-        auto ld = [&](const uint8_t* p) -> v8i {
-          const v4i lo = *reinterpret_cast<const v4i*>(p + c0);
-          const v4i hi = *reinterpret_cast<const v4i*>(p + c1);
-          return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-        };
-        if (!FULL && n_tt == 0) continue;
-        v8i fb[2];
-#pragma unroll
-        for (int ft = 0; ft < 2; ++ft) fb[ft] = ld(st + b_base + ft * 128 * BK);
-        if constexpr (TT <= 4) {
-          // all token fragments of the slice at once
-          v8i fa[TT];
-#pragma unroll
-          for (int tt = 0; tt < TT; ++tt) {
-            if (!FULL && tt >= n_tt) continue;
-            fa[tt] = ld(st + a_base + tt * 32 * BK);
-          }
-#pragma unroll
-          for (int ft = 0; ft < 2; ++ft)
-#pragma unroll
-            for (int tt = 0; tt < TT; ++tt) {
-              if (!FULL && tt >= n_tt) continue;
-              acc[ft][tt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[ft], fa[tt], acc[ft][tt], 0, 0, 0, 0, 0, 0);
-            }
-        } else {
-          // taller tiles: one token fragment ahead of the MFMAs instead of all of them (registers)
-          v8i fa_cur = ld(st + a_base), fa_nxt = fa_cur;
-#pragma unroll
-          for (int tt = 0; tt < TT; ++tt) {
-            if (!FULL && tt >= n_tt) continue;
-            if (tt + 1 < TT && (FULL || tt + 1 < n_tt)) fa_nxt = ld(st + a_base + (tt + 1) * 32 * BK);
-            acc[0][tt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[0], fa_cur, acc[0][tt], 0, 0, 0, 0, 0, 0);
-            acc[1][tt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fb[1], fa_cur, acc[1][tt], 0, 0, 0, 0, 0, 0);
-            fa_cur = fa_nxt;
-          }
-        }
-      }
-    } else {
+    const uint8_t* sa = smem + (stage ? A_OFF1 : 0) + a_base;
+    const uint8_t* sb = smem + (stage ? B_OFF1 : B_OFF0) + b_base;
+    if constexpr (!FP8) {
 #pragma unroll
       for (int ks = 0; ks < 4; ++ks) {
         const int c0 = ((ks * 2 + fr_grp) ^ fr_swz) * 16;
@@ -316,12 +352,12 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
 #pragma unroll
         for (int tt = 0; tt < TT; ++tt) {
           if (!FULL && tt >= n_tt) continue;
-          fa[tt] = *reinterpret_cast<const v8bf*>(st + a_base + tt * 32 * BK + c0);
+          fa[tt] = *reinterpret_cast<const v8bf*>(sa + tt * 32 * BK + c0);
         }
         if (!FULL && n_tt == 0) continue;
 #pragma unroll
         for (int ft = 0; ft < 2; ++ft)
-          fb[ft] = *reinterpret_cast<const v8bf*>(st + b_base + ft * 128 * BK + c0);
+          fb[ft] = *reinterpret_cast<const v8bf*>(sb + ft * 128 * BK + c0);
 #pragma unroll
         for (int ft = 0; ft < 2; ++ft)
 #pragma unroll
@@ -331,6 +367,75 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
           }
       }
     }
+  };
+
+  // ---- fp8: software-pipelined K loop in assembly (macros above the kernel) --------------------------------
+  [[maybe_unused]] v8i fb0, fb1, fa0, fa1, fa2, fa3, fa4;
+  [[maybe_unused]] uint32_t tok_addr[2][2], w_addr[2][2];  // LDS byte address of this lane's reads, [slice][16-byte half]
+  if constexpr (FP8) {
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(lds_ptr_t)smem;
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int c = (((ks * 4 + fr_grp * 2) ^ fr_swz) * 16) ^ (h * 16);
+        tok_addr[ks][h] = lds0 + a_base + c;
+        w_addr[ks][h] = lds0 + B_OFF0 + b_base + c;
+      }
+  }
+#define HDMOE_FRAGS4                                                                                           \
+  "+{v[200:207]}"(fb0), "+{v[208:215]}"(fb1), "+{v[216:223]}"(fa0), "+{v[224:231]}"(fa1), "+{v[232:239]}"(fa2), \
+      "+{v[240:247]}"(fa3)
+#define HDMOE_FRAGS5 HDMOE_FRAGS4, "+{v[248:255]}"(fa4)
+#define HDMOE_FRAGS4_OUT                                                                                       \
+  "={v[200:207]}"(fb0), "={v[208:215]}"(fb1), "={v[216:223]}"(fa0), "={v[224:231]}"(fa1), "={v[232:239]}"(fa2), \
+      "={v[240:247]}"(fa3)
+#define HDMOE_FRAGS5_OUT HDMOE_FRAGS4_OUT, "={v[248:255]}"(fa4)
+#define HDMOE_SRC(KS, OA, OB)                                                                                  \
+  [w0] "v"(w_addr[KS][0]), [w1] "v"(w_addr[KS][1]), [t0] "v"(tok_addr[KS][0]), [t1] "v"(tok_addr[KS][1]),      \
+      [ob0] "i"(OB), [ob1] "i"(OB + 128 * BK), [oa0] "i"(OA), [oa1] "i"(OA + 32 * BK), [oa2] "i"(OA + 64 * BK), \
+      [oa3] "i"(OA + 96 * BK), [oa4] "i"(OA + 128 * BK)
+  // the tile's first fragments: slice 0 of stage 0
+  [[maybe_unused]] auto fp8_fill = [&] {
+    if constexpr (FP8 && TT == 5)
+      asm volatile(HDMOE_FILL5 : HDMOE_FRAGS5_OUT : HDMOE_SRC(0, 0, 0) : "memory");
+    else if constexpr (FP8)
+      asm volatile(HDMOE_FILL4 : HDMOE_FRAGS4_OUT : HDMOE_SRC(0, 0, 0) : "memory");
+  };
+  // Part A / part B of a slice as plain (non-generic) lambdas. MZ variants: first slice of a tile, the accumulators
+  // start from zero (C = 0) and are outputs only. Part B refills from slice KS of stage SS.
+#define HDMOE_ACC_A4(C) [c0] C(acc[0][0]), [c1] C(acc[0][1]), [c2] C(acc[0][2]), [c3] C(acc[0][3])
+#define HDMOE_ACC_B4(C) [d0] C(acc[1][0]), [d1] C(acc[1][1]), [d2] C(acc[1][2]), [d3] C(acc[1][3])
+#define HDMOE_INOUT(x) "+v"(x)
+#define HDMOE_OUT(x) "=&v"(x)
+#define HDMOE_DEF_PART_A(NAME, M, C)                                                                          \
+  [[maybe_unused]] auto NAME = [&] {                                                                          \
+    if constexpr (FP8 && TT == 5)                                                                             \
+      asm volatile(HDMOE_PART_A5(M) : HDMOE_ACC_A4(C), [c4] C(acc[0][TT - 1]), HDMOE_FRAGS5 : : "memory");    \
+    else if constexpr (FP8)                                                                                   \
+      asm volatile(HDMOE_PART_A4(M) : HDMOE_ACC_A4(C), HDMOE_FRAGS4 : : "memory");                            \
+  }
+#define HDMOE_DEF_PART_B(NAME, M, C, SS, KS)                                                                  \
+  [[maybe_unused]] auto NAME = [&] {                                                                          \
+    if constexpr (FP8 && TT == 5)                                                                             \
+      asm volatile(HDMOE_PART_B5(M) : HDMOE_ACC_B4(C), [d4] C(acc[1][TT - 1]), HDMOE_FRAGS5                   \
+                   : HDMOE_SRC(KS, (SS) * A_BYTES, (SS) * B_BYTES) : "memory");                               \
+    else if constexpr (FP8)                                                                                   \
+      asm volatile(HDMOE_PART_B4(M) : HDMOE_ACC_B4(C), HDMOE_FRAGS4                                           \
+                   : HDMOE_SRC(KS, (SS) * A_BYTES, (SS) * B_BYTES) : "memory");                               \
+  }
+  HDMOE_DEF_PART_A(fp8_a, HDMOE_MF, HDMOE_INOUT);
+  HDMOE_DEF_PART_B(fp8_b_s0k1, HDMOE_MF, HDMOE_INOUT, 0, 1);
+  HDMOE_DEF_PART_B(fp8_b_s1k1, HDMOE_MF, HDMOE_INOUT, 1, 1);
+  HDMOE_DEF_PART_B(fp8_b_s1k0, HDMOE_MF, HDMOE_INOUT, 1, 0);
+  // end of a pair of steps: refills from slice 0 of stage 0 if another pair follows
+  [[maybe_unused]] auto fp8_b_s0k0_if = [&](int more) {
+    if constexpr (FP8 && TT == 5)
+      asm volatile(HDMOE_PART_B5_SEL : HDMOE_ACC_B4(HDMOE_INOUT), [d4] "+v"(acc[1][TT - 1]), HDMOE_FRAGS5
+                   : HDMOE_SRC(0, 0, 0), [more] "s"(__builtin_amdgcn_readfirstlane(more)) : "memory", "scc");
+    else if constexpr (FP8)
+      asm volatile(HDMOE_PART_B4_SEL : HDMOE_ACC_B4(HDMOE_INOUT), HDMOE_FRAGS4
+                   : HDMOE_SRC(0, 0, 0), [more] "s"(__builtin_amdgcn_readfirstlane(more)) : "memory", "scc");
   };
 
   // ---- epilogue ----------------------------------------------------------------------
@@ -343,7 +448,10 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
   // the segment end are dropped by the range check.
   const int tok32 = lane & 31;
   const int hi32 = lane >> 5;
-  uint8_t* const stg = smem + STAGE_BYTES;
+  // Staging room for the outputs once the K loop is over: whatever is not stage 0 (which takes the next tile's
+  // first K step meanwhile). fp8: the token tile of stage 1 (BM x 128 bytes: exactly the SwiGLU tile) and the
+  // weight tile of stage 1; bf16: stage 1 as a whole.
+  uint8_t* const stg = smem + (FP8 ? A_OFF1 : STAGE_BYTES);
   auto wave_sync = [] {
     // orders this wave's LDS writes before its LDS reads of other lanes' data (LDS executes a wave's requests
     // in order; this only stops the compiler from moving them)
@@ -470,7 +578,8 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
       const int ldo = gg.n_out * 2;
       const __amdgpu_buffer_rsrc_t ro = make_rsrc(gg.out + (size_t)d.row0 * ldo, (uint32_t)d.rows_here * (uint32_t)ldo);
       // each wave stages its own 32 tokens x 64 features (128 bytes per token) at a time, two buffers in turn
-      uint8_t* const mine = stg + wave * 8192;
+      uint8_t* const mine = FP8 ? (wave < 4 ? smem + A_OFF1 + wave * 8192 : smem + B_OFF1 + (wave - 4) * 8192)
+                                : stg + wave * 8192;
       const int rd_row = lane >> 3, rd_c = lane & 7;
 #pragma unroll
       for (int tt = 0; tt < TT; ++tt) {
@@ -541,6 +650,7 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
   issue_loads(0, 0);
   for (int i = 0; cur.g >= 0; ++i) {
     const int KT = cur.kbytes / BK;
+    kt_real = KT;
     load_scales(cur);
     const Tile nxt = decode(i + 1);
     if (nxt.g >= 0) load_gather(nxt, gi_nxt);  // lands during the K loop
@@ -550,7 +660,41 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
       for (int b2 = 0; b2 < TT; ++b2)
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[a2][b2][r] = 0.0f;
-    auto k_loop = [&](auto full_c, int n_tt) {
+    // fp8: two K steps per trip, the first out of stage 0, the second out of stage 1. The barrier of a step (the
+    // loads of the next step have landed for everyone, everyone has read this stage) sits between the two parts
+    // of the second slice, in front of the first refill from the other stage, with TT MFMAs still to issue behind
+    // it: they cover the barrier skew and the LDS latency of the first new fragments. Rows past the end of a
+    // partial tile are read as zeros and multiplied like the others.
+    [[maybe_unused]] auto k_loop_fp8 = [&] {
+      // An odd number of steps is padded with one whose loads come from an empty buffer (zeros).
+      const int KTP = (KT + 1) & ~1;
+      __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's part of the first stage has landed
+      __syncthreads();
+      issue_loads(1, 1);
+      fp8_fill();
+      for (int kt = 0; kt < KTP; kt += 2) {
+        const int more = __builtin_amdgcn_readfirstlane(kt + 2 < KTP ? 1 : 0);
+        // step kt out of stage 0
+        fp8_a();
+        fp8_b_s0k1();
+        fp8_a();
+        __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0): my loads of the next step, my reads of this stage
+        __syncthreads();
+        if (more) issue_loads(0, kt + 2);
+        fp8_b_s1k0();
+        // step kt + 1 out of stage 1
+        fp8_a();
+        fp8_b_s1k1();
+        fp8_a();
+        if (more) {
+          __builtin_amdgcn_s_waitcnt(0x0070);
+          __syncthreads();
+          if (kt + 3 < KTP) issue_loads(1, kt + 3);
+        }
+        fp8_b_s0k0_if(more);
+      }
+    };
+    [[maybe_unused]] auto k_loop = [&](auto full_c, int n_tt) {
       for (int kt = 0; kt < KT; kt += 2) {
         __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's part of the stage has landed
         __syncthreads();                      // everyone's part has; everyone is done reading the other stage
@@ -565,8 +709,12 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
       }
     };
     const int my_rows = __builtin_amdgcn_readfirstlane(cur.rows_here) - wt * WAVE_TOK;  // rows of the tile in this wave's half
-    if (my_rows > 32 * (TT - 1)) k_loop(std::true_type{}, TT);
-    else k_loop(std::false_type{}, my_rows <= 0 ? 0 : (my_rows + 31) / 32);
+    if constexpr (FP8) {
+      k_loop_fp8();
+    } else {
+      if (my_rows > 32 * (TT - 1)) k_loop(std::true_type{}, TT);
+      else k_loop(std::false_type{}, my_rows <= 0 ? 0 : (my_rows + 31) / 32);
+    }
     // Every wave is done reading both stages: stage 0 can take the next tile's first K step, stage 1 the
     // staged outputs of this one (it is not loaded into again before the barrier of that K step).
     __syncthreads();
