@@ -37,6 +37,7 @@ class FfnWeights(ctypes.Structure):
         ("w1", c_void_p), ("w2", c_void_p), ("w3", c_void_p),
         ("scale_w1", c_void_p), ("scale_w2", c_void_p), ("scale_w3", c_void_p),
         ("scale_in1", c_void_p), ("scale_in2", c_void_p), ("scale_in3", c_void_p),
+        ("same_scale_in13", c_int),
     ]
 
 

@@ -30,6 +30,18 @@ static inline int hdmoe_check_launch(const char* what) {
     if ((p) == nullptr) return hdmoe_fail(HDMOE_E_NULL, "%s: %s is NULL", __func__, #p); \
   } while (0)
 
+// w1 and w3 of a SwiGLU feed-forward quantise the same input once, with scale_in1 (see hdmoe_ffn_weights).
+static inline int hdmoe_check_scale_in13(const char* what, const hdmoe_ffn_weights& w, int index) {
+  if (w.scale_in1 == w.scale_in3) return HDMOE_OK;
+  if (w.scale_in1 == nullptr || w.scale_in3 == nullptr)
+    return hdmoe_fail(HDMOE_E_SHAPE, "%s: group %d: w1 and w3 disagree on having a scale_input", what, index);
+  if (!w.same_scale_in13)
+    return hdmoe_fail(HDMOE_E_SHAPE,
+                      "%s: group %d: scale_in1 and scale_in3 are different pointers and same_scale_in13 is not set "
+                      "(the fused kernels quantise the input once, so the two values must be equal)", what, index);
+  return HDMOE_OK;
+}
+
 static inline size_t hdmoe_align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 constexpr int HDMOE_NUM_CU = 256;   // MI355X

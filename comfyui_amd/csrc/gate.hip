@@ -314,10 +314,8 @@ template <int E>
 int launch_gate(const void* x, const void* wg, int T, int D, int32_t* idx, void* w, const GateQuant* quant,
                 hipStream_t s, const char* what) {
   // about 4 tokens per wave amortise the register-resident weight slice and still give 8 waves per CU at T = 8192
-#ifndef GATE_TPW
-#define GATE_TPW 4
-#endif
-  int blocks = (T + WAVES_PER_BLOCK * GATE_TPW - 1) / (WAVES_PER_BLOCK * GATE_TPW);
+  constexpr int TOKENS_PER_WAVE = 4;
+  int blocks = (T + WAVES_PER_BLOCK * TOKENS_PER_WAVE - 1) / (WAVES_PER_BLOCK * TOKENS_PER_WAVE);
   if (blocks < 1) blocks = 1;
   if (blocks > HDMOE_NUM_CU * 8) blocks = HDMOE_NUM_CU * 8;
   dim3 grid(blocks), block(WAVES_PER_BLOCK * 64);

@@ -102,15 +102,16 @@ typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
 // ---- fp8 K loop in assembly ---------------------------------------------------------------------
 // The fragment registers of the fp8 K loop are fixed and its slices are written in assembly: the schedule below
-// depends on every fragment being refilled in place right after its last use, which the register allocator does
-// not do (it rotates registers and then spills the loop-invariant addresses, whose reloads wait on vmcnt and
-// with it on the global->LDS loads in flight).
+// depends on every fragment being refilled in place right after its last use and on the global->LDS loads of the
+// next step being issued one at a time between the MFMAs (the register allocator rotates fragment registers
+// and then spills loop-invariant addresses, and a burst of loads behind the barrier keeps both waves of a SIMD
+// in the vector-memory issue queue while the matrix pipe runs dry).
 //   weight fragments  fb0 v[200:207]  fb1 v[208:215]        token fragments  fa(t) v[216+8t : 223+8t]
 // One slice (64 K bytes) = part A (weight half 0 against every token block) + part B (weight half 1). LDS
 // requests in flight at the start of a slice, oldest first: fb0, fa0 .. fa(TT-1), fb1 (two ds_read_b128 each);
 // LDS returns in order, so part A waits with lgkmcnt(2*(TT-t)) in front of MFMA t. Part B refills fb0 first,
 // then fa(t) behind the MFMA that last reads it, then fb1: every fragment is requested TT or more MFMAs (320+
-// cycles of matrix pipe) before its first use.
+// cycles of matrix pipe) before its first use. The global->LDS loads count on vmcnt, not lgkmcnt.
 #define HDMOE_FB0 "v[200:207]"
 #define HDMOE_FB1 "v[208:215]"
 #define HDMOE_FA0 "v[216:223]"
@@ -119,33 +120,63 @@ typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 #define HDMOE_FA3 "v[240:247]"
 #define HDMOE_FA4 "v[248:255]"
 #define HDMOE_MF(C, A, B) "v_mfma_f32_32x32x64_f8f6f4 %[" C "], " A ", " B ", %[" C "]\n"
-#define HDMOE_MZ(C, A, B) "v_mfma_f32_32x32x64_f8f6f4 %[" C "], " A ", " B ", 0\n"
+// fragment reads: operands w0/w1 (weights) and t0/t1 (tokens) are the lane's two 16-byte halves of the slice read,
+// ob / oa the byte offset of the stage read from
 #define HDMOE_RD(LO, HI, A0, A1, OFF) \
-  "ds_read_b128 " LO ", %[" A0 "] offset:%[" OFF "]\nds_read_b128 " HI ", %[" A1 "] offset:%[" OFF "]\n"
-#define HDMOE_RD_FB0 HDMOE_RD("v[200:203]", "v[204:207]", "w0", "w1", "ob0")
-#define HDMOE_RD_FB1 HDMOE_RD("v[208:211]", "v[212:215]", "w0", "w1", "ob1")
-#define HDMOE_RD_FA0 HDMOE_RD("v[216:219]", "v[220:223]", "t0", "t1", "oa0")
-#define HDMOE_RD_FA1 HDMOE_RD("v[224:227]", "v[228:231]", "t0", "t1", "oa1")
-#define HDMOE_RD_FA2 HDMOE_RD("v[232:235]", "v[236:239]", "t0", "t1", "oa2")
-#define HDMOE_RD_FA3 HDMOE_RD("v[240:243]", "v[244:247]", "t0", "t1", "oa3")
-#define HDMOE_RD_FA4 HDMOE_RD("v[248:251]", "v[252:255]", "t0", "t1", "oa4")
-// part A: M = HDMOE_MF (accumulate) or HDMOE_MZ (first slice of a tile: C = 0)
-#define HDMOE_PART_A4(M)                                                                                   \
-  "s_waitcnt lgkmcnt(8)\n" M("c0", HDMOE_FB0, HDMOE_FA0) "s_waitcnt lgkmcnt(6)\n" M("c1", HDMOE_FB0, HDMOE_FA1) \
-  "s_waitcnt lgkmcnt(4)\n" M("c2", HDMOE_FB0, HDMOE_FA2) "s_waitcnt lgkmcnt(2)\n" M("c3", HDMOE_FB0, HDMOE_FA3)
-#define HDMOE_PART_A5(M)                                                                                    \
-  "s_waitcnt lgkmcnt(10)\n" M("c0", HDMOE_FB0, HDMOE_FA0) "s_waitcnt lgkmcnt(8)\n" M("c1", HDMOE_FB0, HDMOE_FA1) \
-  "s_waitcnt lgkmcnt(6)\n" M("c2", HDMOE_FB0, HDMOE_FA2) "s_waitcnt lgkmcnt(4)\n" M("c3", HDMOE_FB0, HDMOE_FA3)  \
-  "s_waitcnt lgkmcnt(2)\n" M("c4", HDMOE_FB0, HDMOE_FA4)
-// part B with the refills for the next slice
-#define HDMOE_PART_B4(M)                                                                        \
-  HDMOE_RD_FB0 "s_waitcnt lgkmcnt(2)\n" M("d0", HDMOE_FB1, HDMOE_FA0) HDMOE_RD_FA0               \
-  M("d1", HDMOE_FB1, HDMOE_FA1) HDMOE_RD_FA1 M("d2", HDMOE_FB1, HDMOE_FA2) HDMOE_RD_FA2          \
-  M("d3", HDMOE_FB1, HDMOE_FA3) HDMOE_RD_FA3 HDMOE_RD_FB1
-#define HDMOE_PART_B5(M)                                                                        \
-  HDMOE_RD_FB0 "s_waitcnt lgkmcnt(2)\n" M("d0", HDMOE_FB1, HDMOE_FA0) HDMOE_RD_FA0               \
-  M("d1", HDMOE_FB1, HDMOE_FA1) HDMOE_RD_FA1 M("d2", HDMOE_FB1, HDMOE_FA2) HDMOE_RD_FA2          \
-  M("d3", HDMOE_FB1, HDMOE_FA3) HDMOE_RD_FA3 M("d4", HDMOE_FB1, HDMOE_FA4) HDMOE_RD_FA4 HDMOE_RD_FB1
+  "ds_read_b128 " LO ", %[" A0 "] offset:" OFF "\nds_read_b128 " HI ", %[" A1 "] offset:" OFF "\n"
+#define HDMOE_RD_FB0 HDMOE_RD("v[200:203]", "v[204:207]", "w0", "w1", "%[ob]")
+#define HDMOE_RD_FB1 HDMOE_RD("v[208:211]", "v[212:215]", "w0", "w1", "%[ob]+16384")
+#define HDMOE_RD_FA0 HDMOE_RD("v[216:219]", "v[220:223]", "t0", "t1", "%[oa]")
+#define HDMOE_RD_FA1 HDMOE_RD("v[224:227]", "v[228:231]", "t0", "t1", "%[oa]+4096")
+#define HDMOE_RD_FA2 HDMOE_RD("v[232:235]", "v[236:239]", "t0", "t1", "%[oa]+8192")
+#define HDMOE_RD_FA3 HDMOE_RD("v[240:243]", "v[244:247]", "t0", "t1", "%[oa]+12288")
+#define HDMOE_RD_FA4 HDMOE_RD("v[248:251]", "v[252:255]", "t0", "t1", "%[oa]+16384")
+// one global->LDS load of 8 rows x 128 bytes per wave: M0 = LDS address of the wave's rows (ldsd: the wave's
+// offset inside a 64-row slab, IMM: stage and slab), vector offset = the lane's row and chunk, scalar offset = K
+#define HDMOE_LD(RS, VO, IMM) \
+  "s_add_u32 m0, %[ldsd], " IMM "\ns_nop 0\nbuffer_load_dwordx4 %[" VO "], %[" RS "], %[so] offen lds\n"
+#define HDMOE_LDW0 HDMOE_LD("rb0", "vb0", "%[wd]")
+#define HDMOE_LDW1 HDMOE_LD("rb0", "vb1", "%[wd]+8192")
+#define HDMOE_LDW2 HDMOE_LD("rb1", "vb0", "%[wd]+16384")
+#define HDMOE_LDW3 HDMOE_LD("rb1", "vb1", "%[wd]+24576")
+#define HDMOE_LDT0 HDMOE_LD("ra", "va0", "%[td]")
+#define HDMOE_LDT1 HDMOE_LD("ra", "va1", "%[td]+8192")
+#define HDMOE_LDT2 HDMOE_LD("ra", "va2", "%[td]+16384")
+#define HDMOE_LDT3 HDMOE_LD("ra", "va3", "%[td]+24576")
+#define HDMOE_LDT4 HDMOE_LD("ra", "va4", "%[td]+32768")
+#define HDMOE_NONE ""
+// part A; L0..L4: what follows each MFMA (a token load of the next step, or nothing)
+#define HDMOE_PART_A4(L0, L1, L2, L3)                                                      \
+  "s_waitcnt lgkmcnt(8)\n" HDMOE_MF("c0", HDMOE_FB0, HDMOE_FA0) L0                         \
+  "s_waitcnt lgkmcnt(6)\n" HDMOE_MF("c1", HDMOE_FB0, HDMOE_FA1) L1                         \
+  "s_waitcnt lgkmcnt(4)\n" HDMOE_MF("c2", HDMOE_FB0, HDMOE_FA2) L2                         \
+  "s_waitcnt lgkmcnt(2)\n" HDMOE_MF("c3", HDMOE_FB0, HDMOE_FA3) L3
+#define HDMOE_PART_A5(L0, L1, L2, L3, L4)                                                  \
+  "s_waitcnt lgkmcnt(10)\n" HDMOE_MF("c0", HDMOE_FB0, HDMOE_FA0) L0                        \
+  "s_waitcnt lgkmcnt(8)\n" HDMOE_MF("c1", HDMOE_FB0, HDMOE_FA1) L1                         \
+  "s_waitcnt lgkmcnt(6)\n" HDMOE_MF("c2", HDMOE_FB0, HDMOE_FA2) L2                         \
+  "s_waitcnt lgkmcnt(4)\n" HDMOE_MF("c3", HDMOE_FB0, HDMOE_FA3) L3                         \
+  "s_waitcnt lgkmcnt(2)\n" HDMOE_MF("c4", HDMOE_FB0, HDMOE_FA4) L4
+#define HDMOE_PART_A4_PLAIN HDMOE_PART_A4(HDMOE_NONE, HDMOE_NONE, HDMOE_NONE, HDMOE_NONE)
+#define HDMOE_PART_A5_PLAIN HDMOE_PART_A5(HDMOE_NONE, HDMOE_NONE, HDMOE_NONE, HDMOE_NONE, HDMOE_NONE)
+#define HDMOE_PART_A4_LOADS HDMOE_PART_A4(HDMOE_LDT0, HDMOE_LDT1, HDMOE_LDT2, HDMOE_LDT3)
+#define HDMOE_PART_A5_LOADS HDMOE_PART_A5(HDMOE_LDT0, HDMOE_LDT1, HDMOE_LDT2, HDMOE_LDT3, HDMOE_LDT4)
+// part B with the refills for the next slice; L0..L3: a weight load of the step after the next, or nothing
+#define HDMOE_PART_B4(L0, L1, L2, L3)                                                            \
+  HDMOE_RD_FB0 "s_waitcnt lgkmcnt(2)\n" HDMOE_MF("d0", HDMOE_FB1, HDMOE_FA0) HDMOE_RD_FA0 L0     \
+  HDMOE_MF("d1", HDMOE_FB1, HDMOE_FA1) HDMOE_RD_FA1 L1                                           \
+  HDMOE_MF("d2", HDMOE_FB1, HDMOE_FA2) HDMOE_RD_FA2 L2                                           \
+  HDMOE_MF("d3", HDMOE_FB1, HDMOE_FA3) HDMOE_RD_FA3 HDMOE_RD_FB1 L3
+#define HDMOE_PART_B5(L0, L1, L2, L3)                                                            \
+  HDMOE_RD_FB0 "s_waitcnt lgkmcnt(2)\n" HDMOE_MF("d0", HDMOE_FB1, HDMOE_FA0) HDMOE_RD_FA0 L0     \
+  HDMOE_MF("d1", HDMOE_FB1, HDMOE_FA1) HDMOE_RD_FA1 L1                                           \
+  HDMOE_MF("d2", HDMOE_FB1, HDMOE_FA2) HDMOE_RD_FA2 L2                                           \
+  HDMOE_MF("d3", HDMOE_FB1, HDMOE_FA3) HDMOE_RD_FA3 L3                                           \
+  HDMOE_MF("d4", HDMOE_FB1, HDMOE_FA4) HDMOE_RD_FA4 HDMOE_RD_FB1
+#define HDMOE_PART_B4_PLAIN HDMOE_PART_B4(HDMOE_NONE, HDMOE_NONE, HDMOE_NONE, HDMOE_NONE)
+#define HDMOE_PART_B5_PLAIN HDMOE_PART_B5(HDMOE_NONE, HDMOE_NONE, HDMOE_NONE, HDMOE_NONE)
+#define HDMOE_PART_B4_LOADS HDMOE_PART_B4(HDMOE_LDW0, HDMOE_LDW1, HDMOE_LDW2, HDMOE_LDW3)
+#define HDMOE_PART_B5_LOADS HDMOE_PART_B5(HDMOE_LDW0, HDMOE_LDW1, HDMOE_LDW2, HDMOE_LDW3)
 // part B of the last slice of a tile: no refills; the trailing wait states cover the distance the hardware wants
 // between the last MFMA and the first VALU read of an accumulator (the compiler cannot see into the block)
 #define HDMOE_PART_B4_LAST                                                                                  \
@@ -155,12 +186,10 @@ typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
   "s_waitcnt lgkmcnt(0)\n" HDMOE_MF("d0", HDMOE_FB1, HDMOE_FA0) HDMOE_MF("d1", HDMOE_FB1, HDMOE_FA1)        \
   HDMOE_MF("d2", HDMOE_FB1, HDMOE_FA2) HDMOE_MF("d3", HDMOE_FB1, HDMOE_FA3)                                 \
   HDMOE_MF("d4", HDMOE_FB1, HDMOE_FA4) "s_nop 15\ns_nop 7\n"
-// part B whose refills depend on a wave-uniform flag (the last slice of a tile has nothing to refill): both forms in
-// one block, so that the accumulators pass through the same statement either way
-#define HDMOE_PART_B4_SEL \
-  "s_cmp_lg_u32 %[more], 0\ns_cbranch_scc0 1f\n" HDMOE_PART_B4(HDMOE_MF) "s_branch 2f\n1:\n" HDMOE_PART_B4_LAST "2:\n"
-#define HDMOE_PART_B5_SEL \
-  "s_cmp_lg_u32 %[more], 0\ns_cbranch_scc0 1f\n" HDMOE_PART_B5(HDMOE_MF) "s_branch 2f\n1:\n" HDMOE_PART_B5_LAST "2:\n"
+// Two forms of a part in one block, chosen by the wave-uniform operand fl, so that the accumulators pass through the
+// same statement either way (a branch around separate statements makes the compiler copy and spill them).
+#define HDMOE_SELECT(IF_SET, IF_CLEAR) \
+  "s_cmp_lg_u32 %[fl], 0\ns_cbranch_scc0 1f\n" IF_SET "s_branch 2f\n1:\n" IF_CLEAR "2:\n"
 // the first fragments of a tile, in the order the waits of part A assume
 #define HDMOE_FILL4 HDMOE_RD_FB0 HDMOE_RD_FA0 HDMOE_RD_FA1 HDMOE_RD_FA2 HDMOE_RD_FA3 HDMOE_RD_FB1
 #define HDMOE_FILL5 HDMOE_RD_FB0 HDMOE_RD_FA0 HDMOE_RD_FA1 HDMOE_RD_FA2 HDMOE_RD_FA3 HDMOE_RD_FA4 HDMOE_RD_FB1
@@ -285,8 +314,24 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
       gi[j] = (gg.gather != nullptr && r < d.rows_here) ? gg.gather[d.row0 + r] : -1;
     }
   };
+  // the same three resources as plain descriptor words, for the loads issued from the assembly blocks
+  [[maybe_unused]] v4i ra4 = {0, 0, 0, 0}, rb04 = ra4, rb14 = ra4;
+  auto raw_rsrc = [](const void* p, uint32_t bytes) -> v4i {
+    const uint64_t a = reinterpret_cast<uint64_t>(p);
+    v4i r;
+    r.x = (int)(uint32_t)a; r.y = (int)(uint32_t)((a >> 32) & 0xffffu); r.z = (int)bytes; r.w = 0x00020000;
+    return r;
+  };
   auto set_src = [&](const Tile& d, const int (&gi)[MAX_SLABS]) {
     const GemmGroup& gg = args.g[d.g];
+    if constexpr (FP8) {
+      if (gg.gather != nullptr) ra4 = raw_rsrc(gg.a, (uint32_t)gg.a_rows * (uint32_t)d.kbytes);
+      else ra4 = raw_rsrc(gg.a + (size_t)d.row0 * d.kbytes, (uint32_t)d.rows_here * (uint32_t)d.kbytes);
+      const uint32_t wrows = SWIGLU ? BN / 2 : BN - 32;
+      rb04 = raw_rsrc(gg.b0 + (size_t)d.n0 * d.kbytes, wrows * (uint32_t)d.kbytes);
+      rb14 = raw_rsrc(SWIGLU ? gg.b1 + (size_t)d.n0 * d.kbytes : gg.b0 + (size_t)(d.n0 + 32) * d.kbytes,
+                      wrows * (uint32_t)d.kbytes);
+    }
     if (gg.gather != nullptr) {
       // rows past the segment end get an offset beyond the buffer and read as zero
       src_a = make_rsrc(gg.a, (uint32_t)gg.a_rows * (uint32_t)d.kbytes);
@@ -391,51 +436,75 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
   "={v[200:207]}"(fb0), "={v[208:215]}"(fb1), "={v[216:223]}"(fa0), "={v[224:231]}"(fa1), "={v[232:239]}"(fa2), \
       "={v[240:247]}"(fa3)
 #define HDMOE_FRAGS5_OUT HDMOE_FRAGS4_OUT, "={v[248:255]}"(fa4)
-#define HDMOE_SRC(KS, OA, OB)                                                                                  \
+#define HDMOE_ACC_A4 [c0] "+v"(acc[0][0]), [c1] "+v"(acc[0][1]), [c2] "+v"(acc[0][2]), [c3] "+v"(acc[0][3])
+#define HDMOE_ACC_B4 [d0] "+v"(acc[1][0]), [d1] "+v"(acc[1][1]), [d2] "+v"(acc[1][2]), [d3] "+v"(acc[1][3])
+#define HDMOE_ACC_A5 HDMOE_ACC_A4, [c4] "+v"(acc[0][TT - 1])
+#define HDMOE_ACC_B5 HDMOE_ACC_B4, [d4] "+v"(acc[1][TT - 1])
+  // fragment reads of slice KS out of stage SS
+#define HDMOE_SRC(KS, SS)                                                                                      \
   [w0] "v"(w_addr[KS][0]), [w1] "v"(w_addr[KS][1]), [t0] "v"(tok_addr[KS][0]), [t1] "v"(tok_addr[KS][1]),      \
-      [ob0] "i"(OB), [ob1] "i"(OB + 128 * BK), [oa0] "i"(OA), [oa1] "i"(OA + 32 * BK), [oa2] "i"(OA + 64 * BK), \
-      [oa3] "i"(OA + 96 * BK), [oa4] "i"(OA + 128 * BK)
+      [oa] "i"((SS) * A_BYTES), [ob] "i"((SS) * B_BYTES)
+  // token loads into stage TS: resource, the lane offsets of the slabs, K offset, the wave's LDS offset
+#define HDMOE_TOK_LOADS(TS)                                                                                    \
+  [fl] "s"(fl), [ra] "s"(ra), [so] "s"(so), [ldsd] "s"(lds_wave), [td] "i"((TS) ? A_OFF1 : 0),                 \
+      [va0] "v"(src_voff[0]), [va1] "v"(src_voff[1]), [va2] "v"(src_voff[2]), [va3] "v"(src_voff[3]),          \
+      [va4] "v"(src_voff[A_SLABS - 1])
+  // weight loads into stage WS
+#define HDMOE_W_LOADS(WS)                                                                                      \
+  [fl] "s"(fl), [rb0] "s"(rb0), [rb1] "s"(rb1), [so] "s"(so), [ldsd] "s"(lds_wave),                            \
+      [wd] "i"((WS) ? B_OFF1 : B_OFF0), [vb0] "v"(src_voff_b[0]), [vb1] "v"(src_voff_b[1])
+  [[maybe_unused]] uint32_t lds_wave = 0;  // LDS address of this wave's rows inside a 64-row slab of stage 0's token tile
+  if constexpr (FP8) lds_wave = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr_t)smem + ld_lds);
   // the tile's first fragments: slice 0 of stage 0
   [[maybe_unused]] auto fp8_fill = [&] {
-    if constexpr (FP8 && TT == 5)
-      asm volatile(HDMOE_FILL5 : HDMOE_FRAGS5_OUT : HDMOE_SRC(0, 0, 0) : "memory");
-    else if constexpr (FP8)
-      asm volatile(HDMOE_FILL4 : HDMOE_FRAGS4_OUT : HDMOE_SRC(0, 0, 0) : "memory");
+    if constexpr (FP8 && TT == 5) asm volatile(HDMOE_FILL5 : HDMOE_FRAGS5_OUT : HDMOE_SRC(0, 0) : "memory");
+    else if constexpr (FP8) asm volatile(HDMOE_FILL4 : HDMOE_FRAGS4_OUT : HDMOE_SRC(0, 0) : "memory");
   };
-  // Part A / part B of a slice as plain (non-generic) lambdas. MZ variants: first slice of a tile, the accumulators
-  // start from zero (C = 0) and are outputs only. Part B refills from slice KS of stage SS.
-#define HDMOE_ACC_A4(C) [c0] C(acc[0][0]), [c1] C(acc[0][1]), [c2] C(acc[0][2]), [c3] C(acc[0][3])
-#define HDMOE_ACC_B4(C) [d0] C(acc[1][0]), [d1] C(acc[1][1]), [d2] C(acc[1][2]), [d3] C(acc[1][3])
-#define HDMOE_INOUT(x) "+v"(x)
-#define HDMOE_OUT(x) "=&v"(x)
-#define HDMOE_DEF_PART_A(NAME, M, C)                                                                          \
-  [[maybe_unused]] auto NAME = [&] {                                                                          \
-    if constexpr (FP8 && TT == 5)                                                                             \
-      asm volatile(HDMOE_PART_A5(M) : HDMOE_ACC_A4(C), [c4] C(acc[0][TT - 1]), HDMOE_FRAGS5 : : "memory");    \
-    else if constexpr (FP8)                                                                                   \
-      asm volatile(HDMOE_PART_A4(M) : HDMOE_ACC_A4(C), HDMOE_FRAGS4 : : "memory");                            \
+  [[maybe_unused]] auto fp8_a = [&] {
+    if constexpr (FP8 && TT == 5) asm volatile(HDMOE_PART_A5_PLAIN : HDMOE_ACC_A5, HDMOE_FRAGS5 : : "memory");
+    else if constexpr (FP8) asm volatile(HDMOE_PART_A4_PLAIN : HDMOE_ACC_A4, HDMOE_FRAGS4 : : "memory");
+  };
+  // part A that, if fl is set, also requests the token rows of K offset so into stage TS, one load behind each MFMA
+#define HDMOE_DEF_PART_A_LOADS(NAME, TS)                                                                        \
+  [[maybe_unused]] auto NAME = [&](int fl, v4i ra, int so) {                                                    \
+    if constexpr (FP8 && TT == 5)                                                                               \
+      asm volatile(HDMOE_SELECT(HDMOE_PART_A5_LOADS, HDMOE_PART_A5_PLAIN)                                       \
+                   : HDMOE_ACC_A5, HDMOE_FRAGS5 : HDMOE_TOK_LOADS(TS) : "memory", "scc");                       \
+    else if constexpr (FP8)                                                                                     \
+      asm volatile(HDMOE_SELECT(HDMOE_PART_A4_LOADS, HDMOE_PART_A4_PLAIN)                                       \
+                   : HDMOE_ACC_A4, HDMOE_FRAGS4 : HDMOE_TOK_LOADS(TS) : "memory", "scc");                       \
   }
-#define HDMOE_DEF_PART_B(NAME, M, C, SS, KS)                                                                  \
-  [[maybe_unused]] auto NAME = [&] {                                                                          \
-    if constexpr (FP8 && TT == 5)                                                                             \
-      asm volatile(HDMOE_PART_B5(M) : HDMOE_ACC_B4(C), [d4] C(acc[1][TT - 1]), HDMOE_FRAGS5                   \
-                   : HDMOE_SRC(KS, (SS) * A_BYTES, (SS) * B_BYTES) : "memory");                               \
-    else if constexpr (FP8)                                                                                   \
-      asm volatile(HDMOE_PART_B4(M) : HDMOE_ACC_B4(C), HDMOE_FRAGS4                                           \
-                   : HDMOE_SRC(KS, (SS) * A_BYTES, (SS) * B_BYTES) : "memory");                               \
+  HDMOE_DEF_PART_A_LOADS(fp8_a_loads_to0, 0);
+  HDMOE_DEF_PART_A_LOADS(fp8_a_loads_to1, 1);
+  // part B with the refills from slice KS of stage SS
+#define HDMOE_DEF_PART_B(NAME, SS, KS)                                                                          \
+  [[maybe_unused]] auto NAME = [&] {                                                                            \
+    if constexpr (FP8 && TT == 5)                                                                               \
+      asm volatile(HDMOE_PART_B5_PLAIN : HDMOE_ACC_B5, HDMOE_FRAGS5 : HDMOE_SRC(KS, SS) : "memory");            \
+    else if constexpr (FP8)                                                                                     \
+      asm volatile(HDMOE_PART_B4_PLAIN : HDMOE_ACC_B4, HDMOE_FRAGS4 : HDMOE_SRC(KS, SS) : "memory");            \
   }
-  HDMOE_DEF_PART_A(fp8_a, HDMOE_MF, HDMOE_INOUT);
-  HDMOE_DEF_PART_B(fp8_b_s0k1, HDMOE_MF, HDMOE_INOUT, 0, 1);
-  HDMOE_DEF_PART_B(fp8_b_s1k1, HDMOE_MF, HDMOE_INOUT, 1, 1);
-  HDMOE_DEF_PART_B(fp8_b_s1k0, HDMOE_MF, HDMOE_INOUT, 1, 0);
-  // end of a pair of steps: refills from slice 0 of stage 0 if another pair follows
-  [[maybe_unused]] auto fp8_b_s0k0_if = [&](int more) {
+  HDMOE_DEF_PART_B(fp8_b_s0k1, 0, 1);
+  HDMOE_DEF_PART_B(fp8_b_s1k1, 1, 1);
+  // second slice of an even step: refills from slice 0 of stage 1; if fl is set, the weight rows of K offset so
+  // go into stage 0
+  [[maybe_unused]] auto fp8_b_even = [&](int fl, v4i rb0, v4i rb1, int so) {
     if constexpr (FP8 && TT == 5)
-      asm volatile(HDMOE_PART_B5_SEL : HDMOE_ACC_B4(HDMOE_INOUT), [d4] "+v"(acc[1][TT - 1]), HDMOE_FRAGS5
-                   : HDMOE_SRC(0, 0, 0), [more] "s"(__builtin_amdgcn_readfirstlane(more)) : "memory", "scc");
+      asm volatile(HDMOE_SELECT(HDMOE_PART_B5_LOADS, HDMOE_PART_B5_PLAIN)
+                   : HDMOE_ACC_B5, HDMOE_FRAGS5 : HDMOE_SRC(0, 1), HDMOE_W_LOADS(0) : "memory", "scc");
     else if constexpr (FP8)
-      asm volatile(HDMOE_PART_B4_SEL : HDMOE_ACC_B4(HDMOE_INOUT), HDMOE_FRAGS4
-                   : HDMOE_SRC(0, 0, 0), [more] "s"(__builtin_amdgcn_readfirstlane(more)) : "memory", "scc");
+      asm volatile(HDMOE_SELECT(HDMOE_PART_B4_LOADS, HDMOE_PART_B4_PLAIN)
+                   : HDMOE_ACC_B4, HDMOE_FRAGS4 : HDMOE_SRC(0, 1), HDMOE_W_LOADS(0) : "memory", "scc");
+  };
+  // second slice of an odd step: if fl is set (another pair of steps follows), refills from slice 0 of stage 0 and
+  // the weight rows of K offset so go into stage 1; else it is the last slice of the tile
+  [[maybe_unused]] auto fp8_b_odd = [&](int fl, v4i rb0, v4i rb1, int so) {
+    if constexpr (FP8 && TT == 5)
+      asm volatile(HDMOE_SELECT(HDMOE_PART_B5_LOADS, HDMOE_PART_B5_LAST)
+                   : HDMOE_ACC_B5, HDMOE_FRAGS5 : HDMOE_SRC(0, 0), HDMOE_W_LOADS(1) : "memory", "scc");
+    else if constexpr (FP8)
+      asm volatile(HDMOE_SELECT(HDMOE_PART_B4_LOADS, HDMOE_PART_B4_LAST)
+                   : HDMOE_ACC_B4, HDMOE_FRAGS4 : HDMOE_SRC(0, 0), HDMOE_W_LOADS(1) : "memory", "scc");
   };
 
   // ---- epilogue ----------------------------------------------------------------------
@@ -668,30 +737,35 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
     [[maybe_unused]] auto k_loop_fp8 = [&] {
       // An odd number of steps is padded with one whose loads come from an empty buffer (zeros).
       const int KTP = (KT + 1) & ~1;
+      auto sgpr = [](int v) { return __builtin_amdgcn_readfirstlane(v); };
+      auto rsrc4 = [&](const v4i& r, bool real) -> v4i {  // the resource, or an empty one (every load returns zeros)
+        v4i o;
+        o.x = sgpr(r.x); o.y = sgpr(r.y); o.z = sgpr(real ? r.z : 0); o.w = sgpr(r.w);
+        return o;
+      };
       __builtin_amdgcn_s_waitcnt(0x0f70);  // vmcnt(0): this wave's part of the first stage has landed
       __syncthreads();
-      issue_loads(1, 1);
+      issue_loads(1, 1);                   // step 1 as a burst; from step 2 on the loads sit between the MFMAs
       fp8_fill();
       for (int kt = 0; kt < KTP; kt += 2) {
-        const int more = __builtin_amdgcn_readfirstlane(kt + 2 < KTP ? 1 : 0);
-        // step kt out of stage 0
-        fp8_a();
+        const int more = sgpr(kt + 2 < KTP ? 1 : 0);
+        // step kt out of stage 0. Its first slice requests the token rows of step kt + 1 into stage 1 (the weight
+        // rows of that step went out in the second slice of step kt - 1; step 1 was requested above).
+        fp8_a_loads_to1(sgpr(kt > 0 ? 1 : 0), rsrc4(ra4, kt + 1 < KT), sgpr((kt + 1) * BK));
         fp8_b_s0k1();
         fp8_a();
-        __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0): my loads of the next step, my reads of this stage
+        __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0): my loads of step kt + 1, my reads of stage 0
         __syncthreads();
-        if (more) issue_loads(0, kt + 2);
-        fp8_b_s1k0();
+        fp8_b_even(more, rsrc4(rb04, true), rsrc4(rb14, true), sgpr((kt + 2) * BK));  // weights of step kt + 2 -> stage 0
         // step kt + 1 out of stage 1
-        fp8_a();
+        fp8_a_loads_to0(more, rsrc4(ra4, true), sgpr((kt + 2) * BK));                 // tokens of step kt + 2 -> stage 0
         fp8_b_s1k1();
         fp8_a();
         if (more) {
           __builtin_amdgcn_s_waitcnt(0x0070);
           __syncthreads();
-          if (kt + 3 < KTP) issue_loads(1, kt + 3);
         }
-        fp8_b_s0k0_if(more);
+        fp8_b_odd(more, rsrc4(rb04, kt + 3 < KT), rsrc4(rb14, kt + 3 < KT), sgpr((kt + 3) * BK));  // weights of step kt + 3 -> stage 1
       }
     };
     [[maybe_unused]] auto k_loop = [&](auto full_c, int n_tt) {
@@ -933,6 +1007,9 @@ extern "C" int hdmoe_grouped_swiglu(int weight_dtype, const void* a, const int32
   HDMOE_REQUIRE_PTR(h);
   if (E < 1 || E > HDMOE_MAX_EXPERTS) return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_grouped_swiglu: E=%d", E);
   if (int rc = hdmoe_check_gemm_shape("hdmoe_grouped_swiglu", weight_dtype, rows_total, D, H, BN / 2)) return rc;
+  if (weight_dtype == HDMOE_W_E4M3FN)
+    for (int e = 0; e < E; ++e)
+      if (int rc = hdmoe_check_scale_in13("hdmoe_grouped_swiglu", experts[e], e)) return rc;
   if (rows_total == 0) return HDMOE_OK;
   return hdmoe_launch_ffn_gemm(true, weight_dtype, static_cast<const uint8_t*>(a), offsets, rows_total, E, experts,
                                static_cast<uint8_t*>(h), nullptr, 0, nullptr, nullptr, D, H, 0, 0,

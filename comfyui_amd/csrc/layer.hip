@@ -116,10 +116,11 @@ extern "C" int hdmoe_moe_ffn(const hdmoe_layer_args* p, hdmoe_stream_t stream) {
   uint8_t* y_shared = y_routed + (size_t)n * D * 2;
   hipStream_t s = static_cast<hipStream_t>(stream);
 
-  for (int e = 0; e < E; ++e) {
-    const hdmoe_ffn_weights& w = p->experts[e];
-    if (fp8 && w.scale_in1 != w.scale_in3 && (w.scale_in1 == nullptr || w.scale_in3 == nullptr))
-      return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_moe_ffn: expert %d: w1 and w3 disagree on having a scale_input", e);
+  if (fp8) {
+    for (int e = 0; e < E; ++e)
+      if (int rc = hdmoe_check_scale_in13("hdmoe_moe_ffn", p->experts[e], e)) return rc;
+    if (Hs > 0)
+      if (int rc = hdmoe_check_scale_in13("hdmoe_moe_ffn (shared expert)", *p->shared, E)) return rc;
   }
 
   int ev = 0;
@@ -216,8 +217,8 @@ extern "C" int hdmoe_ffn_swiglu(int weight_dtype, const void* x_bf16, int rows, 
                       workspace_bytes, need);
   if (rows == 0) return HDMOE_OK;
   const bool fp8 = weight_dtype == HDMOE_W_E4M3FN;
-  if (fp8 && w->scale_in1 != w->scale_in3 && (w->scale_in1 == nullptr || w->scale_in3 == nullptr))
-    return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_ffn_swiglu: w1 and w3 disagree on having a scale_input");
+  if (fp8)
+    if (int rc = hdmoe_check_scale_in13("hdmoe_ffn_swiglu", *w, 0)) return rc;
   hipStream_t s = static_cast<hipStream_t>(stream);
   uint8_t* ws = static_cast<uint8_t*>(workspace);
   const uint8_t* a = static_cast<const uint8_t*>(x_bf16);

@@ -266,14 +266,16 @@ def gated_residual(y2d, gate, residual2d, tokens_per_batch):
     return out
 
 
-def make_ffn_weights(w1, w2, w3, scales=None):
+def make_ffn_weights(w1, w2, w3, scales=None, same_scale_in13=False):
     """Fill an hdmoe_ffn_weights. scales: dict with optional fp32 scalar tensors
-    scale_w1/2/3 and scale_in1/2/3 (fp8 only)."""
+    scale_w1/2/3 and scale_in1/2/3 (fp8 only). same_scale_in13: the caller has checked that scale_in1 and
+    scale_in3, two different tensors, hold the same value (the library refuses two different pointers otherwise)."""
     fw = FfnWeights()
     fw.w1, fw.w2, fw.w3 = ptr(w1), ptr(w2), ptr(w3)
     if scales:
         for k, v in scales.items():
             setattr(fw, k, ptr(v))
+    fw.same_scale_in13 = 1 if same_scale_in13 else 0
     return fw
 
 

@@ -16,7 +16,6 @@ otherwise it composes the same HIP stages per expert through the Linear modules,
 needs the per-expert row counts on the host (one sync, as the reference's mask indexing).
 Inputs must be bf16 HIP tensors: there is no CPU path.
 """
-import weakref
 from typing import Optional
 
 import torch
@@ -27,24 +26,6 @@ from . import ops as amd_ops
 
 FP8 = torch.float8_e4m3fn
 BF16 = torch.bfloat16
-
-
-_scale_cache = {}
-
-
-def _scale_value(p):
-    """Host copy of an fp32 scalar Parameter, read once per (parameter object, version, address), so steady-state
-    forwards do not synchronise. The entry keeps a weak reference to the tensor it was read from: an id or an
-    address alone can be reused by a different tensor after the first one is freed."""
-    key = id(p)
-    hit = _scale_cache.get(key)
-    if hit is not None and hit[0]() is p and hit[1] == p._version and hit[2] == p.data_ptr():
-        return hit[3]
-    if len(_scale_cache) > 4096:
-        _scale_cache.clear()
-    v = float(p.detach().float().cpu())
-    _scale_cache[key] = (weakref.ref(p), p._version, p.data_ptr(), v)
-    return v
 
 
 def _plain(lin):
@@ -59,6 +40,7 @@ def _pack_ffn(ffn, x, wdt, keep):
     fp8 = wdt == FP8
     dev = x.device
     scales = {}
+    own = {}   # the Linear's own scale_input (Parameter or tensor, wherever it lives): the stable object to cache on
     ws = []
     for name, l in (("1", ffn.w1), ("2", ffn.w2), ("3", ffn.w3)):
         if _plain(l) and l.weight.device == dev:
@@ -72,19 +54,25 @@ def _pack_ffn(ffn, x, wdt, keep):
             sw = getattr(l, "scale_weight", None)
             sw = amd_ops._one(dev) if sw is None else sw.to(dev)
             si = getattr(l, "scale_input", None)
+            own[name] = si
             if si is not None:
                 si = si.to(dev)
                 keep.append(si)
             keep.append(sw)
             scales["scale_w" + name] = sw
             scales["scale_in" + name] = si
+    same13 = False
     if fp8:
         s1, s3 = scales["scale_in1"], scales["scale_in3"]
         if (s1 is None) != (s3 is None):
             return None
-        if s1 is not None and s1.data_ptr() != s3.data_ptr() and _scale_value(s1) != _scale_value(s3):
-            return None  # w1 and w3 quantise the same input differently: one fp8 copy cannot serve both
-    return HF.make_ffn_weights(ws[0], ws[1], ws[2], scales)
+        if s1 is not None and s1.data_ptr() != s3.data_ptr():
+            # two tensors: the values are read from the Linears' own tensors (a host tensor of an offloaded module
+            # costs no device synchronisation; a device Parameter is read once and cached)
+            if amd_ops.scale_value(own["1"]) != amd_ops.scale_value(own["3"]):
+                return None  # w1 and w3 quantise the same input differently: one fp8 copy cannot serve both
+            same13 = True
+    return HF.make_ffn_weights(ws[0], ws[1], ws[2], scales, same_scale_in13=same13)
 
 
 def _fusable_dtype(ffns):
@@ -99,6 +87,8 @@ def _fusable_dtype(ffns):
         return None
     if wdt == FP8 and not all(getattr(l, "hdmoe_fp8_matrix_mult", isinstance(l, amd_ops.fp8_ops.Linear)) for l in lins):
         return None  # scaled fp8 without fp8 matrix multiply: dequantising Linear path
+    if wdt == FP8 and any(isinstance(l, amd_ops.fp8_ops.Linear) and l.training for l in lins):
+        return None  # fp8_ops.Linear computes in the activation dtype while training (comfy/ops.py:368)
     return wdt
 
 

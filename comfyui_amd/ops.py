@@ -20,6 +20,8 @@ Every forward needs HIP tensors; a CPU tensor raises (the package has no CPU pat
 import contextlib
 import logging
 
+import weakref
+
 import torch
 
 from . import functional as HF
@@ -107,6 +109,37 @@ class CastWeightBiasOp:
     bias_function = []
 
 
+_scale_cache = {}
+_scale_epoch = 0
+
+
+def invalidate_scale_cache():
+    """Forget every cached scale_input value. Called when a Linear of this package loads a state dict or takes a new
+    weight (ops.py); call it after changing a scale_input Parameter in place by other means (`p.data.copy_()` does
+    not bump the version counter the cache looks at)."""
+    global _scale_epoch
+    _scale_epoch += 1
+    _scale_cache.clear()
+
+
+def scale_value(p, use_cache=None):
+    """Host value of an fp32 scalar Parameter. A host tensor is read directly (no device involved). A device tensor is
+    read once per (parameter object, version, address, cache epoch), so steady-state forwards do not synchronise.
+    The entry keeps a weak reference to the tensor it was read from: an id or an address alone can be reused by a
+    different tensor after the first one is freed. use_cache: None = only for device tensors."""
+    if not (p.is_cuda if use_cache is None else use_cache):
+        return float(p.detach().float())
+    key = id(p)
+    hit = _scale_cache.get(key)
+    if hit is not None and hit[0]() is p and hit[1] == p._version and hit[2] == p.data_ptr() and hit[4] == _scale_epoch:
+        return hit[3]
+    if len(_scale_cache) > 4096:
+        _scale_cache.clear()
+    v = float(p.detach().float().cpu())
+    _scale_cache[key] = (weakref.ref(p), p._version, p.data_ptr(), v, _scale_epoch)
+    return v
+
+
 def _linear_bf16(input, weight, bias):
     shape = input.shape
     x2 = input.reshape(-1, shape[-1]).contiguous()
@@ -119,6 +152,10 @@ class disable_weight_init:
     class Linear(torch.nn.Linear, CastWeightBiasOp):
         def reset_parameters(self):
             return None
+
+        def _load_from_state_dict(self, *args, **kwargs):
+            invalidate_scale_cache()   # load_state_dict copies into the Parameters in place
+            return super()._load_from_state_dict(*args, **kwargs)
 
         def forward_comfy_cast_weights(self, input):
             weight, bias = cast_bias_weight(self, input)
@@ -180,9 +217,14 @@ class fp8_ops(manual_cast):
 
         def forward_comfy_cast_weights(self, input):
             if not self.training:
-                out = fp8_linear(self, input)
-                if out is not None:
-                    return out
+                # as comfy/ops.py:367-374: whatever goes wrong in the fp8 path is logged and the Linear is
+                # computed in the activation dtype instead
+                try:
+                    out = fp8_linear(self, input)
+                    if out is not None:
+                        return out
+                except Exception as e:
+                    logging.info("Exception during fp8 op: {}".format(e))
             weight, bias = cast_bias_weight(self, input)
             return _linear_bf16(input, weight, bias)
 

@@ -13,8 +13,11 @@
  *   - all matrices are row-major and contiguous; weights are [out_features, in_features]
  *     exactly as torch.nn.Linear stores them;
  *   - `stream` is a hipStream_t passed as void*; kernels are enqueued on it and the
- *     call returns without synchronising; nothing is allocated and no global state
- *     is mutated, so calls on different streams may overlap;
+ *     call returns without synchronising; nothing is allocated, so calls on different
+ *     streams may overlap;
+ *   - the only state the library keeps between calls: the thread-local error message, and per device one flag per
+ *     GEMM kernel variant recording that hipFuncSetAttribute (the opt-in for more than 64 KiB of dynamic LDS) has
+ *     been called for it on that device, plus the device address of the built-in buffer of hdmoe_dispatch_static;
  *   - return value 0 = enqueued; negative = HDMOE_E_* and nothing was enqueued;
  *     hdmoe_last_error() gives a thread-local message for the last failure;
  *   - scale pointers (float*, device) address the fp32 scalar Parameters
@@ -33,7 +36,7 @@
 extern "C" {
 #endif
 
-#define HDMOE_VERSION 106
+#define HDMOE_VERSION 107
 
 #define HDMOE_OK 0
 #define HDMOE_E_NULL (-1)      /* required pointer is NULL */
@@ -115,9 +118,14 @@ typedef struct hdmoe_ffn_weights {
   const float* scale_w1;
   const float* scale_w2;
   const float* scale_w3;
-  const float* scale_in1; /* scale_input of w1; must describe the same value as scale_in3 */
+  const float* scale_in1; /* scale_input of w1 */
   const float* scale_in2; /* scale_input of w2 */
-  const float* scale_in3;
+  const float* scale_in3; /* scale_input of w3 */
+  /* w1 and w3 read the same input, which the fused kernels quantise once, with scale_in1: the two scale_inputs must
+   * hold the same value. The library cannot compare device scalars without synchronising, so it accepts
+   * scale_in1 == scale_in3 as pointers (both NULL included) and, for two different non-NULL pointers, only a caller
+   * that sets this field to nonzero, asserting that the two values are equal; anything else is HDMOE_E_SHAPE. */
+  int same_scale_in13;
 } hdmoe_ffn_weights;
 
 /* First half of FeedForwardSwiGLU.forward (model.py:238) for every expert at once:

@@ -6,8 +6,10 @@ Gates (fp8 weights tolerance 3e-2, bf16 weights 1e-2, from the task statement):
     rms(err)/rms(ref) <= TOL_RMS and max|err|/max|ref| <= tol;
   * output vs the same dataflow evaluated with fp32 intermediates (no bf16 rounding between ops):
     rms(err)/rms(ref) <= tol.
-max|err|/rms(ref) is reported, not gated: rounding the output itself to bf16 already costs up to
-2^-8 * |y|, i.e. 1.6e-2 * rms at |y| = 4 rms.
+max|err|/rms(ref) is gated at MAX_OVER_RMS: rounding the output itself to bf16 already costs up to
+2^-8 * |y|, i.e. 1.6e-2 * rms at |y| = 4 rms and 3.1e-2 * rms at 8 rms, which the largest of the 21 million outputs
+of the headline configuration reach; one e4m3 neighbour flipped in the intermediate by a one-step difference of its
+bf16 input adds to that. The bounds are about twice what the five configurations measure.
 """
 import pytest
 import torch
@@ -20,6 +22,7 @@ pytestmark = pytest.mark.gpu
 BF16 = torch.bfloat16
 TOL = {"fp8": 3e-2, "bf16": 1e-2}
 TOL_RMS_SAME_DATAFLOW = {"fp8": 1e-2, "bf16": 4e-3}
+MAX_OVER_RMS = {"fp8": 1.2e-1, "bf16": 6e-2}   # max|err| / rms(ref) against the bf16-dataflow oracle
 
 
 def run_gpu(sd, x, weights, dev, dim, hidden_arg=None, num_experts=4, **kw):
@@ -50,8 +53,9 @@ def check_layer(sd, x, weights, y, idx, w, num_experts, token_subset=None, gate_
     m_same = O.error_metrics(got, ref_same)
     m_f32 = O.error_metrics(got, ref_f32)
     print(f"\n[{weights}] T={x2.shape[0]} vs bf16-dataflow oracle {m_same}\n        vs fp32-intermediate oracle {m_f32}")
-    assert not bool(got.float().isnan().any())
+    assert bool(torch.isfinite(y.float()).all()), "the whole output must be finite, not only the compared tokens"
     assert m_same["rel_rms"] <= TOL_RMS_SAME_DATAFLOW[weights], m_same
+    assert m_same["max_over_rms"] <= MAX_OVER_RMS[weights], m_same
     assert m_same["max_over_max"] <= TOL[weights], m_same
     if gate_f32:
         assert m_f32["rel_rms"] <= TOL[weights], m_f32
@@ -141,18 +145,18 @@ def test_composed_path_matches_fused(dev):
     assert diff["rel_rms"] < 2e-3
 
 
-@pytest.mark.parametrize("name,subset", [("cfg1", 256), ("cfg2", 192), ("cfg3", 192), ("cfg5-256", 256), ("cfg5-4096", 192)])
-def test_benchmark_configs(dev, name, subset):
+@pytest.mark.parametrize("name", ["cfg1", "cfg2", "cfg3", "cfg5-256", "cfg5-4096"])
+def test_benchmark_configs(dev, name):
+    """The benchmark configurations at their full size: EVERY token of the output is compared with the oracle (an
+    unwritten or misplaced output tile anywhere would show), routing and permutation bit-exact on every token."""
     cfg = synth.make_config(name)
     weights = cfg["weights"]
     sd = synth.to_state_dict(cfg["master"], weights)
     x = cfg["x"]
     y, idx, w, _ = run_gpu(sd, x, weights, dev, synth.DIM)
     T = x.shape[0] * x.shape[1]
-    g = torch.Generator().manual_seed(1)
-    sel = torch.randperm(T, generator=g)[:subset].sort().values
+    sel = None
     if name.startswith("cfg5"):
-        sel = torch.unique(torch.cat([sel, torch.arange(0, T, 64)[:32]]))  # include exact-tie tokens
         counts = torch.bincount(idx.reshape(-1).long(), minlength=4).float() / T
         print("expert share of tokens", counts.tolist())
         assert 0.65 < counts[0] < 0.8 and counts[3] < 0.02

@@ -224,33 +224,44 @@ def test_gate_module_signature(dev):
 
 
 def test_stacked_layers_at_32768_tokens(dev):
-    """Stacked sweep (benchmark configuration 4) on a reduced stack: 3 independent fp8 layers at 2 x 16384 tokens,
+    """Stacked sweep (benchmark configuration 4) at its full depth: 48 independent fp8 layers at 2 x 16384 tokens,
     x <- x + FFN(LayerNorm(x)) with the block's affine-free LayerNorm (model.py:393,430) so the residual stream
-    stays in range. Tokens are independent through the whole stack, so the oracle follows a token subset."""
-    T, D, L = 32768, synth.DIM, 3
+    stays in range. Weights are drawn on the device (the CPU generator would need minutes for 11.5 GB) and copied
+    back for the oracle, which follows a token subset: tokens are independent through the whole stack. Every layer's
+    whole output must be finite and routing is compared bit for bit on the subset."""
+    from comfyui_amd import functional as HF
+    T, D, L = 32768, synth.DIM, 48
     g = torch.Generator().manual_seed(99)
     x0 = torch.randn((2, T // 2, D), generator=g).to(BF16)
-    sel = torch.randperm(T, generator=g)[:48].sort().values
+    sel = torch.randperm(T, generator=g)[:16].sort().values
     xd = x0.to(dev)
     ln = lambda t: torch.nn.functional.layer_norm(t.float(), (D,), eps=1e-6).to(BF16)
+    worst = dict(rel_rms=0.0, max_over_max=0.0)
     for layer in range(L):
-        master, _ = synth.make_weights(layer)
-        sd = synth.to_state_dict(master, "fp8")
+        master, _ = synth.make_weights(layer, device=dev)
+        sd_dev = synth.to_state_dict(master, "fp8")
         del master
-        m = synth.build_module({k: v.to(dev) for k, v in sd.items()}, "fp8", dev)
+        m = synth.build_module(sd_dev, "fp8", dev)
+        sd = {k: v.cpu() for k, v in sd_dev.items()}
         # the oracle starts every layer from the device's own residual stream (for the token subset): rounding
         # differences of one layer would otherwise flip e4m3 neighbours in the next and the two runs drift apart
         xs = xd.reshape(-1, D)[sel].cpu().unsqueeze(0)
-        xd = xd + m(ln(xd))
+        hd = ln(xd)
+        idx_d, w_d = HF.gate_top2(hd.reshape(-1, D)[sel.to(dev)].contiguous(), m.gate.weight)
+        xd = xd + m(hd)
+        assert bool(torch.isfinite(xd.float()).all()), f"layer {layer}: non-finite residual stream"
         h = ln(xs)
         idx, w, _, _ = O.gate_fixed_order(h.reshape(-1, D), sd["gate.weight"])
+        assert torch.equal(idx_d.cpu(), idx) and torch.equal(w_d.cpu().view(torch.int16), w.view(torch.int16)), layer
         ref = xs + O.moe_forward(h, oracle_params(sd, 4), "fp8mm", gate_result=(idx, w))
         got = xd.reshape(-1, D)[sel].cpu()
         met = O.error_metrics(got, ref.reshape(-1, D))
-        print(f"layer {layer}: rms(x)={float(got.float().pow(2).mean().sqrt()):.3f} {met}")
-        assert not bool(got.float().isnan().any())
-        assert met["rel_rms"] <= 1e-2 and met["max_over_max"] <= 3e-2, met
-        del m
+        worst = {k: max(worst[k], met[k]) for k in worst}
+        if layer % 8 == 0 or layer == L - 1:
+            print(f"layer {layer}: rms(x)={float(got.float().pow(2).mean().sqrt()):.3f} {met}", flush=True)
+        assert met["rel_rms"] <= 1e-2 and met["max_over_max"] <= 3e-2, (layer, met)
+        del m, sd_dev, sd
+    print("worst over the stack", worst)
 
 
 @pytest.mark.parametrize("weights", ["fp8", "bf16"])

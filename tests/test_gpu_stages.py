@@ -200,7 +200,8 @@ def test_swiglu_epilogue_cast_overflows_to_nan_like_torch(dev, rows, next_scale)
     one = torch.ones((), dtype=torch.float32)
     s1, s3 = torch.tensor(0.5), torch.tensor(1.0)
     sn = None if next_scale is None else torch.tensor(float(next_scale))
-    scales = dict(scale_w1=s1.to(dev), scale_w3=s3.to(dev), scale_in1=one.to(dev))
+    one_d = one.to(dev)
+    scales = dict(scale_w1=s1.to(dev), scale_w3=s3.to(dev), scale_in1=one_d, scale_in3=one_d)
     if sn is not None:
         scales["scale_in2"] = sn.to(dev)
     w1d, w3d = w1.to(FP8).to(dev), w3.to(FP8).to(dev)

@@ -153,15 +153,47 @@ def test_product_never_imports_the_oracle():
 
 
 def test_scale_cache_is_not_fooled_by_a_reused_id_or_address():
-    """The host copy of a scale is cached per parameter object; an entry left by a freed tensor whose id and address
-    a new tensor happens to reuse must not be served for the new one."""
+    """The host copy of a device scale is cached per parameter object; an entry left by a freed tensor whose id and
+    address a new tensor happens to reuse must not be served for the new one. (Host tensors are read directly; the
+    cache is exercised here on host tensors by asking for it.)"""
     import weakref
-    from comfyui_amd import hidream
+    from comfyui_amd import ops
     old = torch.nn.Parameter(torch.tensor(3.0), requires_grad=False)
     new = torch.nn.Parameter(torch.tensor(0.25), requires_grad=False)
-    hidream._scale_cache[id(new)] = (weakref.ref(old), new._version, new.data_ptr(), 3.0)
-    assert hidream._scale_value(new) == 0.25
-    assert hidream._scale_value(new) == 0.25          # now served from the refreshed entry
+    ops._scale_cache[id(new)] = (weakref.ref(old), new._version, new.data_ptr(), 3.0, ops._scale_epoch)
+    assert ops.scale_value(new, use_cache=True) == 0.25
+    assert ops.scale_value(new, use_cache=True) == 0.25          # now served from the refreshed entry
     with torch.no_grad():
         new.fill_(0.5)                                 # in-place update bumps the version
-    assert hidream._scale_value(new) == 0.5
+    assert ops.scale_value(new, use_cache=True) == 0.5
+
+
+def test_scale_cache_is_dropped_on_load_and_on_request():
+    """`p.data.copy_()`, which is how a state dict is loaded and how ModelPatcher writes in place, does not bump the
+    version counter: the cache is dropped whenever a Linear of this package loads a state dict, and on request."""
+    from comfyui_amd import ops
+    p = torch.nn.Parameter(torch.tensor(2.0), requires_grad=False)
+    assert ops.scale_value(p, use_cache=True) == 2.0
+    p.data.copy_(torch.tensor(4.0))
+    assert ops.scale_value(p, use_cache=True) == 2.0             # the stale entry the hooks exist for
+    ops.invalidate_scale_cache()
+    assert ops.scale_value(p, use_cache=True) == 4.0
+    p.data.copy_(torch.tensor(8.0))
+    lin = ops.disable_weight_init.Linear(4, 4, bias=False)
+    lin.load_state_dict({"weight": torch.zeros(4, 4)})
+    assert ops.scale_value(p, use_cache=True) == 8.0
+    assert ops.scale_value(p) == 8.0                             # host tensors are read directly by default
+
+
+def test_fp8_ops_linear_falls_back_when_the_fp8_path_raises(monkeypatch, caplog):
+    """comfy/ops.py:367-377: an exception inside fp8_linear is logged and the Linear is computed the plain way."""
+    import logging
+    from comfyui_amd import ops
+    lin = ops.fp8_ops.Linear(8, 8, bias=False, dtype=torch.float8_e4m3fn).eval()
+    calls = []
+    monkeypatch.setattr(ops, "fp8_linear", lambda self, x: (_ for _ in ()).throw(TypeError("no fp8 for this input")))
+    monkeypatch.setattr(ops, "_linear_bf16", lambda x, w, b: calls.append((x.dtype, w.dtype)) or "plain result")
+    with caplog.at_level(logging.INFO):
+        out = lin.forward_comfy_cast_weights(torch.zeros((2, 8), dtype=torch.bfloat16))
+    assert out == "plain result" and calls == [(torch.bfloat16, torch.bfloat16)]
+    assert any("Exception during fp8 op" in r.message for r in caplog.records)
