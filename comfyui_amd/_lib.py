@@ -64,7 +64,7 @@ class LayerLayout(ctypes.Structure):
     """hdmoe_layer_layout"""
     _fields_ = [(n, c_size_t) for n in
                 ("topk_idx", "topk_weight", "counts", "offsets", "perm", "inv_perm", "dispatch_ws",
-                 "a", "h", "y", "normed", "total")]
+                 "a", "h", "y", "normed", "partials", "total")]
 
 
 # name -> (restype, argtypes); every symbol include/hdmoe.h declares

@@ -80,6 +80,7 @@ struct GemmGroup {
   int act;              // BF16_PLAIN_BIAS: 0 = none, 1 = erf GELU on the rounded output
   int n_out;            // output features (H for swiglu, N for plain)
   int kbytes;           // bytes per row of a and of the weights
+  float* pout;          // split K: row 0 of this group in part 0 of the fp32 partial sums, [parts][rows][n_out]
 };
 
 struct GemmArgs {
@@ -88,6 +89,11 @@ struct GemmArgs {
   int n_offsets;
   int G;
   int spread;  // 0: one tile list cut in eighths; 1 / -1: every group cut in eighths, groups walked up / down
+  // Split K (plain modes, few tiles): every tile exists nparts times, part p multiplying K steps
+  // [KT*p/nparts, KT*(p+1)/nparts) and leaving its raw fp32 sums in pout + p * part_stride; a second kernel adds the
+  // parts up. 1 = off.
+  int nparts;
+  long long part_stride;  // floats between two parts
 };
 
 __device__ __forceinline__ int swz(int row) { return ((row >> 1) & 7) ^ ((row & 1) << 2); }
@@ -230,7 +236,7 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
   for (int g = 0; g < args.G; ++g) {
     int rb, re;
     seg(args.g[g], rb, re);
-    total += ((re - rb + BM - 1) / BM) * (args.g[g].n_out / FEAT_PER_TILE);
+    total += ((re - rb + BM - 1) / BM) * (args.g[g].n_out / FEAT_PER_TILE) * args.nparts;
   }
   // Each XCD (block ids congruent mod 8) walks one contiguous eighth of the tile list and its blocks take
   // consecutive tiles, so the CUs of an XCD share operand tiles in their L2.
@@ -238,9 +244,9 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
   const int xcd = blockIdx.x % HDMOE_NUM_XCD, slot = blockIdx.x / HDMOE_NUM_XCD;
   const int nslots = gridDim.x / HDMOE_NUM_XCD;
 
-  struct Tile { int g, row0, rows_here, n0, kbytes; };
+  struct Tile { int g, row0, rows_here, n0, kbytes, part, kt0, nkt; };
   auto decode = [&](int i) -> Tile {
-    Tile d = {-1, 0, 0, 0, 0};
+    Tile d = {-1, 0, 0, 0, 0, 0, 0, 0};
     int in_xcd = slot + i * nslots;
     int L = 0, g = 0, rb = 0, re = 0, mtiles = 0, ntiles = 0;
     if (args.spread != 0) {
@@ -253,7 +259,7 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
         seg(args.g[g], rb, re);
         mtiles = (re - rb + BM - 1) / BM;
         ntiles = args.g[g].n_out / FEAT_PER_TILE;
-        const long long tiles = (long long)mtiles * ntiles;
+        const long long tiles = (long long)mtiles * ntiles * args.nparts;
         const int lo = (int)(xcd * tiles / HDMOE_NUM_XCD), hi = (int)((xcd + 1) * tiles / HDMOE_NUM_XCD);
         if (in_xcd < hi - lo) { L = lo + in_xcd; break; }
         in_xcd -= hi - lo;
@@ -266,12 +272,15 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
         seg(args.g[g], rb, re);
         mtiles = (re - rb + BM - 1) / BM;
         ntiles = args.g[g].n_out / FEAT_PER_TILE;
-        const int tiles = mtiles * ntiles;
+        const int tiles = mtiles * ntiles * args.nparts;
         if (L < tiles) break;
         L -= tiles;
       }
       if (g >= args.G) return d;
     }
+    // split K: the parts of a group one after the other (tiles of one part share operand slices, parts do not)
+    const int part = L / (mtiles * ntiles);
+    L -= part * (mtiles * ntiles);
     // bands of GROUP_M m-tiles; a short remainder joins the last band, so that the cheap partial m-tile at the
     // end of a segment is interleaved with full ones instead of forming a run of its own
     const int nbands = max(1, (mtiles + GROUP_M / 2) / GROUP_M);
@@ -284,6 +293,10 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
     d.rows_here = min(re - d.row0, BM);
     d.n0 = (within / gm) * FEAT_PER_TILE;
     d.kbytes = args.g[g].kbytes;
+    const int ktf = d.kbytes / BK;
+    d.part = part;
+    d.kt0 = ktf * part / args.nparts;
+    d.nkt = ktf * (part + 1) / args.nparts - d.kt0;
     return d;
   };
 
@@ -322,8 +335,10 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
     r.x = (int)(uint32_t)a; r.y = (int)(uint32_t)((a >> 32) & 0xffffu); r.z = (int)bytes; r.w = 0x00020000;
     return r;
   };
+  int k_base = 0;  // K byte offset of step 0 of the tile being loaded (split K)
   auto set_src = [&](const Tile& d, const int (&gi)[MAX_SLABS]) {
     const GemmGroup& gg = args.g[d.g];
+    k_base = d.kt0 * BK;
     if constexpr (FP8) {
       if (gg.gather != nullptr) ra4 = raw_rsrc(gg.a, (uint32_t)gg.a_rows * (uint32_t)d.kbytes);
       else ra4 = raw_rsrc(gg.a + (size_t)d.row0 * d.kbytes, (uint32_t)d.rows_here * (uint32_t)d.kbytes);
@@ -359,7 +374,7 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
   auto issue_loads = [&](int stage, int kt) {
     uint8_t* sa = smem + (stage ? A_OFF1 : 0);
     uint8_t* sb = smem + (stage ? B_OFF1 : B_OFF0);
-    const int k0 = kt * BK;
+    const int k0 = k_base + kt * BK;
     const __amdgpu_buffer_rsrc_t empty = make_rsrc(nullptr, 0);
     const bool pad = kt >= kt_real;
     const __amdgpu_buffer_rsrc_t ra = pad ? empty : src_a, rb0 = pad ? empty : src_b0, rb1 = pad ? empty : src_b1;
@@ -643,6 +658,30 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
         __builtin_amdgcn_raw_buffer_store_b128(v, ro, r * ldo + d.n0 * EB + c * 16, 0, 0);
       }
     } else {
+      if constexpr (!BIAS) {
+        if (args.nparts > 1) {
+          // split K: this part's raw fp32 sums; scale and rounding happen where the parts are added up. A lane holds
+          // four consecutive features of a token per accumulator quad: one 16-byte store each.
+          const int ldp = gg.n_out * 4;
+          float* const pb = gg.pout + (size_t)d.part * (size_t)args.part_stride + (size_t)d.row0 * gg.n_out;
+          const __amdgpu_buffer_rsrc_t rp = make_rsrc(pb, (uint32_t)d.rows_here * (uint32_t)ldp);
+#pragma unroll
+          for (int tt = 0; tt < TT; ++tt)
+#pragma unroll
+            for (int ft = 0; ft < 2; ++ft)
+#pragma unroll
+              for (int q = 0; q < 4; ++q) {
+                v4i v;
+                v.x = __float_as_int(acc[ft][tt][q * 4 + 0]);
+                v.y = __float_as_int(acc[ft][tt][q * 4 + 1]);
+                v.z = __float_as_int(acc[ft][tt][q * 4 + 2]);
+                v.w = __float_as_int(acc[ft][tt][q * 4 + 3]);
+                __builtin_amdgcn_raw_buffer_store_b128(
+                    v, rp, (wt * WAVE_TOK + tt * 32 + tok32) * ldp + (d.n0 + wq * 64 + ft * 32 + q * 8 + hi32 * 4) * 4, 0, 0);
+              }
+          return;
+        }
+      }
       const float sc = ep_a;
       const int ldo = gg.n_out * 2;
       const __amdgpu_buffer_rsrc_t ro = make_rsrc(gg.out + (size_t)d.row0 * ldo, (uint32_t)d.rows_here * (uint32_t)ldo);
@@ -718,7 +757,7 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
   set_src(cur, gi_cur);
   issue_loads(0, 0);
   for (int i = 0; cur.g >= 0; ++i) {
-    const int KT = cur.kbytes / BK;
+    const int KT = cur.nkt;
     kt_real = KT;
     load_scales(cur);
     const Tile nxt = decode(i + 1);
@@ -751,21 +790,21 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
         const int more = sgpr(kt + 2 < KTP ? 1 : 0);
         // step kt out of stage 0. Its first slice requests the token rows of step kt + 1 into stage 1 (the weight
         // rows of that step went out in the second slice of step kt - 1; step 1 was requested above).
-        fp8_a_loads_to1(sgpr(kt > 0 ? 1 : 0), rsrc4(ra4, kt + 1 < KT), sgpr((kt + 1) * BK));
+        fp8_a_loads_to1(sgpr(kt > 0 ? 1 : 0), rsrc4(ra4, kt + 1 < KT), sgpr(k_base + (kt + 1) * BK));
         fp8_b_s0k1();
         fp8_a();
         __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0): my loads of step kt + 1, my reads of stage 0
         __syncthreads();
-        fp8_b_even(more, rsrc4(rb04, true), rsrc4(rb14, true), sgpr((kt + 2) * BK));  // weights of step kt + 2 -> stage 0
+        fp8_b_even(more, rsrc4(rb04, true), rsrc4(rb14, true), sgpr(k_base + (kt + 2) * BK));  // weights of step kt + 2 -> stage 0
         // step kt + 1 out of stage 1
-        fp8_a_loads_to0(more, rsrc4(ra4, true), sgpr((kt + 2) * BK));                 // tokens of step kt + 2 -> stage 0
+        fp8_a_loads_to0(more, rsrc4(ra4, true), sgpr(k_base + (kt + 2) * BK));                 // tokens of step kt + 2 -> stage 0
         fp8_b_s1k1();
         fp8_a();
         if (more) {
           __builtin_amdgcn_s_waitcnt(0x0070);
           __syncthreads();
         }
-        fp8_b_odd(more, rsrc4(rb04, kt + 3 < KT), rsrc4(rb14, kt + 3 < KT), sgpr((kt + 3) * BK));  // weights of step kt + 3 -> stage 1
+        fp8_b_odd(more, rsrc4(rb04, kt + 3 < KT), rsrc4(rb14, kt + 3 < KT), sgpr(k_base + (kt + 3) * BK));  // weights of step kt + 3 -> stage 1
       }
     };
     [[maybe_unused]] auto k_loop = [&](auto full_c, int n_tt) {
@@ -798,6 +837,47 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
     }
     epilogue(cur);
     cur = nxt;
+  }
+}
+
+// ---- split K: adding the parts up ---------------------------------------------------------------------------
+// out[r, n] = bf16( (sum over parts of partial[p][r][n]) * scale(r) ), parts in ascending order (deterministic);
+// scale(r) = scale_input * scale_weight of the Linear of the group that owns row r (fp8), 1 for bf16 weights.
+struct SplitKReduceArgs {
+  const float* partial;     // [nparts][rows_dyn + rows_static][n_out]
+  long long part_stride;
+  int nparts, n_out, rows_dyn, rows_static, n_dyn, fp8;
+  const int32_t* offsets;   // segment bounds of the dynamic rows, n_dyn + 1 entries
+  const float* sw[MAX_GROUPS];   // scale_weight per group (fp8); the static group is entry n_dyn
+  const float* sin[MAX_GROUPS];  // scale_input per group or NULL
+  uint16_t* out_dyn;        // [rows_dyn, n_out] bf16
+  uint16_t* out_static;     // [rows_static, n_out] bf16
+};
+
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const SplitKReduceArgs a) {
+  const int rows = a.rows_dyn + a.rows_static;
+  const int per_row = a.n_out / 4;  // threads per row, 4 features each
+  const long long total = (long long)rows * per_row;
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long long)gridDim.x * blockDim.x) {
+    const int r = (int)(i / per_row), c = (int)(i % per_row) * 4;
+    int g = a.n_dyn;  // the static group
+    if (r < a.rows_dyn) {
+      g = 0;
+      while (g + 1 < a.n_dyn && r >= a.offsets[g + 1]) ++g;
+    }
+    float sc = 1.0f;
+    if (a.fp8) sc = (a.sin[g] ? *a.sin[g] : 1.0f) * *a.sw[g];
+    const float* src = a.partial + (size_t)r * a.n_out + c;
+    float4 s = *reinterpret_cast<const float4*>(src);
+    for (int p = 1; p < a.nparts; ++p) {
+      const float4 t = *reinterpret_cast<const float4*>(src + (size_t)p * (size_t)a.part_stride);
+      s.x += t.x; s.y += t.y; s.z += t.z; s.w += t.w;
+    }
+    uint2 o;
+    o.x = hdmoe_dev_pack_bf16(s.x * sc, s.y * sc);
+    o.y = hdmoe_dev_pack_bf16(s.z * sc, s.w * sc);
+    uint16_t* dst = r < a.rows_dyn ? a.out_dyn + (size_t)r * a.n_out + c : a.out_static + (size_t)(r - a.rows_dyn) * a.n_out + c;
+    *reinterpret_cast<uint2*>(dst) = o;
   }
 }
 
@@ -840,7 +920,8 @@ int hdmoe_launch_ffn_gemm(bool swiglu, int weight_dtype, const uint8_t* a_dyn, c
                           int n_dyn, const hdmoe_ffn_weights* experts, uint8_t* out_dyn, const uint8_t* a_static,
                           int rows_static, const hdmoe_ffn_weights* shared, uint8_t* out_static, int K_dyn, int N_dyn,
                           int K_static, int N_static, hipStream_t s, const char* what,
-                          const int32_t* gather_dyn = nullptr, int gather_rows = 0) {
+                          const int32_t* gather_dyn = nullptr, int gather_rows = 0, float* partial = nullptr,
+                          int nparts = 1) {
   const int eb = elem_bytes(weight_dtype);
   const bool fp8 = weight_dtype == HDMOE_W_E4M3FN;
   const int feat_per_tile = swiglu ? BN / 2 : BN;
@@ -853,13 +934,15 @@ int hdmoe_launch_ffn_gemm(bool swiglu, int weight_dtype, const uint8_t* a_dyn, c
     if (shared != nullptr && rows_static > 0) tiles += (long)((rows_static + bm - 1) / bm) * (N_static / feat_per_tile);
     return ((tiles + HDMOE_NUM_CU - 1) / HDMOE_NUM_CU) * (tt + 1);
   };
-  const bool tall = fp8 && expected_cost(5) < expected_cost(4);
+  const bool split = !swiglu && partial != nullptr && nparts > 1;  // split K runs on the 256-token tile
+  const bool tall = fp8 && !split && expected_cost(5) < expected_cost(4);
   const int BM = tall ? TileCfg<5>::BM : TileCfg<4>::BM;  // tokens per block tile of the kernel that will run
   if (gather_dyn != nullptr && (unsigned long long)gather_rows * K_dyn * eb >= (1ull << 31))
     return hdmoe_fail(HDMOE_E_SHAPE, "%s: %d gathered rows of %d bytes exceed the 2 GiB offset range", what, gather_rows,
                       K_dyn * eb);
   GemmArgs args;
   memset(&args, 0, sizeof(args));
+  args.nparts = 1;
   args.offsets = offsets;
   args.n_offsets = n_dyn;
   int G = 0, tile_bound = 0;
@@ -909,12 +992,86 @@ int hdmoe_launch_ffn_gemm(bool swiglu, int weight_dtype, const uint8_t* a_dyn, c
   args.G = G;
   // tiles of the static group are shorter or longer than the experts' when the two K differ (down projection)
   if (n_dyn > 0 && shared != nullptr && rows_static > 0 && K_static != K_dyn) args.spread = K_static < K_dyn ? 1 : -1;
+  if (split) {
+    // fp32 partial sums [nparts][rows_dyn + rows_static][N] (N_dyn == N_static is required), then the kernel that
+    // adds them up, applies the scales and rounds to bf16
+    if (n_dyn > 0 && shared != nullptr && rows_static > 0 && N_dyn != N_static)
+      return hdmoe_fail(HDMOE_E_SHAPE, "%s: split K needs one output width, got %d and %d", what, N_dyn, N_static);
+    const int N = n_dyn > 0 ? N_dyn : N_static;
+    const int rows_all = (n_dyn > 0 ? rows_dyn : 0) + ((shared != nullptr && rows_static > 0) ? rows_static : 0);
+    args.nparts = nparts;
+    args.part_stride = (long long)rows_all * N;
+    for (int g = 0; g < G; ++g)
+      args.g[g].pout = partial + (args.g[g].row_begin < 0 ? 0 : (size_t)(n_dyn > 0 ? rows_dyn : 0) * N);
+    tile_bound *= nparts;
+    const int rc = fp8 ? launch_grouped<FP8_PLAIN>(args, tile_bound, s, what) : launch_grouped<BF16_PLAIN>(args, tile_bound, s, what);
+    if (rc != HDMOE_OK) return rc;
+    SplitKReduceArgs ra;
+    memset(&ra, 0, sizeof(ra));
+    ra.partial = partial;
+    ra.part_stride = args.part_stride;
+    ra.nparts = nparts;
+    ra.n_out = N;
+    ra.rows_dyn = n_dyn > 0 ? rows_dyn : 0;
+    ra.rows_static = (shared != nullptr && rows_static > 0) ? rows_static : 0;
+    ra.n_dyn = n_dyn;
+    ra.fp8 = fp8 ? 1 : 0;
+    ra.offsets = offsets;
+    for (int g = 0; g < G; ++g) {
+      const int slot = args.g[g].row_begin < 0 ? args.g[g].dyn : n_dyn;
+      ra.sw[slot] = args.g[g].sb0;
+      ra.sin[slot] = args.g[g].s_in;
+    }
+    ra.out_dyn = reinterpret_cast<uint16_t*>(out_dyn);
+    ra.out_static = reinterpret_cast<uint16_t*>(out_static);
+    const long long work = (long long)rows_all * (N / 4);
+    int blocks = (int)((work + 255) / 256);
+    if (blocks > HDMOE_NUM_CU * 8) blocks = HDMOE_NUM_CU * 8;
+    if (blocks < 1) blocks = 1;
+    hipLaunchKernelGGL(splitk_reduce_kernel, dim3(blocks), dim3(256), 0, s, ra);
+    return hdmoe_check_launch(what);
+  }
   if (fp8 && tall) return swiglu ? launch_grouped<FP8_SWIGLU, 5>(args, tile_bound, s, what)
                                  : launch_grouped<FP8_PLAIN, 5>(args, tile_bound, s, what);
   if (fp8) return swiglu ? launch_grouped<FP8_SWIGLU>(args, tile_bound, s, what)
                          : launch_grouped<FP8_PLAIN>(args, tile_bound, s, what);
   return swiglu ? launch_grouped<BF16_SWIGLU>(args, tile_bound, s, what)
                 : launch_grouped<BF16_PLAIN>(args, tile_bound, s, what);
+}
+
+// How many K parts the down projection of a layer is cut into: a pure function of the sizes, so that the workspace
+// layout and the launch agree. With few tiles (small token counts) most CUs would idle through a long K loop.
+// Cost model in units of one K step of one tile: rounds of tiles over the CUs x (steps per part + a fixed 3 for
+// the tile's prologue and epilogue), expert segments taken 12 % more uneven than the mean; plus, when cut, the fp32
+// partial sums written and read again (8 bytes per output and part; they stay in the memory-side cache at these
+// sizes, about 10 TB/s; one step is about 1.4 us).
+int hdmoe_down_parts(int rows_dyn, int n_dyn, int rows_static, int N, int K_dyn, int K_static, int weight_dtype) {
+  const int eb = elem_bytes(weight_dtype);
+  const int bm = TileCfg<4>::BM;
+  double tiles = 0;
+  int kt = 0;
+  if (n_dyn > 0 && rows_dyn > 0) {
+    tiles += 1.12 * n_dyn * ((rows_dyn / n_dyn + bm - 1) / bm) * (N / BN);
+    kt = K_dyn * eb / BK;
+  }
+  if (rows_static > 0) {
+    tiles += (double)((rows_static + bm - 1) / bm) * (N / BN);
+    if (K_static * eb / BK > kt) kt = K_static * eb / BK;
+  }
+  if (tiles <= 0 || kt <= 0) return 1;
+  const double rows_all = (double)(n_dyn > 0 ? rows_dyn : 0) + rows_static;
+  const double reduce_steps_per_part = rows_all * N * 8.0 / 10e12 / 1.4e-6;
+  int best = 1;
+  double best_cost = 0;
+  for (int parts = 1; parts <= 6 && kt / parts >= 6; ++parts) {
+    const double rounds = (double)(long)((tiles * parts + HDMOE_NUM_CU - 1) / HDMOE_NUM_CU);
+    const double cost = rounds * ((double)kt / parts + 3.0) + (parts > 1 ? parts * reduce_steps_per_part : 0.0);
+    if (parts == 1 || cost < best_cost * 0.95) {  // a cut has to pay
+      best = parts;
+      best_cost = cost;
+    }
+  }
+  return best;
 }
 
 // Linear with bias and optional GELU over expert row segments plus an optional static group (bf16 weights):
@@ -925,6 +1082,7 @@ int hdmoe_launch_linear_groups(const uint8_t* a_dyn, const int32_t* offsets, int
                                int act, hipStream_t s, const char* what) {
   GemmArgs args;
   memset(&args, 0, sizeof(args));
+  args.nparts = 1;
   args.offsets = offsets;
   args.n_offsets = n_dyn;
   int G = 0, tile_bound = 0;
@@ -968,6 +1126,7 @@ int hdmoe_launch_linear_bias(int weight_dtype, const uint8_t* a, int rows, int K
   const bool fp8 = weight_dtype == HDMOE_W_E4M3FN;
   GemmArgs args;
   memset(&args, 0, sizeof(args));
+  args.nparts = 1;
   GemmGroup& gg = args.g[0];
   gg.a = a;
   gg.out = out;

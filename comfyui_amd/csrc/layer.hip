@@ -8,7 +8,9 @@ int hdmoe_launch_ffn_gemm(bool swiglu, int weight_dtype, const uint8_t* a_dyn, c
                           int n_dyn, const hdmoe_ffn_weights* experts, uint8_t* out_dyn, const uint8_t* a_static,
                           int rows_static, const hdmoe_ffn_weights* shared, uint8_t* out_static, int K_dyn, int N_dyn,
                           int K_static, int N_static, hipStream_t s, const char* what,
-                          const int32_t* gather_dyn = nullptr, int gather_rows = 0);
+                          const int32_t* gather_dyn = nullptr, int gather_rows = 0, float* partial = nullptr,
+                          int nparts = 1);
+int hdmoe_down_parts(int rows_dyn, int n_dyn, int rows_static, int N, int K_dyn, int K_static, int weight_dtype);
 int hdmoe_check_gemm_shape(const char* what, int weight_dtype, long rows, int K, int N, int feat_per_tile);
 int hdmoe_launch_quant_dispatch(const void* x_bf16, const int32_t* perm, const int32_t* offsets, int T, int D, int E,
                                 const float* const* scale_input, const float* shared_scale, bool with_shared,
@@ -58,6 +60,9 @@ extern "C" int hdmoe_layer_layout_get(int T, int D, int H, int Hs, int E, int we
   out->y = take((n + (Hs > 0 ? (size_t)T : 0)) * D * 2);
   // normalised + modulated tokens of the optional block fusion, [T,D] bf16
   out->normed = take((size_t)T * D * 2);
+  // fp32 partial sums of a down projection cut along K (small token counts), [parts][2T + T][D]
+  const int parts = hdmoe_down_parts((int)n, E, Hs > 0 ? T : 0, D, H, Hs, weight_dtype);
+  out->partials = take(parts > 1 ? (size_t)parts * (n + (Hs > 0 ? (size_t)T : 0)) * D * 4 : 0);
   out->total = off;
   return HDMOE_OK;
 }
@@ -181,8 +186,10 @@ extern "C" int hdmoe_moe_ffn(const hdmoe_layer_args* p, hdmoe_stream_t stream) {
     return rc;
   mark();
   // down projections, both in one launch
+  const int parts = hdmoe_down_parts((int)n, E, Hs > 0 ? T : 0, D, H, Hs, wd);
   if (int rc = hdmoe_launch_ffn_gemm(false, wd, h_routed, offsets, (int)n, E, p->experts, y_routed, h_shared,
-                                     Hs > 0 ? T : 0, p->shared, y_shared, H, D, Hs, D, s, "hdmoe_moe_ffn (down)"))
+                                     Hs > 0 ? T : 0, p->shared, y_shared, H, D, Hs, D, s, "hdmoe_moe_ffn (down)",
+                                     nullptr, 0, parts > 1 ? reinterpret_cast<float*>(ws + l.partials) : nullptr, parts))
     return rc;
   mark();
   const int rc = hdmoe_launch_combine(y_routed, inv_perm, tw, Hs > 0 ? y_shared : nullptr,
@@ -197,9 +204,12 @@ extern "C" int hdmoe_moe_ffn(const hdmoe_layer_args* p, hdmoe_stream_t stream) {
 extern "C" size_t hdmoe_ffn_workspace_bytes(int rows, int D, int H, int weight_dtype) {
   if (rows < 0 || D <= 0 || H <= 0 || (weight_dtype != HDMOE_W_BF16 && weight_dtype != HDMOE_W_E4M3FN)) return 0;
   const size_t eb = weight_dtype == HDMOE_W_E4M3FN ? 1 : 2;
-  // fp8: quantised copy of x, then h; bf16: h only (x itself is the GEMM operand)
+  // fp8: quantised copy of x, then h; bf16: h only (x itself is the GEMM operand); then the fp32 partial sums of a
+  // down projection cut along K (few rows)
   const size_t a = weight_dtype == HDMOE_W_E4M3FN ? hdmoe_align_up((size_t)rows * D * eb, 256) : 0;
-  return a + hdmoe_align_up((size_t)rows * H * eb, 256);
+  const int parts = hdmoe_down_parts(0, 0, rows, D, 0, H, weight_dtype);
+  const size_t pbytes = parts > 1 ? hdmoe_align_up((size_t)parts * rows * D * 4, 256) : 0;
+  return a + hdmoe_align_up((size_t)rows * H * eb, 256) + pbytes;
 }
 
 extern "C" int hdmoe_ffn_swiglu(int weight_dtype, const void* x_bf16, int rows, int D, int H,
@@ -231,6 +241,9 @@ extern "C" int hdmoe_ffn_swiglu(int weight_dtype, const void* x_bf16, int rows, 
   if (int rc = hdmoe_launch_ffn_gemm(true, weight_dtype, nullptr, nullptr, 0, 0, nullptr, nullptr, a, rows, w, h, 0, 0, D, H,
                                      s, "hdmoe_ffn_swiglu (gate/up)"))
     return rc;
+  const int parts = hdmoe_down_parts(0, 0, rows, D, 0, H, weight_dtype);
+  float* partial = parts > 1 ? reinterpret_cast<float*>(h + hdmoe_align_up((size_t)rows * H * (fp8 ? 1 : 2), 256)) : nullptr;
   return hdmoe_launch_ffn_gemm(false, weight_dtype, nullptr, nullptr, 0, 0, nullptr, nullptr, h, rows, w,
-                               static_cast<uint8_t*>(out_bf16), 0, 0, H, D, s, "hdmoe_ffn_swiglu (down)");
+                               static_cast<uint8_t*>(out_bf16), 0, 0, H, D, s, "hdmoe_ffn_swiglu (down)", nullptr, 0,
+                               partial, parts);
 }

@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define HDMOE_VERSION 107
+#define HDMOE_VERSION 108
 
 #define HDMOE_OK 0
 #define HDMOE_E_NULL (-1)      /* required pointer is NULL */
@@ -283,7 +283,7 @@ int hdmoe_ffn_swiglu(int weight_dtype, const void* x_bf16, int rows, int D, int 
 /* Where the pieces of the workspace live, for tests that inspect intermediates. */
 typedef struct hdmoe_layer_layout {
   size_t topk_idx, topk_weight, counts, offsets, perm, inv_perm, dispatch_ws;
-  size_t a, h, y, normed, total;
+  size_t a, h, y, normed, partials, total;
 } hdmoe_layer_layout;
 int hdmoe_layer_layout_get(int T, int D, int H, int Hs, int E, int weight_dtype,
                            hdmoe_layer_layout* out);
