@@ -56,7 +56,7 @@ class LayerArgs(ctypes.Structure):
         ("topk_idx", c_void_p), ("topk_weight", c_void_p),
         ("stage_events", ctypes.POINTER(c_void_p)),
         ("mod_scale", c_void_p), ("mod_shift", c_void_p), ("mod_gate", c_void_p),
-        ("tokens_per_batch", c_int), ("ln_eps", ctypes.c_float),
+        ("tokens_per_batch", c_int), ("ln_eps", ctypes.c_float), ("uniform_scale_in", c_int),
     ]
 
 

@@ -180,7 +180,8 @@ __device__ __forceinline__ void ln_stats(const uint4 (&v)[NCHUNK], float fD, flo
 
 // D == NCHUNK * 512: the lane's Wg slice lives in registers.
 // Optional second output of both kernels (QUANT): the token's fp8 rows for the expert GEMMs, cast while the row
-// is at hand. Row 2t+s of xq_routed is x[t] cast with the scale_input of the expert in slot s, row t of xq_shared
+// is at hand. Row 2t+s of xq_routed (NULL: every Linear that reads the tokens shares one scale_input, the shared copy
+// serves them all) is x[t] cast with the scale_input of the expert in slot s, row t of xq_shared
 // the cast for the shared expert; the GEMM reads them through the dispatch permutation.
 struct GateQuant {
   HdmoeScalePtrs scale_in;    // per expert, NULL = clamp rule
@@ -196,18 +197,19 @@ struct GateQuant {
 };
 
 template <int E, int NCHUNK, bool QUANT, bool LN = false>
-__global__ __launch_bounds__(WAVES_PER_BLOCK * 64, LN ? 2 : 1) void gate_top2_reg_kernel(
+__global__ __launch_bounds__(WAVES_PER_BLOCK * 64, 3) void gate_top2_reg_kernel(
     const uint4* __restrict__ x, const uint4* __restrict__ wg, int T, int32_t* __restrict__ idx,
     uint16_t* __restrict__ wout, GateQuant q) {
   const int lane = threadIdx.x & 63;
   const int wave = blockIdx.x * WAVES_PER_BLOCK + (threadIdx.x >> 6);
   const int nwaves = gridDim.x * WAVES_PER_BLOCK;
   constexpr int ROW16 = NCHUNK * 64;  // 16-byte units per row
-  uint4 w[E][NCHUNK];
-#pragma unroll
-  for (int e = 0; e < E; ++e)
-#pragma unroll
-    for (int c = 0; c < NCHUNK; ++c) w[e][c] = wg[(size_t)e * ROW16 + c * 64 + lane];
+  // The gate weight (E rows) sits in LDS, not in registers: 80 registers less per lane, i.e. four waves per SIMD
+  // instead of two, which is what a kernel that only streams needs. A lane reads the same 16-byte units of every
+  // row for every token (lane-contiguous, conflict-free).
+  __shared__ uint4 w[E * ROW16];
+  for (int i = threadIdx.x; i < E * ROW16; i += WAVES_PER_BLOCK * 64) w[i] = wg[i];
+  __syncthreads();
 
   int t = wave;
   if (t >= T) return;
@@ -237,15 +239,16 @@ __global__ __launch_bounds__(WAVES_PER_BLOCK * 64, LN ? 2 : 1) void gate_top2_re
         cur[c] = modulate8(cur[c], q.mod_scale[brow + c * 64 + lane], q.mod_shift[brow + c * 64 + lane], mean, rstd);
     }
     float logit[E];
+    // opaque per token, or the compiler hoists the E * NCHUNK weight reads out of the token loop and keeps the
+    // slice in registers after all
+    int wlane = lane;
+    asm volatile("" : "+v"(wlane));
 #pragma unroll
     for (int e = 0; e < E; ++e) {
       float acc = 0.0f;
 #pragma unroll
       for (int c = 0; c < NCHUNK; ++c) {
-        // keep the weight slice packed (bf16 pairs): without this the compiler hoists the unpacking out of the
-        // token loop and doubles the register footprint, which halves the waves in flight
-        asm volatile("" : "+v"(w[e][c].x), "+v"(w[e][c].y), "+v"(w[e][c].z), "+v"(w[e][c].w));
-        acc = dot8(cur[c], w[e][c], acc);
+        acc = dot8(cur[c], w[e * ROW16 + c * 64 + wlane], acc);
       }
       logit[e] = acc;
     }
@@ -260,15 +263,21 @@ __global__ __launch_bounds__(WAVES_PER_BLOCK * 64, LN ? 2 : 1) void gate_top2_re
       }
       inv0 = hdmoe_q_uniform(inv0);
       inv1 = hdmoe_q_uniform(inv1);
-      uint2* r0 = q.xq_routed + (size_t)(2 * t) * ROW16;
-      const bool same01 = inv0 == inv1, same0s = inv0 == invs;  // equal scales: cast once, store again
+      if (q.xq_routed == nullptr) {
+        // one scale_input for all: one row per token
 #pragma unroll
-      for (int c = 0; c < NCHUNK; ++c) {
-        const uint2 v0 = hdmoe_q_8(cur[c], inv0);
-        r0[c * 64 + lane] = v0;
-        r0[ROW16 + c * 64 + lane] = same01 ? v0 : hdmoe_q_8(cur[c], inv1);
-        if (q.xq_shared != nullptr)
-          q.xq_shared[(size_t)t * ROW16 + c * 64 + lane] = same0s ? v0 : hdmoe_q_8(cur[c], invs);
+        for (int c = 0; c < NCHUNK; ++c) q.xq_shared[(size_t)t * ROW16 + c * 64 + lane] = hdmoe_q_8(cur[c], invs);
+      } else {
+        uint2* r0 = q.xq_routed + (size_t)(2 * t) * ROW16;
+        const bool same01 = inv0 == inv1, same0s = inv0 == invs;  // equal scales: cast once, store again
+#pragma unroll
+        for (int c = 0; c < NCHUNK; ++c) {
+          const uint2 v0 = hdmoe_q_8(cur[c], inv0);
+          r0[c * 64 + lane] = v0;
+          r0[ROW16 + c * 64 + lane] = same01 ? v0 : hdmoe_q_8(cur[c], inv1);
+          if (q.xq_shared != nullptr)
+            q.xq_shared[(size_t)t * ROW16 + c * 64 + lane] = same0s ? v0 : hdmoe_q_8(cur[c], invs);
+        }
       }
     }
 #pragma unroll
@@ -302,8 +311,10 @@ __global__ __launch_bounds__(WAVES_PER_BLOCK * 64) void gate_top2_generic_kernel
       const float invs = hdmoe_q_uniform(hdmoe_q_inv_scale(q.shared_scale));
       for (int u = lane; u < row16; u += 64) {
         const uint4 xv = x[(size_t)t * row16 + u];
-        q.xq_routed[(size_t)(2 * t) * row16 + u] = hdmoe_q_8(xv, inv0);
-        q.xq_routed[(size_t)(2 * t + 1) * row16 + u] = hdmoe_q_8(xv, inv1);
+        if (q.xq_routed != nullptr) {
+          q.xq_routed[(size_t)(2 * t) * row16 + u] = hdmoe_q_8(xv, inv0);
+          q.xq_routed[(size_t)(2 * t + 1) * row16 + u] = hdmoe_q_8(xv, inv1);
+        }
         if (q.xq_shared != nullptr) q.xq_shared[(size_t)t * row16 + u] = hdmoe_q_8(xv, invs);
       }
     }
@@ -313,11 +324,12 @@ __global__ __launch_bounds__(WAVES_PER_BLOCK * 64) void gate_top2_generic_kernel
 template <int E>
 int launch_gate(const void* x, const void* wg, int T, int D, int32_t* idx, void* w, const GateQuant* quant,
                 hipStream_t s, const char* what) {
-  // about 4 tokens per wave amortise the register-resident weight slice and still give 8 waves per CU at T = 8192
-  constexpr int TOKENS_PER_WAVE = 4;
+  // at least two tokens per wave amortise the block's copy of the gate weight into LDS; at most three blocks per CU,
+  // which is what the register kernels' 12 waves per CU hold at once (the waves stride over the tokens)
+  constexpr int TOKENS_PER_WAVE = 2;
   int blocks = (T + WAVES_PER_BLOCK * TOKENS_PER_WAVE - 1) / (WAVES_PER_BLOCK * TOKENS_PER_WAVE);
   if (blocks < 1) blocks = 1;
-  if (blocks > HDMOE_NUM_CU * 8) blocks = HDMOE_NUM_CU * 8;
+  if (blocks > HDMOE_NUM_CU * 3) blocks = HDMOE_NUM_CU * 3;
   dim3 grid(blocks), block(WAVES_PER_BLOCK * 64);
   const uint4* xp = static_cast<const uint4*>(x);
   const uint4* wp = static_cast<const uint4*>(wg);

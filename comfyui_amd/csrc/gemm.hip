@@ -64,7 +64,8 @@ enum Mode { FP8_SWIGLU = 0, FP8_PLAIN = 1, BF16_SWIGLU = 2, BF16_PLAIN = 3, BF16
 
 struct GemmGroup {
   const uint8_t* a;     // activations; row indices below are relative to this base
-  const int32_t* gather;  // NULL: row r of the group is row r of a; else it is row gather[r] of a (a_rows rows)
+  const int32_t* gather;  // NULL: row r of the group is row r of a; else it is row gather[r] >> gather_shift of a (a_rows rows)
+  int gather_shift;       // 1: gather holds flat slots 2t+s and a has one row per token
   int a_rows;
   const uint8_t* b0;    // plain: W [N,K]; swiglu: w1 [H,K]
   const uint8_t* b1;    // swiglu: w3 [H,K]
@@ -324,7 +325,7 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
 #pragma unroll
     for (int j = 0; j < A_SLABS; ++j) {
       const int r = j * 64 + ld_row;
-      gi[j] = (gg.gather != nullptr && r < d.rows_here) ? gg.gather[d.row0 + r] : -1;
+      gi[j] = (gg.gather != nullptr && r < d.rows_here) ? (gg.gather[d.row0 + r] >> gg.gather_shift) : -1;
     }
   };
   // the same three resources as plain descriptor words, for the loads issued from the assembly blocks
@@ -921,7 +922,7 @@ int hdmoe_launch_ffn_gemm(bool swiglu, int weight_dtype, const uint8_t* a_dyn, c
                           int rows_static, const hdmoe_ffn_weights* shared, uint8_t* out_static, int K_dyn, int N_dyn,
                           int K_static, int N_static, hipStream_t s, const char* what,
                           const int32_t* gather_dyn = nullptr, int gather_rows = 0, float* partial = nullptr,
-                          int nparts = 1) {
+                          int nparts = 1, int gather_shift = 0) {
   const int eb = elem_bytes(weight_dtype);
   const bool fp8 = weight_dtype == HDMOE_W_E4M3FN;
   const int feat_per_tile = swiglu ? BN / 2 : BN;
@@ -951,6 +952,7 @@ int hdmoe_launch_ffn_gemm(bool swiglu, int weight_dtype, const uint8_t* a_dyn, c
     const hdmoe_ffn_weights& w = experts[e];
     gg.a = a_dyn;
     gg.gather = gather_dyn;
+    gg.gather_shift = gather_shift;
     gg.a_rows = gather_rows;
     gg.out = out_dyn;
     gg.row_begin = -1;

@@ -9,7 +9,7 @@ int hdmoe_launch_ffn_gemm(bool swiglu, int weight_dtype, const uint8_t* a_dyn, c
                           int rows_static, const hdmoe_ffn_weights* shared, uint8_t* out_static, int K_dyn, int N_dyn,
                           int K_static, int N_static, hipStream_t s, const char* what,
                           const int32_t* gather_dyn = nullptr, int gather_rows = 0, float* partial = nullptr,
-                          int nparts = 1);
+                          int nparts = 1, int gather_shift = 0);
 int hdmoe_down_parts(int rows_dyn, int n_dyn, int rows_static, int N, int K_dyn, int K_static, int weight_dtype);
 int hdmoe_check_gemm_shape(const char* what, int weight_dtype, long rows, int K, int N, int feat_per_tile);
 int hdmoe_launch_quant_dispatch(const void* x_bf16, const int32_t* perm, const int32_t* offsets, int T, int D, int E,
@@ -150,14 +150,32 @@ extern "C" int hdmoe_moe_ffn(const hdmoe_layer_args* p, hdmoe_stream_t stream) {
       return rc;
     xin = normed;
   }
-  // fp8 experts: the gate kernel also casts each token to e4m3fn for its two experts (rows 2t, 2t+1 of a_routed,
-  // i.e. in flat slot order) and for the shared expert while it holds the row; the gate/up GEMM then reads the
-  // routed rows through the permutation instead of from a permuted copy.
+  // fp8 experts: the gate kernel also casts each token to e4m3fn while it holds the row. When every Linear that reads
+  // the tokens (w1/w3 of every routed expert and of the shared expert) has the same scale_input, one row per token
+  // serves them all and the gate/up GEMM reads row perm[r] / 2 of it. Otherwise the token is cast for its two experts
+  // (rows 2t, 2t+1 of a_routed, i.e. in flat slot order) and for the shared expert, and the GEMM reads the routed rows
+  // through the permutation instead of from a permuted copy.
+  bool one_copy = false;
+  if (fp8) {
+    one_copy = true;
+    const float* first = p->experts[0].scale_in1;
+    for (int e = 1; e < E; ++e) one_copy = one_copy && p->experts[e].scale_in1 == first;
+    if (Hs > 0) one_copy = one_copy && p->shared->scale_in1 == first;
+    one_copy = one_copy || p->uniform_scale_in != 0;
+    // a mix of NULL (clamp rule) and non-NULL scale_inputs is never uniform, whatever the caller says
+    for (int e = 0; e < E; ++e) one_copy = one_copy && ((p->experts[e].scale_in1 == nullptr) == (first == nullptr));
+    if (Hs > 0) one_copy = one_copy && ((p->shared->scale_in1 == nullptr) == (first == nullptr));
+  }
   if (fp8) {
     const float* sin[HDMOE_MAX_EXPERTS];
     for (int e = 0; e < E; ++e) sin[e] = p->experts[e].scale_in1;
-    if (int rc = hdmoe_launch_gate_quant(xin, p->gate_w, T, D, E, idx, tw, sin, Hs > 0 ? p->shared->scale_in1 : nullptr,
-                                         a_routed, Hs > 0 ? a_shared : nullptr, s, "hdmoe_moe_ffn (gate + quantise)",
+    const float* token_scale = (Hs > 0 && !one_copy) ? p->shared->scale_in1 : p->experts[0].scale_in1;
+    // the one copy sits where the shared expert's copy would (without a shared expert that room does not exist: the
+    // start of the routed rows' room then)
+    if (one_copy && Hs == 0) a_shared = a_routed;
+    if (int rc = hdmoe_launch_gate_quant(xin, p->gate_w, T, D, E, idx, tw, sin, (Hs > 0 || one_copy) ? token_scale : nullptr,
+                                         one_copy ? nullptr : a_routed, (Hs > 0 || one_copy) ? a_shared : nullptr, s,
+                                         "hdmoe_moe_ffn (gate + quantise)",
                                          ln_in_gate ? p->mod_scale : nullptr, ln_in_gate ? p->mod_shift : nullptr,
                                          p->tokens_per_batch, p->ln_eps))
       return rc;
@@ -180,9 +198,10 @@ extern "C" int hdmoe_moe_ffn(const hdmoe_layer_args* p, hdmoe_stream_t stream) {
 
   mark();
   // gate/up projections + SiLU*mul, routed experts and shared expert in one launch
-  if (int rc = hdmoe_launch_ffn_gemm(true, wd, a_routed, offsets, (int)n, E, p->experts, h_routed, a_static,
-                                     Hs > 0 ? T : 0, p->shared, h_shared, D, H, D, Hs, s, "hdmoe_moe_ffn (gate/up)",
-                                     fp8 ? perm : nullptr, (int)n))
+  if (int rc = hdmoe_launch_ffn_gemm(true, wd, one_copy ? a_shared : a_routed, offsets, (int)n, E, p->experts, h_routed,
+                                     a_static, Hs > 0 ? T : 0, p->shared, h_shared, D, H, D, Hs, s,
+                                     "hdmoe_moe_ffn (gate/up)", fp8 ? perm : nullptr, one_copy ? T : (int)n, nullptr, 1,
+                                     one_copy ? 1 : 0))
     return rc;
   mark();
   // down projections, both in one launch

@@ -198,6 +198,15 @@ class MOEFeedForwardSwiGLU(nn.Module):
             if fw is None:
                 return None
             packed.append(fw)
+        # one scale_input value for every Linear that reads the tokens: they are cast to fp8 once
+        self._uniform_scale_in = False
+        if wdt == FP8:
+            sis = [getattr(f.w1, "scale_input", None) for f in ffns]
+            if all(si is None for si in sis):
+                self._uniform_scale_in = True
+            elif all(si is not None for si in sis):
+                v0 = amd_ops.scale_value(sis[0])
+                self._uniform_scale_in = all(amd_ops.scale_value(si) == v0 for si in sis[1:])
         return wdt, packed[:-1], packed[-1], keep
 
     def forward(self, x, stage_events=None):
@@ -215,7 +224,8 @@ class MOEFeedForwardSwiGLU(nn.Module):
             wdt, experts, shared, keep = got
             H = self.experts[0].w1.weight.shape[0]
             Hs = self.shared_experts.w1.weight.shape[0]
-            y = HF.moe_ffn(x2, gate_w, experts, shared, H, Hs, wdt, stage_events=stage_events)
+            y = HF.moe_ffn(x2, gate_w, experts, shared, H, Hs, wdt, stage_events=stage_events,
+                           uniform_scale_in=self._uniform_scale_in)
             del keep
             return y.view(*orig_shape)
         return self._forward_composed(x2, gate_w).view(*orig_shape)
@@ -239,6 +249,7 @@ class MOEFeedForwardSwiGLU(nn.Module):
             H = self.experts[0].w1.weight.shape[0]
             Hs = self.shared_experts.w1.weight.shape[0]
             y = HF.moe_ffn(x2, gate_w, experts, shared, H, Hs, wdt, stage_events=stage_events, modulation=mods,
+                           uniform_scale_in=self._uniform_scale_in,
                            tokens_per_batch=S, ln_eps=eps)
             del keep
             return y.view(B, S, D)

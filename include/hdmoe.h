@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define HDMOE_VERSION 108
+#define HDMOE_VERSION 109
 
 #define HDMOE_OK 0
 #define HDMOE_E_NULL (-1)      /* required pointer is NULL */
@@ -261,6 +261,11 @@ typedef struct hdmoe_layer_args {
   const void* mod_gate;
   int tokens_per_batch;
   float ln_eps;
+  /* fp8 only. When w1/w3 of every routed expert and of the shared expert have the same scale_input, the tokens are
+   * cast to e4m3fn once (one row per token instead of three) and every group of the gate/up GEMM reads that copy.
+   * The library sees this by itself when all those scale_in1 pointers are equal (all NULL included); nonzero here is
+   * the caller's assertion that different pointers hold the same value. */
+  int uniform_scale_in;
 } hdmoe_layer_args;
 
 #define HDMOE_NUM_STAGES 6
