@@ -32,10 +32,20 @@ PEAK_FP8_TFLOPS = 5000.0    # MI355X dense fp8 MFMA
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBPS = 8000.0      # MI355X HBM3E
 
-# L2-side traffic of the dominant kernel per launch (bytes fetched + written), from the two rocprofv3 --pmc runs
-# summarised in profiles/bench_cfg3_pmc.txt (FETCH_SIZE x 2.000 and WRITE_SIZE x 1.000 after calibration against a
-# plain 256 MiB copy). Only known for the workload that was profiled.
-MEASURED_TRAFFIC_BYTES = {"cfg3": 1084.5e6 + 145.8e6}
+
+
+def measured_traffic(workload):
+    """L2-side traffic of the dominant kernel per launch (bytes fetched + written) as the last rocprofv3 --pmc runs
+    measured it: profiles/traffic.json holds, per workload, the calibrated FETCH_SIZE and WRITE_SIZE readings, the
+    commit they were taken at and the summary file they come from. None for a workload that was not profiled."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
+            entry = json.load(f).get(workload)
+    except (OSError, ValueError):
+        return None, None
+    if not entry:
+        return None, None
+    return entry["fetch_bytes"] + entry["write_bytes"], entry
 
 
 class HipEvents:
@@ -277,12 +287,14 @@ def main():
     eb = 1 if fp8 else 2
     gate_bytes = T * D * 2 + E * D * 2 + T * 2 * (4 + 2)
     # dispatch as built: index sort (read 2T ids twice, write perm + inv_perm). fp8: the gate kernel also writes the
-    # token's three e4m3fn rows (two routed slots + shared expert), and nothing is permuted; bf16: the routed rows are
-    # materialised in expert order (read + write 2T rows).
-    dispatch_bytes = 2 * (2 * T * 4) + 2 * (2 * T * 4) + (3 * T * D if fp8 else 2 * (2 * T * D * 2))
+    # token's e4m3fn row, once, because every scale_input of these configurations is the same value (it would be three
+    # rows, two routed slots + shared expert, with differing scales), and nothing is permuted; bf16: the routed rows
+    # are materialised in expert order (read + write 2T rows).
+    dispatch_bytes = 2 * (2 * T * 4) + 2 * (2 * T * 4) + (T * D if fp8 else 2 * (2 * T * D * 2))
     gd_ms = stage_ms["gate"] + stage_ms["dispatch"] + stage_ms["quant_permute"]
     combine_bytes = 2 * T * D * 2 + T * D * 2 + T * D * 2 + T * 2 * 2 + 2 * T * 4
 
+    traffic_bytes, traffic_entry = measured_traffic(args.workload)
     out = {
         "metric": "MoE-FFN tokens/sec at 8192 tok fp8" if args.workload == "cfg3" else f"MoE-FFN tokens/sec ({args.workload})",
         "value": tokens_per_s,
@@ -329,8 +341,9 @@ def main():
             "peak": peak,
             "unit": "TFLOP/s",
             "frac": gemm1_tflops / peak,
-            "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
-            "traffic_note": "rocprofv3 FETCH_SIZE+WRITE_SIZE per launch, calibrated; see profiles/bench_cfg3_pmc.txt",
+            "traffic": traffic_bytes,
+            "traffic_note": ("rocprofv3 FETCH_SIZE + WRITE_SIZE per launch, calibrated against a plain copy; taken at commit "
+                             f"{traffic_entry['commit']}, see profiles/{traffic_entry['source']}") if traffic_entry else None,
             "algorithmic_bytes": T * (3 * D * eb + (2 * H + Hs) * eb) + (E * 2 * H + 2 * Hs) * D * eb,
             "flop_per_launch": T * fl["gate_up"],
             "avg_launch_ms": stage_ms["gemm_gate_up"],
