@@ -72,6 +72,7 @@ SIGNATURES = {
     "hdmoe_version": (c_int, []),
     "hdmoe_last_error": (ctypes.c_char_p, []),
     "hdmoe_gate_top2": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),
+    "hdmoe_renorm_top2_bf16": (c_int, [c_void_p, c_int, c_void_p, c_void_p]),
     "hdmoe_dispatch_workspace_bytes": (c_size_t, [c_int, c_int]),
     "hdmoe_dispatch": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t,
                                c_void_p]),
@@ -89,6 +90,7 @@ SIGNATURES = {
     "hdmoe_linear_bias": (c_int, [c_int, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                   c_void_p]),
     "hdmoe_silu_mul_bf16": (c_int, [c_void_p, c_void_p, c_int64, c_void_p, c_void_p]),
+    "hdmoe_gelu_bf16": (c_int, [c_void_p, c_int64, c_void_p, c_void_p]),
     "hdmoe_scale_to_bf16": (c_int, [c_int, c_void_p, c_int64, c_void_p, c_void_p, c_void_p]),
     "hdmoe_grouped_linear": (c_int, [c_void_p, c_void_p, c_int, c_int, ctypes.POINTER(LinearWeights), c_void_p, c_void_p,
                                      c_int, ctypes.POINTER(LinearWeights), c_void_p, c_int, c_int, c_int, c_void_p]),

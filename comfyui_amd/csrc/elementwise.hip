@@ -118,6 +118,36 @@ __global__ __launch_bounds__(THREADS) void silu_mul_kernel(const uint4* __restri
   }
 }
 
+// F.gelu (erf form) of a bf16 tensor, evaluated in fp32 and rounded once
+// (/root/reference/comfy/ldm/hunyuan3dv2_1/hunyuandit.py:14-26), for projections whose Linear is not the plain bf16 one.
+__device__ __forceinline__ float gelu1(float h) { return 0.5f * h * (1.0f + erff(h * 0.70710678118654752440f)); }
+
+__global__ __launch_bounds__(THREADS) void gelu_kernel(const uint4* __restrict__ x, int64_t n8, uint4* __restrict__ out) {
+  for (int64_t i = blockIdx.x * (int64_t)THREADS + threadIdx.x; i < n8; i += (int64_t)gridDim.x * THREADS) {
+    const uint4 v = x[i];
+    uint4 o;
+    o.x = pack_bf16(gelu1(bf16_lo(v.x)), gelu1(bf16_hi(v.x)));
+    o.y = pack_bf16(gelu1(bf16_lo(v.y)), gelu1(bf16_hi(v.y)));
+    o.z = pack_bf16(gelu1(bf16_lo(v.z)), gelu1(bf16_hi(v.z)));
+    o.w = pack_bf16(gelu1(bf16_lo(v.w)), gelu1(bf16_hi(v.w)));
+    out[i] = o;
+  }
+}
+
+// topk_weight / (topk_weight.sum(-1, keepdim=True) + 1e-20) on a [T, 2] bf16 tensor
+// (/root/reference/comfy/ldm/hidream/model.py:277-280): the sum is rounded to bf16, the scalar is added in fp32 and the
+// result rounded to bf16 again, then each quotient is rounded to bf16, as the three torch ops do.
+__global__ __launch_bounds__(THREADS) void renorm_top2_kernel(const uint32_t* __restrict__ w, int T,
+                                                              uint32_t* __restrict__ out) {
+  for (int t = blockIdx.x * THREADS + threadIdx.x; t < T; t += gridDim.x * THREADS) {
+    const uint32_t v = w[t];
+    const float w0 = bf16_lo(v), w1 = bf16_hi(v);
+    const float sum = __uint_as_float(pack_bf16(w0 + w1, 0.0f) << 16);
+    const float den = __uint_as_float(pack_bf16(sum + 1e-20f, 0.0f) << 16);
+    out[t] = pack_bf16(__fdiv_rn(w0, den), __fdiv_rn(w1, den));
+  }
+}
+
 // (y.view(T,2,D) * w.unsqueeze(-1)).sum(1) + shared at bf16
 // (/root/reference/comfy/ldm/hidream/model.py:319,324): each product is rounded to
 // bf16, the two-term sum is formed in fp32 and rounded, then the shared row is added
@@ -311,6 +341,31 @@ extern "C" int hdmoe_silu_mul_bf16(const void* a_bf16, const void* b_bf16, int64
                      static_cast<const uint4*>(a_bf16), static_cast<const uint4*>(b_bf16), n16,
                      static_cast<uint4*>(out_bf16));
   return hdmoe_check_launch("hdmoe_silu_mul_bf16");
+}
+
+extern "C" int hdmoe_gelu_bf16(const void* x_bf16, int64_t n, void* out_bf16, hdmoe_stream_t stream) {
+  HDMOE_REQUIRE_PTR(x_bf16);
+  HDMOE_REQUIRE_PTR(out_bf16);
+  if (n < 0 || n % 8 != 0) return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_gelu_bf16: n=%lld must be a multiple of 8", (long long)n);
+  if (n == 0) return HDMOE_OK;
+  const int64_t n8 = n / 8;
+  int64_t blocks = (n8 + THREADS - 1) / THREADS;
+  if (blocks > HDMOE_NUM_CU * 8) blocks = HDMOE_NUM_CU * 8;
+  hipLaunchKernelGGL(gelu_kernel, dim3((unsigned)blocks), dim3(THREADS), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const uint4*>(x_bf16), n8, static_cast<uint4*>(out_bf16));
+  return hdmoe_check_launch("hdmoe_gelu_bf16");
+}
+
+extern "C" int hdmoe_renorm_top2_bf16(const void* topk_weight_bf16, int T, void* out_bf16, hdmoe_stream_t stream) {
+  HDMOE_REQUIRE_PTR(topk_weight_bf16);
+  HDMOE_REQUIRE_PTR(out_bf16);
+  if (T < 0) return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_renorm_top2_bf16: T=%d", T);
+  if (T == 0) return HDMOE_OK;
+  int blocks = (T + THREADS - 1) / THREADS;
+  if (blocks > HDMOE_NUM_CU * 4) blocks = HDMOE_NUM_CU * 4;
+  hipLaunchKernelGGL(renorm_top2_kernel, dim3(blocks), dim3(THREADS), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const uint32_t*>(topk_weight_bf16), T, static_cast<uint32_t*>(out_bf16));
+  return hdmoe_check_launch("hdmoe_renorm_top2_bf16");
 }
 
 int hdmoe_launch_combine(const void* y_sorted_bf16, const int32_t* inv_perm, const void* topk_weight_bf16,

@@ -50,6 +50,18 @@ def gate_top2(x2d, gate_w):
     return idx, w
 
 
+def renorm_top2(topk_weight):
+    """topk_weight / (topk_weight.sum(-1, keepdim=True) + 1e-20) for the [T, 2] bf16 gate weights."""
+    _need_hip(topk_weight, "renorm_top2 topk_weight", BF16)
+    if topk_weight.dim() != 2 or topk_weight.shape[1] != 2 or not topk_weight.is_contiguous():
+        raise ValueError("renorm_top2: expected a contiguous [T, 2] tensor")
+    out = torch.empty_like(topk_weight)
+    if topk_weight.shape[0] == 0:
+        return out
+    check(lib.hdmoe_renorm_top2_bf16(ptr(topk_weight), topk_weight.shape[0], ptr(out), _stream(topk_weight)))
+    return out
+
+
 def dispatch(topk_idx, E):
     """Stable permutation of the flat slots by expert.
     -> counts [E], offsets [E+1], perm [2T], inv_perm [2T] (int32, device)."""
@@ -132,6 +144,16 @@ def silu_mul(a, b):
         raise ValueError("silu_mul: shape mismatch")
     out = torch.empty_like(a)
     check(lib.hdmoe_silu_mul_bf16(ptr(a), ptr(b), a.numel(), ptr(out), _stream(a)))
+    return out
+
+
+def gelu(x):
+    """F.gelu (erf form) of a contiguous bf16 tensor."""
+    _need_hip(x, "gelu x", BF16)
+    if not x.is_contiguous():
+        raise ValueError("gelu: expected a contiguous tensor")
+    out = torch.empty_like(x)
+    check(lib.hdmoe_gelu_bf16(ptr(x), x.numel(), ptr(out), _stream(x)))
     return out
 
 

@@ -154,8 +154,8 @@ class MoEGate(nn.Module):
     def _check(self):
         if self.scoring_func != 'softmax':
             raise NotImplementedError(f'insupportable scoring function for MoE gating: {self.scoring_func}')
-        if self.top_k != 2 or self.norm_topk_prob:
-            raise NotImplementedError("the HIP gate kernel selects the top 2 experts without renormalisation")
+        if self.top_k != 2:
+            raise NotImplementedError("the HIP gate kernel selects the top 2 experts")
 
     def device_weight(self, hidden_states):
         """The gate weight in the activations' dtype on their device (model.py:268 routes it through
@@ -167,6 +167,8 @@ class MoEGate(nn.Module):
         bsz, seq_len, h = hidden_states.shape
         x2 = hidden_states.reshape(-1, h).contiguous()
         idx, w = HF.gate_top2(x2, self.device_weight(x2))
+        if self.norm_topk_prob:   # model.py:277-280; HiDream leaves it off
+            w = HF.renorm_top2(w)
         return idx.to(torch.int64), w, None
 
 
@@ -219,7 +221,8 @@ class MOEFeedForwardSwiGLU(nn.Module):
         orig_shape = x.shape
         x2 = x.reshape(-1, orig_shape[-1]).contiguous()
         gate_w = self.gate.device_weight(x2)
-        got = self._collect(x2)
+        # renormalised gate weights are not part of the one-call path: the stages are composed
+        got = None if self.gate.norm_topk_prob else self._collect(x2)
         if got is not None:
             wdt, experts, shared, keep = got
             H = self.experts[0].w1.weight.shape[0]
@@ -243,7 +246,7 @@ class MOEFeedForwardSwiGLU(nn.Module):
         x2 = x.reshape(-1, D).contiguous()
         mods = tuple(m.reshape(B, D).contiguous() for m in (shift, scale, gate))
         gate_w = self.gate.device_weight(x2)
-        got = self._collect(x2)
+        got = None if self.gate.norm_topk_prob else self._collect(x2)
         if got is not None:
             wdt, experts, shared, keep = got
             H = self.experts[0].w1.weight.shape[0]
@@ -263,6 +266,8 @@ class MOEFeedForwardSwiGLU(nn.Module):
         offloaded or mixed-dtype weights, dequantising scaled-fp8 Linears)."""
         E = len(self.experts)
         idx, w = HF.gate_top2(x2, gate_w)
+        if self.gate.norm_topk_prob:
+            w = HF.renorm_top2(w)
         counts, offsets, perm, inv_perm = HF.dispatch(idx, E)
         xs = HF.permute_bf16(x2, perm)
         y = torch.empty_like(xs)

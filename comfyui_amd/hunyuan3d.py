@@ -10,7 +10,14 @@ and erf-GELU epilogue for the experts.
 
 Inference only (the reference's training branch and auxiliary loss are not part of this path). A token meets at
 most two experts, so the index_add_ accumulation bf16(bf16(w_a y_a) + bf16(w_b y_b)) is the same two-term sum the
-HiDream combine forms. Inputs must be bf16 HIP tensors and the Linears bf16: there is no CPU path.
+HiDream combine forms. Inputs must be bf16 HIP tensors: there is no CPU path.
+
+Two ways through the experts:
+  * every Linear a plain bf16 one resident on the device (no weight function, no scale_weight): two grouped launches
+    for all experts and the shared expert;
+  * anything else the `operations` argument brings (scaled-fp8 Linears with or without the fp8 matrix multiply,
+    manual-cast or offloaded weights, weight functions): one expert at a time through the Linear modules' own
+    forward, the GELU as an elementwise kernel, with the same gate, dispatch and combine kernels around them.
 """
 import torch
 import torch.nn as nn
@@ -44,15 +51,29 @@ class GELU(nn.Module):
 
     def forward(self, hidden_states):
         x2 = hidden_states.reshape(-1, hidden_states.shape[-1]).contiguous()
-        _need(x2, self.proj)
+        _need(x2)
+        if not _plain_bf16(self.proj, x2):
+            return HF.gelu(self.proj(x2).contiguous()).view(*hidden_states.shape[:-1], self.proj.weight.shape[0])
         _, y = HF.grouped_linear(x2[:0], None, [], a_static=x2, shared=(self.proj.weight, self.proj.bias), act="gelu")
         return y.view(*hidden_states.shape[:-1], self.proj.weight.shape[0])
 
 
-def _need(x, lin):
-    if not (x.is_cuda and x.dtype == BF16 and lin.weight.dtype == BF16 and lin.weight.is_cuda):
-        raise RuntimeError(f"comfyui_amd.hunyuan3d: expected bfloat16 HIP activations and weights, got {x.dtype} on "
-                           f"{x.device} and {lin.weight.dtype} on {lin.weight.device}; there is no CPU path")
+def _need(x):
+    if not (x.is_cuda and x.dtype == BF16):
+        raise RuntimeError(f"comfyui_amd.hunyuan3d: expected bfloat16 HIP activations, got {x.dtype} on {x.device}; "
+                           "there is no CPU path")
+
+
+def _plain_bf16(lin, x):
+    """True when `lin` can join a grouped launch as it stands: bf16 weight (and bias) on x's device, nothing to
+    apply to them first."""
+    if getattr(lin, "weight_function", None) or getattr(lin, "bias_function", None):
+        return False
+    if getattr(lin, "scale_weight", None) is not None:
+        return False
+    if lin.weight.dtype != BF16 or lin.weight.device != x.device:
+        return False
+    return lin.bias is None or (lin.bias.dtype == BF16 and lin.bias.device == x.device)
 
 
 class FeedForward(nn.Module):
@@ -72,9 +93,15 @@ class FeedForward(nn.Module):
         """((proj weight, bias), (out weight, bias))"""
         return (self.net[0].proj.weight, self.net[0].proj.bias), (self.net[2].weight, self.net[2].bias)
 
+    def fusable(self, x):
+        return _plain_bf16(self.net[0].proj, x) and _plain_bf16(self.net[2], x)
+
     def forward(self, hidden_states: torch.Tensor) -> torch.Tensor:
         x2 = hidden_states.reshape(-1, hidden_states.shape[-1]).contiguous()
-        _need(x2, self.net[0].proj)
+        _need(x2)
+        if not self.fusable(x2):
+            y = self.net[2](self.net[0](x2))     # net[1] is Dropout, the identity at inference
+            return y.view(*hidden_states.shape[:-1], y.shape[-1])
         w_in, w_out = self.stage_weights()
         _, h = HF.grouped_linear(x2[:0], None, [], a_static=x2, shared=w_in, act="gelu")
         _, y = HF.grouped_linear(h[:0], None, [], a_static=h, shared=w_out, act="none")
@@ -120,11 +147,19 @@ class MoEBlock(nn.Module):
             raise NotImplementedError("the HIP gate kernel selects the top 2 experts")
         orig_shape = hidden_states.shape
         x2 = hidden_states.reshape(-1, orig_shape[-1]).contiguous()
-        _need(x2, self.experts[0].net[0].proj)
+        _need(x2)
         gate_w = amd_ops.cast_to(self.gate.weight, dtype=x2.dtype, device=x2.device).contiguous()
         idx, w = HF.gate_top2(x2, gate_w)
         _, offsets, perm, inv_perm = HF.dispatch(idx, self.num_experts)
         xs = HF.permute_bf16(x2, perm)
+        if not (all(e.fusable(x2) for e in self.experts) and self.shared_experts.fusable(x2)):
+            y = torch.empty_like(xs)
+            bounds = offsets.tolist()  # host sync: segment sizes steer the per-expert calls
+            for i, expert in enumerate(self.experts):
+                lo, hi = bounds[i], bounds[i + 1]
+                if hi > lo:
+                    y[lo:hi] = expert(xs[lo:hi])
+            return HF.combine(y, inv_perm, w, self.shared_experts(x2)).view(*orig_shape)
         stage1 = [e.stage_weights()[0] for e in self.experts]
         stage2 = [e.stage_weights()[1] for e in self.experts]
         sh1, sh2 = self.shared_experts.stage_weights()

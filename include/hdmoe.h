@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define HDMOE_VERSION 109
+#define HDMOE_VERSION 110
 
 #define HDMOE_OK 0
 #define HDMOE_E_NULL (-1)      /* required pointer is NULL */
@@ -66,6 +66,11 @@ const char* hdmoe_last_error(void);
  * D % 8 == 0, 2 <= E <= 16. The same gate serves comfy/ldm/hunyuan3dv2_1/hunyuandit.py:73-112 (E = 6 or 8). */
 int hdmoe_gate_top2(const void* x_bf16, const void* gate_w_bf16, int T, int D, int E,
                     int32_t* topk_idx, void* topk_weight_bf16, hdmoe_stream_t stream);
+
+/* Optional renormalisation of the two gate weights, comfy/ldm/hidream/model.py:277-280 (`norm_topk_prob`, off in
+ * HiDream): out[t, s] = bf16( w[t, s] / bf16( bf16(w[t,0] + w[t,1]) + 1e-20 ) ), the rounding points of the three torch
+ * ops on bf16 tensors. topk_weight and out are [T, 2] bf16 (out may be topk_weight). */
+int hdmoe_renorm_top2_bf16(const void* topk_weight_bf16, int T, void* out_bf16, hdmoe_stream_t stream);
 
 /* Token dispatch, comfy/ldm/hidream/model.py:313-318: the boolean-mask gathers
  * `x[flat_topk_idx == i]` for i = 0..E-1 select flat slots p = 2t+s in ascending p,
@@ -167,6 +172,10 @@ int hdmoe_linear_bias(int weight_dtype, const void* a, int rows, int K, int N, c
 /* Elementwise middle of model.py:238 for the unfused path: out = bf16(bf16(silu(a)) * b). */
 int hdmoe_silu_mul_bf16(const void* a_bf16, const void* b_bf16, int64_t n, void* out_bf16,
                         hdmoe_stream_t stream);
+
+/* F.gelu (erf form) of a bf16 tensor for the unfused Hunyuan3D expert, comfy/ldm/hunyuan3dv2_1/hunyuandit.py:14-26
+ * (`gelu(proj(x))` when proj is not the plain bf16 Linear): out = bf16(gelu(fp32(x))). n % 8 == 0. */
+int hdmoe_gelu_bf16(const void* x_bf16, int64_t n, void* out_bf16, hdmoe_stream_t stream);
 
 /* `weight * scale_weight` or `input * scale_weight` of the scaled-fp8 Linear WITHOUT fp8
  * matmul (comfy/ops.py:407-410), after the operand was cast to bf16:

@@ -266,7 +266,11 @@ def linear_bias(x, weight, bias):
 
 
 def gelu_feed_forward(x, ff):
-    """hunyuandit.py:28-50: Linear -> F.gelu (erf form) -> Dropout(0) -> Linear. ff = (w_in, b_in, w_out, b_out)."""
+    """hunyuandit.py:28-50: Linear -> F.gelu (erf form) -> Dropout(0) -> Linear. ff = (w_in, b_in, w_out, b_out), or
+    (LinearParams, LinearParams, mode) for Linears of the operation classes (`linear` above)."""
+    if len(ff) == 3:
+        p_in, p_out, mode = ff
+        return linear(F.gelu(linear(x, p_in, mode)), p_out, mode)
     w_in, b_in, w_out, b_out = ff
     return linear_bias(F.gelu(linear_bias(x, w_in, b_in)), w_out, b_out)
 
@@ -398,6 +402,13 @@ def moe_forward_dense(x, params, mode, topk_idx, topk_weight):
     y = (sel.permute(1, 0, 2) * topk_weight.to(x.dtype).unsqueeze(-1)).sum(dim=1)
     y = y.view(x.shape).to(x.dtype)
     return y + ffn_swiglu(x, params["shared"], mode)
+
+
+def renorm_topk(topk_weight):
+    """The optional renormalisation of MoEGate.forward (/root/reference/comfy/ldm/hidream/model.py:277-280) on the
+    bf16 gate weights, as the three torch ops evaluate it: sum -> bf16, + 1e-20 -> bf16, quotient -> bf16."""
+    denominator = topk_weight.sum(dim=-1, keepdim=True) + 1e-20
+    return topk_weight / denominator
 
 
 def error_metrics(got, ref):

@@ -98,6 +98,83 @@ def test_moe_block(dev, E, dim, inner, tokens):
     assert d["rel_rms"] <= 4e-3, d
 
 
+def test_gelu_kernel(dev):
+    from comfyui_amd import functional as HF
+    # every finite bf16 value (65280 patterns, a multiple of 8). For |x| <= 4: equal to torch's F.gelu on the CPU or
+    # one step of bf16 beside it where the two erff implementations differ in the last place. Below that 1 + erf(.)
+    # cancels in fp32 and the results (of size 1e-5 and less) agree in absolute terms only; so do results in the
+    # subnormal range, which torch's CPU kernel flushes to zero and the device keeps.
+    bits = torch.arange(0, 65536, dtype=torch.int32)
+    bits = bits[(bits & 0x7F80) != 0x7F80].to(torch.int16)
+    x = bits.view(BF16)
+    got = HF.gelu(x.to(dev)).cpu()
+    want = torch.nn.functional.gelu(x)
+    core = (x.float().abs() <= 4) & ((x.float().abs() >= 2.0 ** -120) | (x.float() == 0))
+    steps = bf16_steps(got[core], want[core])
+    print(f"\ngelu: max steps {int(steps.max())}, exact {(steps == 0).float().mean().item():.5f}")
+    assert int(steps.max()) <= 1 and (steps == 0).float().mean().item() >= 0.98
+    err = (got.float() - want.float()).abs()
+    assert bool((err <= 2e-6 + 2.0 ** -7 * want.float().abs()).all()), float(err.max())
+    with pytest.raises(Exception):
+        HF.gelu(x[:7].to(dev))
+
+
+@pytest.mark.parametrize("kind", ["fp8mm", "fp8mm_noscale", "upcast", "manual_cast"])
+def test_moe_block_through_operation_classes(dev, kind):
+    """MoEBlock built with one of the operation classes (hunyuandit.py:117-129 passes `operations` down to every
+    Linear): the experts run one at a time through the Linear modules' own forward."""
+    from comfyui_amd import hunyuan3d as H, ops, synth
+    FP8 = torch.float8_e4m3fn
+    E, dim, inner, tokens = 6, 256, 1024, 333
+    sd, g = make_block(dim, inner, E, seed=123, bias_scale=0.2)
+    x = torch.randn((1, tokens, dim), generator=g).to(BF16)
+    if kind == "manual_cast":
+        cls = ops.manual_cast
+        m = H.MoEBlock(dim, num_experts=E, moe_top_k=2, ff_inner_dim=inner, operations=cls, dtype=BF16, device="cpu").eval()
+        m.load_state_dict(sd, strict=True)
+        m.gate.to(dev)                                     # Linear weights stay on the host: cast per call
+        params = O.hunyuan_params(sd, E)
+    else:
+        mm = kind.startswith("fp8mm")
+        with_in = kind == "fp8mm"
+        cls = ops.scaled_fp8_ops(fp8_matrix_mult=mm, scale_input=with_in, override_dtype=FP8)
+        m = H.MoEBlock(dim, num_experts=E, moe_top_k=2, ff_inner_dim=inner, operations=cls, dtype=BF16, device=dev).eval()
+        mode = "fp8mm" if mm else "upcast"
+
+        def quantised(prefix, s_in):
+            w8, sw = synth.quantize_per_tensor(sd[prefix + "weight"].float())
+            bias = sd[prefix + "bias"].to(FP8).to(BF16)    # the class keeps every parameter in the override dtype
+            return O.LinearParams(w8, sw, torch.tensor(s_in) if with_in else None, bias)
+
+        def load(ffm, prefix, s_in):
+            out = []
+            for lin, key in ((ffm.net[0].proj, "net.0.proj."), (ffm.net[2], "net.2.")):
+                p = quantised(prefix + key, s_in)
+                lin.weight = torch.nn.Parameter(p.weight.to(dev), requires_grad=False)
+                with torch.no_grad():
+                    lin.bias.copy_(p.bias)
+                    lin.scale_weight.copy_(p.scale_weight)
+                    if with_in:
+                        lin.scale_input.fill_(s_in)
+                out.append(p)
+            return (out[0], out[1], mode)
+
+        params = dict(gate=sd["gate.weight"], experts=[load(m.experts[i], f"experts.{i}.", 1.0 + 0.25 * i) for i in range(E)],
+                      shared=load(m.shared_experts, "shared_experts.", 0.75))
+        with torch.no_grad():
+            m.gate.weight.copy_(sd["gate.weight"])
+    assert not m.shared_experts.fusable(x.to(dev).reshape(-1, dim))
+    y = m(x.to(dev)).cpu()
+    idx_ref, w_ref, _, _ = O.gate_fixed_order(x.reshape(-1, dim), sd["gate.weight"])
+    ref = O.hunyuan_moe_block(x, params, gate_result=(idx_ref, w_ref))
+    d = O.error_metrics(y, ref)
+    print(f"\n{kind}: {d}")
+    assert d["rel_rms"] <= 1e-2 and d["max_over_max"] <= 2e-2, d
+    ff = m.experts[1](x.to(dev)).cpu()
+    d = O.error_metrics(ff, O.gelu_feed_forward(x, params["experts"][1]))
+    assert d["rel_rms"] <= 1e-2, d
+
+
 def test_training_mode_and_cpu_are_refused(dev):
     from comfyui_amd import hunyuan3d as H
     m = H.MoEBlock(256, num_experts=8, ff_inner_dim=1024, dtype=BF16, device=dev)

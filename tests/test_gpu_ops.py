@@ -223,6 +223,42 @@ def test_gate_module_signature(dev):
     assert torch.equal(idx.cpu(), ridx.long())
 
 
+def test_gate_with_renormalised_weights(dev):
+    """norm_topk_prob (model.py:277-280): the kernel's quotients are the oracle's bit for bit, edge values included,
+    and a layer whose gate has the flag set follows the oracle with the renormalised weights."""
+    from comfyui_amd import functional as HF, hidream
+    g = torch.Generator().manual_seed(77)
+    w = torch.rand((5001, 2), generator=g).to(BF16)
+    w[::9, 1] = w[::9, 0]
+    w[3] = 0
+    w[4] = torch.tensor([1.0, 0.0])
+    w[5] = torch.tensor([2.0 ** -126, 2.0 ** -126])
+    got = HF.renorm_top2(w.to(dev)).cpu()
+    assert torch.equal(got.view(torch.int16), O.renorm_topk(w).view(torch.int16))
+    assert HF.renorm_top2(w[:0].to(dev)).shape == (0, 2)
+
+    gate = hidream.MoEGate(512, 4, 2, dtype=BF16, device=dev)
+    gate.norm_topk_prob = True
+    with torch.no_grad():
+        gate.weight.normal_(0, 512 ** -0.5)
+    x = torch.randn((3, 11, 512), device=dev).to(BF16)
+    idx, wn, _ = gate(x)
+    ridx, rw, _, _ = O.gate_fixed_order(x.cpu().reshape(-1, 512), gate.weight.detach().cpu())
+    assert torch.equal(idx.cpu(), ridx.long())
+    assert torch.equal(wn.cpu().view(torch.int16), O.renorm_topk(rw).view(torch.int16))
+
+    dim = 256
+    sd, x = small_layer(seed=61, dim=dim, tokens=210, weights="fp8")
+    m = synth.build_module({k: v.to(dev) for k, v in sd.items()}, "fp8", dev, dim=dim)
+    plain = m(x.to(dev)).cpu()
+    m.gate.norm_topk_prob = True
+    y = m(x.to(dev)).cpu()
+    idx, w2, _, _ = O.gate_fixed_order(x.reshape(-1, dim), sd["gate.weight"])
+    ref = O.moe_forward(x, oracle_params(sd, 4), "fp8mm", gate_result=(idx, O.renorm_topk(w2)))
+    close(y, ref, 1e-2)
+    assert not torch.equal(y, plain)
+
+
 def test_stacked_layers_at_32768_tokens(dev):
     """Stacked sweep (benchmark configuration 4) at its full depth: 48 independent fp8 layers at 2 x 16384 tokens,
     x <- x + FFN(LayerNorm(x)) with the block's affine-free LayerNorm (model.py:393,430) so the residual stream

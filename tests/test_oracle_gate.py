@@ -113,3 +113,26 @@ def test_generic_D_and_E():
         assert float((logits.double() - ref).abs().max()) <= float(ref.abs().max()) * 2 ** -7
         srt = torch.sort(scores.float(), dim=-1, descending=True, stable=True).indices[:, :2]
         assert torch.equal(idx.long(), srt)
+
+
+def test_renorm_topk_rounding_points_and_closed_forms():
+    """model.py:277-280 on bf16 tensors: equal weights give exactly one half each; the result is the fp64 quotient
+    within the rounding of the bf16 sum and of the bf16 quotient; all-zero weights stay zero (the 1e-20 guard)."""
+    g = torch.Generator().manual_seed(3)
+    w = torch.rand((4096, 2), generator=g).to(torch.bfloat16)
+    w[::7, 1] = w[::7, 0]
+    w[5] = 0
+    r = O.renorm_topk(w)
+    assert r.dtype == torch.bfloat16
+    eq = w[:, 0] == w[:, 1]
+    nz = w[:, 0] != 0
+    assert bool((r[eq & nz].float() == 0.5).all())
+    assert bool((r[5].float() == 0).all())
+    # explicit rounding points
+    s = (w[:, 0].float() + w[:, 1].float()).to(torch.bfloat16)
+    d = (s.float() + 1e-20).to(torch.bfloat16)
+    want = (w.float() / d.float().unsqueeze(-1)).to(torch.bfloat16)
+    assert torch.equal(r.view(torch.int16), want.view(torch.int16))
+    exact = w.double() / (w.double().sum(-1, keepdim=True) + 1e-20)
+    ok = nz
+    assert float(((r.double() - exact).abs()[ok] / exact[ok].clamp_min(1e-3)).max()) < 3 * 2.0 ** -8
