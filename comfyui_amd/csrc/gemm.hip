@@ -31,6 +31,7 @@
 // from its index and exits if its index is past the real tile count. Block ids are
 // remapped so that each XCD (ids congruent mod 8) walks a contiguous range of tiles,
 // 4 m-tiles deep, and its L2 sees each operand tile reused by neighbouring blocks.
+#include <cstdlib>
 #include <type_traits>
 
 #include "common.h"
@@ -903,6 +904,25 @@ int launch_grouped(const GemmArgs& args, int tile_bound, hipStream_t s, const ch
   return hdmoe_check_launch(what);
 }
 
+#include "swiglu4w.h"
+
+int launch_swiglu4w(const GemmArgs& args, int tile_bound, hipStream_t s, const char* what) {
+  static bool attr_set[64] = {};
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) device = -1;
+  if (device < 0 || !attr_set[device]) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&swiglu4w_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, W4_SMEM);
+    if (e != hipSuccess) return hdmoe_fail(HDMOE_E_LAUNCH, "%s: hipFuncSetAttribute: %s", what, hipGetErrorString(e));
+    if (device >= 0) attr_set[device] = true;
+  }
+  if (tile_bound <= 0) return HDMOE_OK;
+  int grid = (tile_bound + HDMOE_NUM_XCD - 1) / HDMOE_NUM_XCD * HDMOE_NUM_XCD;
+  if (grid > HDMOE_NUM_CU) grid = HDMOE_NUM_CU;
+  hipLaunchKernelGGL(swiglu4w_kernel, dim3(grid), dim3(W4_THREADS), W4_SMEM, s, args);
+  return hdmoe_check_launch(what);
+}
+
 inline int elem_bytes(int weight_dtype) { return weight_dtype == HDMOE_W_E4M3FN ? 1 : 2; }
 
 int check_dtype(int weight_dtype, const char* what) {
@@ -1032,6 +1052,16 @@ int hdmoe_launch_ffn_gemm(bool swiglu, int weight_dtype, const uint8_t* a_dyn, c
     if (blocks < 1) blocks = 1;
     hipLaunchKernelGGL(splitk_reduce_kernel, dim3(blocks), dim3(256), 0, s, ra);
     return hdmoe_check_launch(what);
+  }
+  if (fp8 && swiglu && getenv("HDMOE_SWIGLU4W") != nullptr) {
+    long long op_bytes = (long long)(gather_dyn != nullptr ? gather_rows : rows_dyn) * K_dyn;
+    if ((long long)rows_static * K_static > op_bytes) op_bytes = (long long)rows_static * K_static;
+    if (swiglu4w_fits(args, op_bytes)) {
+      int tb = 0;
+      if (n_dyn > 0) tb += (rows_dyn / W4_BM + n_dyn) * (N_dyn / W4_FEAT);
+      if (shared != nullptr && rows_static > 0) tb += ((rows_static + W4_BM - 1) / W4_BM) * (N_static / W4_FEAT);
+      return launch_swiglu4w(args, tb, s, what);
+    }
   }
   if (fp8 && tall) return swiglu ? launch_grouped<FP8_SWIGLU, 5>(args, tile_bound, s, what)
                                  : launch_grouped<FP8_PLAIN, 5>(args, tile_bound, s, what);

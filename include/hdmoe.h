@@ -18,6 +18,10 @@
  *   - the only state the library keeps between calls: the thread-local error message, and per device one flag per
  *     GEMM kernel variant recording that hipFuncSetAttribute (the opt-in for more than 64 KiB of dynamic LDS) has
  *     been called for it on that device, plus the device address of the built-in buffer of hdmoe_dispatch_static;
+ *   - one environment variable is read, at every call that runs the fp8 gate/up contraction: HDMOE_SWIGLU4W set
+ *     (to anything) selects the 4-wave form of that kernel (same results bit for bit; one wave per SIMD, a tile's
+ *     SiLU*mul epilogue issued between the MFMAs of the next tile) where the shapes allow it: K a multiple of 256
+ *     and at least 2048, scale_in2 given. It is not the default because it is not faster on this part;
  *   - return value 0 = enqueued; negative = HDMOE_E_* and nothing was enqueued;
  *     hdmoe_last_error() gives a thread-local message for the last failure;
  *   - scale pointers (float*, device) address the fp32 scalar Parameters
@@ -36,7 +40,7 @@
 extern "C" {
 #endif
 
-#define HDMOE_VERSION 110
+#define HDMOE_VERSION 111
 
 #define HDMOE_OK 0
 #define HDMOE_E_NULL (-1)      /* required pointer is NULL */

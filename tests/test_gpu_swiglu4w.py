@@ -1,0 +1,92 @@
+"""The 4-wave form of the fp8 gate/up kernel (csrc/swiglu4w.h, selected with HDMOE_SWIGLU4W=1 in the environment):
+same contraction and rounding points as the default kernel, so its outputs are the default kernel's bit for bit."""
+import os
+
+import pytest
+import torch
+
+from comfyui_amd import synth
+from oracle import hidream_moe_oracle as O
+from tests.helpers import oracle_params, small_layer
+
+pytestmark = pytest.mark.gpu
+BF16 = torch.bfloat16
+
+
+@pytest.fixture
+def four_wave():
+    old = os.environ.get("HDMOE_SWIGLU4W")
+    yield
+    if old is None:
+        os.environ.pop("HDMOE_SWIGLU4W", None)
+    else:
+        os.environ["HDMOE_SWIGLU4W"] = old
+
+
+def grouped_swiglu(T, D, H, E, seed, dev, s_next):
+    """h of hdmoe_grouped_swiglu on random routed rows, once per kernel form."""
+    from comfyui_amd import _lib, functional as HF
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn((T, D), generator=g).to(BF16)
+    ws = []
+    for _ in range(E):
+        w1, s1 = synth.quantize_per_tensor(torch.randn((H, D), generator=g) * 0.03)
+        w3, s3 = synth.quantize_per_tensor(torch.randn((H, D), generator=g) * 0.03)
+        ws.append((w1.to(dev), s1.to(dev).float().reshape(()), w3.to(dev), s3.to(dev).float().reshape(())))
+    if E >= 2:
+        idx = torch.stack([torch.randperm(E, generator=g)[:2] for _ in range(T)]).to(torch.int32)
+    else:
+        idx = torch.zeros((T, 2), dtype=torch.int32)
+    _, offsets, perm, _ = HF.dispatch(idx.to(dev), E)
+    s_in = torch.tensor(1.0, device=dev)
+    s_nx = torch.tensor(s_next, device=dev)
+    xs = HF.quant_fp8(x.to(dev), s_in)[(perm // 2).long()].contiguous()
+
+    def weights(w):
+        f = _lib.FfnWeights()
+        f.w1, f.w3, f.scale_w1, f.scale_w3 = w[0].data_ptr(), w[2].data_ptr(), w[1].data_ptr(), w[3].data_ptr()
+        f.scale_in1 = f.scale_in3 = s_in.data_ptr()
+        f.scale_in2 = s_nx.data_ptr()
+        return f
+    arr = (_lib.FfnWeights * E)(*[weights(w) for w in ws])
+    out = []
+    for form in ("0", "1"):
+        if form == "1":
+            os.environ["HDMOE_SWIGLU4W"] = "1"
+        else:
+            os.environ.pop("HDMOE_SWIGLU4W", None)
+        h = torch.full((2 * T, H), 0x55, dtype=torch.uint8, device=dev)
+        _lib.check(_lib.lib.hdmoe_grouped_swiglu(_lib.W_E4M3FN, xs.data_ptr(), offsets.data_ptr(), 2 * T, E, D, H, arr,
+                                                 h.data_ptr(), None))
+        torch.cuda.synchronize()
+        out.append(h.cpu())
+    return out
+
+
+@pytest.mark.parametrize("T,D,H,E,s_next", [
+    (64, 2048, 128, 1, 1.0),        # one tile, the fewest K steps the kernel takes (16)
+    (300, 2048, 256, 2, 0.5),       # partial tiles, a scale for the consuming Linear that is not 1
+    (1500, 2560, 1024, 4, 0.37),    # one tile per block
+    (5000, 2048, 3584, 3, 1.0),     # several tiles per block: the epilogue of one rides in the K loop of the next
+])
+def test_same_bytes_as_the_default_kernel(dev, four_wave, T, D, H, E, s_next):
+    base, four = grouped_swiglu(T, D, H, E, seed=T + H, dev=dev, s_next=s_next)
+    assert not bool((base == 0x55).all())
+    assert torch.equal(base, four)
+
+
+def test_layer_through_the_four_wave_kernel(dev, four_wave):
+    """The whole layer (rows gathered through the dispatch permutation, shared expert in the same launch) against
+    the oracle and against the default kernel."""
+    dim = 2048
+    sd, x = small_layer(seed=91, dim=dim, tokens=700, weights="fp8", scale_in=0.5)
+    m = synth.build_module({k: v.to(dev) for k, v in sd.items()}, "fp8", dev, dim=dim)
+    os.environ.pop("HDMOE_SWIGLU4W", None)
+    base = m(x.to(dev)).cpu()
+    os.environ["HDMOE_SWIGLU4W"] = "1"
+    four = m(x.to(dev)).cpu()
+    assert torch.equal(base.view(torch.int16), four.view(torch.int16))
+    idx, w, _, _ = O.gate_fixed_order(x.reshape(-1, dim), sd["gate.weight"])
+    ref = O.moe_forward(x, oracle_params(sd, 4), "fp8mm", gate_result=(idx, w))
+    d = O.error_metrics(four, ref)
+    assert d["rel_rms"] <= 1e-2, d
