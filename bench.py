@@ -335,7 +335,10 @@ def main():
         "stage_ms": stage_ms,
         "gemm_down_tflops": gemm2_tflops,
         "roofline": {
-            "kernel": "grouped_gemm_kernel<FP8_SWIGLU, TT> (TT = 5 at 8192 tokens)" if fp8 else "grouped_gemm_kernel<BF16_SWIGLU>",
+            # fp8: the launcher takes the 8-wave kernel with 320-token tiles where those do not add a round of tiles
+            # (8192 tokens and up for these sizes) and the 4-wave kernel with 256-token tiles below
+            "kernel": ("grouped_gemm_kernel<FP8_SWIGLU, 5> from about 6000 tokens, swiglu4w_kernel below"
+                       if fp8 else "grouped_gemm_kernel<BF16_SWIGLU>"),
             "bound": "mfma",
             "achieved": gemm1_tflops,
             "peak": peak,

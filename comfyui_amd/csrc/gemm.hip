@@ -1053,7 +1053,12 @@ int hdmoe_launch_ffn_gemm(bool swiglu, int weight_dtype, const uint8_t* a_dyn, c
     hipLaunchKernelGGL(splitk_reduce_kernel, dim3(blocks), dim3(256), 0, s, ra);
     return hdmoe_check_launch(what);
   }
-  if (fp8 && swiglu && getenv("HDMOE_SWIGLU4W") != nullptr) {
+  // The 4-wave form of the gate/up kernel (swiglu4w.h) has the 256-token tile; it takes the launch whenever the
+  // 8-wave kernel would not use its 320-token tile (2-3 % faster there: part of its epilogue hides in the K loop).
+  // HDMOE_SWIGLU4W in the environment overrides: "0" = never, anything else = whenever the shapes allow.
+  const char* const env4w = getenv("HDMOE_SWIGLU4W");
+  const bool want4w = env4w != nullptr ? env4w[0] != '0' : !tall;
+  if (fp8 && swiglu && want4w) {
     long long op_bytes = (long long)(gather_dyn != nullptr ? gather_rows : rows_dyn) * K_dyn;
     if ((long long)rows_static * K_static > op_bytes) op_bytes = (long long)rows_static * K_static;
     if (swiglu4w_fits(args, op_bytes)) {

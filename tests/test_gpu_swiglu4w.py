@@ -1,5 +1,5 @@
-"""The 4-wave form of the fp8 gate/up kernel (csrc/swiglu4w.h, selected with HDMOE_SWIGLU4W=1 in the environment):
-same contraction and rounding points as the default kernel, so its outputs are the default kernel's bit for bit."""
+"""The two kernels of the fp8 gate/up contraction (8 waves: csrc/gemm.hip; 4 waves: csrc/swiglu4w.h; HDMOE_SWIGLU4W in
+the environment forces one or the other): same contraction and rounding points, so the same bytes out."""
 import os
 
 import pytest
@@ -51,10 +51,7 @@ def grouped_swiglu(T, D, H, E, seed, dev, s_next):
     arr = (_lib.FfnWeights * E)(*[weights(w) for w in ws])
     out = []
     for form in ("0", "1"):
-        if form == "1":
-            os.environ["HDMOE_SWIGLU4W"] = "1"
-        else:
-            os.environ.pop("HDMOE_SWIGLU4W", None)
+        os.environ["HDMOE_SWIGLU4W"] = form
         h = torch.full((2 * T, H), 0x55, dtype=torch.uint8, device=dev)
         _lib.check(_lib.lib.hdmoe_grouped_swiglu(_lib.W_E4M3FN, xs.data_ptr(), offsets.data_ptr(), 2 * T, E, D, H, arr,
                                                  h.data_ptr(), None))
@@ -69,7 +66,7 @@ def grouped_swiglu(T, D, H, E, seed, dev, s_next):
     (1500, 2560, 1024, 4, 0.37),    # one tile per block
     (5000, 2048, 3584, 3, 1.0),     # several tiles per block: the epilogue of one rides in the K loop of the next
 ])
-def test_same_bytes_as_the_default_kernel(dev, four_wave, T, D, H, E, s_next):
+def test_same_bytes_from_both_kernels(dev, four_wave, T, D, H, E, s_next):
     base, four = grouped_swiglu(T, D, H, E, seed=T + H, dev=dev, s_next=s_next)
     assert not bool((base == 0x55).all())
     assert torch.equal(base, four)
@@ -77,11 +74,11 @@ def test_same_bytes_as_the_default_kernel(dev, four_wave, T, D, H, E, s_next):
 
 def test_layer_through_the_four_wave_kernel(dev, four_wave):
     """The whole layer (rows gathered through the dispatch permutation, shared expert in the same launch) against
-    the oracle and against the default kernel."""
+    the oracle and against the 8-wave kernel."""
     dim = 2048
     sd, x = small_layer(seed=91, dim=dim, tokens=700, weights="fp8", scale_in=0.5)
     m = synth.build_module({k: v.to(dev) for k, v in sd.items()}, "fp8", dev, dim=dim)
-    os.environ.pop("HDMOE_SWIGLU4W", None)
+    os.environ["HDMOE_SWIGLU4W"] = "0"
     base = m(x.to(dev)).cpu()
     os.environ["HDMOE_SWIGLU4W"] = "1"
     four = m(x.to(dev)).cpu()
