@@ -65,6 +65,9 @@ def grouped_swiglu(T, D, H, E, seed, dev, s_next):
     (300, 2048, 256, 2, 0.5),       # partial tiles, a scale for the consuming Linear that is not 1
     (1500, 2560, 1024, 4, 0.37),    # one tile per block
     (5000, 2048, 3584, 3, 1.0),     # several tiles per block: the epilogue of one rides in the K loop of the next
+    (777, 4096, 384, 5, 2.0),       # 16 pairs of K steps, an odd number of feature tiles
+    (40, 2304, 256, 16, 1.0),       # 16 experts, most of them empty or a few rows; 9 pairs of K steps
+    (3000, 6912, 256, 2, 0.25),     # the down projection's K as the contraction length (27 pairs)
 ])
 def test_same_bytes_from_both_kernels(dev, four_wave, T, D, H, E, s_next):
     base, four = grouped_swiglu(T, D, H, E, seed=T + H, dev=dev, s_next=s_next)
@@ -87,3 +90,26 @@ def test_layer_through_the_four_wave_kernel(dev, four_wave):
     ref = O.moe_forward(x, oracle_params(sd, 4), "fp8mm", gate_result=(idx, w))
     d = O.error_metrics(four, ref)
     assert d["rel_rms"] <= 1e-2, d
+
+
+def test_dense_feed_forward_through_both_kernels(dev, four_wave):
+    """hdmoe_ffn_swiglu (the shared expert / text feed-forward on its own: one static group, no gather)."""
+    from comfyui_amd import hidream, ops
+    FP8 = torch.float8_e4m3fn
+    dim, hidden = 2048, 1536
+    g = torch.Generator().manual_seed(5)
+    cls = ops.scaled_fp8_ops(fp8_matrix_mult=True, scale_input=True, override_dtype=FP8)
+    ff = hidream.FeedForwardSwiGLU(dim, hidden, dtype=BF16, device=dev, operations=cls).eval()
+    for lin in (ff.w1, ff.w2, ff.w3):
+        w8, sw = synth.quantize_per_tensor(torch.randn(tuple(lin.weight.shape), generator=g) * 0.03)
+        lin.weight = torch.nn.Parameter(w8.to(dev), requires_grad=False)
+        with torch.no_grad():
+            lin.scale_weight.copy_(sw)
+            lin.scale_input.fill_(0.5)
+    x = torch.randn((2, 450, dim), generator=g).to(BF16).to(dev)
+    os.environ["HDMOE_SWIGLU4W"] = "0"
+    base = ff(x).cpu()
+    os.environ["HDMOE_SWIGLU4W"] = "1"
+    four = ff(x).cpu()
+    assert bool(torch.isfinite(base.float()).all()) and float(base.float().abs().max()) > 0
+    assert torch.equal(base.view(torch.int16), four.view(torch.int16))
