@@ -34,6 +34,17 @@ PEAK_HBM_GBPS = 8000.0      # MI355X HBM3E
 
 
 
+def gate_up_kernel_name(T, H, Hs, E, cus=256):
+    """Which kernel the library's launcher runs for the fp8 gate/up contraction of a layer (the rule of
+    hdmoe_launch_ffn_gemm in comfyui_amd/csrc/gemm.hip, with HDMOE_SWIGLU4W unset): 320-token tiles in the 8-wave
+    kernel when they do not add a round of tiles to the persistent blocks, else 256-token tiles in the 4-wave one."""
+    def cost(tt):
+        bm = 64 * tt
+        tiles = E * (-(-(2 * T // E) // bm)) * (H // 128) + (-(-T // bm)) * (Hs // 128)
+        return -(-tiles // cus) * (tt + 1)
+    return "grouped_gemm_kernel<FP8_SWIGLU, 5>" if cost(5) < cost(4) else "swiglu4w_kernel"
+
+
 def measured_traffic(workload):
     """L2-side traffic of the dominant kernel per launch (bytes fetched + written) as the last rocprofv3 --pmc runs
     measured it: profiles/traffic.json holds, per workload, the calibrated FETCH_SIZE and WRITE_SIZE readings, the
@@ -335,10 +346,7 @@ def main():
         "stage_ms": stage_ms,
         "gemm_down_tflops": gemm2_tflops,
         "roofline": {
-            # fp8: the launcher takes the 8-wave kernel with 320-token tiles where those do not add a round of tiles
-            # (8192 tokens and up for these sizes) and the 4-wave kernel with 256-token tiles below
-            "kernel": ("grouped_gemm_kernel<FP8_SWIGLU, 5> from about 6000 tokens, swiglu4w_kernel below"
-                       if fp8 else "grouped_gemm_kernel<BF16_SWIGLU>"),
+            "kernel": gate_up_kernel_name(T, H, Hs, E) if fp8 else "grouped_gemm_kernel<BF16_SWIGLU, 4>",
             "bound": "mfma",
             "achieved": gemm1_tflops,
             "peak": peak,
