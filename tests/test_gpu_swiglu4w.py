@@ -113,3 +113,31 @@ def test_dense_feed_forward_through_both_kernels(dev, four_wave):
     four = ff(x).cpu()
     assert bool(torch.isfinite(base.float()).all()) and float(base.float().abs().max()) > 0
     assert torch.equal(base.view(torch.int16), four.view(torch.int16))
+
+
+def test_layer_with_the_four_wave_kernel_in_a_graph(dev, four_wave):
+    """Capture and replay of a layer whose gate/up contraction takes the 4-wave kernel (no memset nodes, nothing
+    allocated, the kernel attribute set before the capture)."""
+    os.environ["HDMOE_SWIGLU4W"] = "1"
+    dim = 2048
+    sd, x = small_layer(seed=17, dim=dim, tokens=600, weights="fp8")
+    m = synth.build_module({k: v.to(dev) for k, v in sd.items()}, "fp8", dev, dim=dim)
+    xs = [x.to(dev), (x * 0.5).to(dev), x.flip(1).contiguous().to(dev)]
+    eager = [m(v).clone() for v in xs]
+    torch.cuda.synchronize()
+    static_x = xs[0].clone()
+    side = torch.cuda.Stream()                  # default priority
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        m(static_x)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_y = m(static_x)
+    for rep in range(2):
+        for v, want in zip(xs, eager):
+            static_x.copy_(v)
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(static_y, want)
+            assert torch.equal(m(v), want)      # eager work between replays
