@@ -141,3 +141,17 @@ def test_layer_with_the_four_wave_kernel_in_a_graph(dev, four_wave):
             torch.cuda.synchronize()
             assert torch.equal(static_y, want)
             assert torch.equal(m(v), want)      # eager work between replays
+
+
+def test_random_shapes_same_bytes(dev, four_wave):
+    """A seeded walk over token counts, widths, expert counts and cast scales."""
+    import random
+    rnd = random.Random(7)
+    for it in range(12):
+        E = rnd.choice([1, 2, 3, 4, 6, 8])
+        D = rnd.choice([2048, 2304, 2560, 3072, 4096])
+        H = 128 * rnd.randint(1, 12)
+        T = rnd.choice([1, 7, 33, 100, 257, 511, 1000, 2049])
+        s_next = rnd.choice([1.0, 0.5, 0.37, 2.0])
+        base, four = grouped_swiglu(T, D, H, E, seed=500 + it, dev=dev, s_next=s_next)
+        assert torch.equal(base, four), (T, D, H, E, s_next)
