@@ -44,5 +44,9 @@ static inline int hdmoe_check_scale_in13(const char* what, const hdmoe_ffn_weigh
 
 static inline size_t hdmoe_align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
+// gate kernels: tokens per block (a pure function of T) and the bytes of the per-block expert histograms
+int hdmoe_gate_tokens_per_block(int T);
+size_t hdmoe_gate_hist_bytes(int T, int E);
+
 constexpr int HDMOE_NUM_CU = 256;   // MI355X
 constexpr int HDMOE_NUM_XCD = 8;

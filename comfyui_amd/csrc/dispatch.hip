@@ -11,6 +11,8 @@
 //            writes perm / inv_perm.
 // No atomics, so the result does not depend on scheduling.
 // Traffic: 2T*4 bytes read twice, 2*2T*4 bytes written.
+// Inside the one-call layer the gate kernel does the counting (its blocks own contiguous token ranges and leave
+// one histogram each) and only the scatter launch remains.
 #include <mutex>
 
 #include "common.h"
@@ -53,22 +55,24 @@ __global__ __launch_bounds__(THREADS) void dispatch_count_kernel(const int32_t* 
 
 template <int ITEMS>
 __global__ __launch_bounds__(THREADS) void dispatch_scatter_kernel(
-    const int32_t* __restrict__ flat, int n, int E, int nchunks, const int32_t* __restrict__ chunk_counts,
-    int32_t* __restrict__ counts, int32_t* __restrict__ offsets, int32_t* __restrict__ perm,
-    int32_t* __restrict__ inv_perm) {
+    const int32_t* __restrict__ flat, int n, int E, int nhist, int hist_per_chunk,
+    const int32_t* __restrict__ chunk_counts, int32_t* __restrict__ counts, int32_t* __restrict__ offsets,
+    int32_t* __restrict__ perm, int32_t* __restrict__ inv_perm) {
   __shared__ int32_t total[HDMOE_MAX_EXPERTS];
   __shared__ int32_t before[HDMOE_MAX_EXPERTS];
   __shared__ int32_t cursor[HDMOE_MAX_EXPERTS];  // next sorted row per expert for this block
   __shared__ int32_t wave_cnt[WAVES][HDMOE_MAX_EXPERTS];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 
-  // per expert: rows in earlier chunks, rows overall. Wave w handles experts w, w+WAVES, ...
+  // per expert: rows in earlier chunks, rows overall. Wave w handles experts w, w+WAVES, ... The histograms may be
+  // finer than the chunks (hist_per_chunk consecutive ones make up a chunk: those of the gate kernel's blocks).
+  const int first_mine = (int)blockIdx.x * hist_per_chunk;
   for (int e = wave; e < E; e += WAVES) {
     int32_t tot = 0, bef = 0;
-    for (int c = lane; c < nchunks; c += 64) {
+    for (int c = lane; c < nhist; c += 64) {
       const int32_t v = chunk_counts[(size_t)c * E + e];
       tot += v;
-      if (c < (int)blockIdx.x) bef += v;
+      if (c < first_mine) bef += v;
     }
     for (int off = 32; off >= 1; off >>= 1) {
       tot += __shfl_xor(tot, off, 64);
@@ -143,12 +147,37 @@ int dispatch_enqueue(const char* what, const int32_t* topk_idx, int T, int E, in
   if (items == ITEMS_SMALL) {
     hipLaunchKernelGGL(dispatch_count_kernel<ITEMS_SMALL>, dim3(nchunks), dim3(THREADS), 0, s, topk_idx, n, E, cc);
     hipLaunchKernelGGL(dispatch_scatter_kernel<ITEMS_SMALL>, dim3(nchunks), dim3(THREADS), 0, s, topk_idx, n, E,
-                       nchunks, cc, counts, offsets, perm, inv_perm);
+                       nchunks, 1, cc, counts, offsets, perm, inv_perm);
   } else {
     hipLaunchKernelGGL(dispatch_count_kernel<ITEMS_LARGE>, dim3(nchunks), dim3(THREADS), 0, s, topk_idx, n, E, cc);
     hipLaunchKernelGGL(dispatch_scatter_kernel<ITEMS_LARGE>, dim3(nchunks), dim3(THREADS), 0, s, topk_idx, n, E,
-                       nchunks, cc, counts, offsets, perm, inv_perm);
+                       nchunks, 1, cc, counts, offsets, perm, inv_perm);
   }
+  return hdmoe_check_launch(what);
+}
+
+// Second pass alone: the histograms come from the gate kernel, one per block of tokens_per_hist tokens
+// (hdmoe_gate_tokens_per_block: a power of two that divides a chunk's tokens).
+int dispatch_scatter_enqueue(const char* what, const int32_t* topk_idx, int T, int E, int32_t* counts,
+                             int32_t* offsets, int32_t* perm, int32_t* inv_perm, const int32_t* block_hist,
+                             int tokens_per_hist, hipStream_t s) {
+  const int n = T * HDMOE_TOPK;
+  const int items = items_for((size_t)n);
+  const int chunk = THREADS * items;
+  const int chunk_tokens = chunk / HDMOE_TOPK;
+  if (tokens_per_hist < 1 || chunk_tokens % tokens_per_hist != 0)
+    return hdmoe_fail(HDMOE_E_SHAPE, "%s: histograms of %d tokens do not tile a chunk of %d", what, tokens_per_hist,
+                      chunk_tokens);
+  int nchunks = (n + chunk - 1) / chunk;
+  if (nchunks < 1) nchunks = 1;
+  const int nhist = T > 0 ? (T + tokens_per_hist - 1) / tokens_per_hist : 0;
+  const int per_chunk = chunk_tokens / tokens_per_hist;
+  if (items == ITEMS_SMALL)
+    hipLaunchKernelGGL(dispatch_scatter_kernel<ITEMS_SMALL>, dim3(nchunks), dim3(THREADS), 0, s, topk_idx, n, E, nhist,
+                       per_chunk, block_hist, counts, offsets, perm, inv_perm);
+  else
+    hipLaunchKernelGGL(dispatch_scatter_kernel<ITEMS_LARGE>, dim3(nchunks), dim3(THREADS), 0, s, topk_idx, n, E, nhist,
+                       per_chunk, block_hist, counts, offsets, perm, inv_perm);
   return hdmoe_check_launch(what);
 }
 
@@ -160,6 +189,14 @@ int dispatch_check_sizes(const char* what, int T, int E) {
 }
 
 }  // namespace
+
+// The dispatch of the one-call layer: the gate kernel has already counted.
+int hdmoe_launch_dispatch_scatter(const int32_t* topk_idx, int T, int E, int32_t* counts, int32_t* offsets,
+                                  int32_t* perm, int32_t* inv_perm, const int32_t* block_hist, int tokens_per_hist,
+                                  hipStream_t s, const char* what) {
+  if (int rc = dispatch_check_sizes(what, T, E)) return rc;
+  return dispatch_scatter_enqueue(what, topk_idx, T, E, counts, offsets, perm, inv_perm, block_hist, tokens_per_hist, s);
+}
 
 extern "C" int hdmoe_dispatch(const int32_t* topk_idx, int T, int E, int32_t* counts, int32_t* offsets,
                               int32_t* perm, int32_t* inv_perm, void* workspace, size_t workspace_bytes,

@@ -3,16 +3,16 @@
 //
 // One token per wavefront. Lane l owns the 8-element groups starting at element
 // l*8 + c*512 (c = 0, 1, ...): a 16-byte load per lane and chunk, so a wave reads
-// 1 KiB of the token row per load instruction, fully coalesced. Each lane keeps
-// its slice of Wg in registers (packed bf16) for the whole kernel, because the
-// slice is the same for every token the wave processes. The E dot products are
+// 1 KiB of the token row per load instruction, fully coalesced. A lane needs the
+// same slice of Wg for every token; the block keeps Wg in LDS (packed bf16) and a
+// lane re-reads its slice per token. The E dot products are
 // accumulated in fp32 with fma in ascending element order per lane and reduced
 // across the wave with an xor butterfly (32, 16, 8, 4, 2, 1). That order is fixed
 // on purpose: it is the order the CPU checker restates, which makes logits,
 // scores and therefore the routing reproducible bit for bit.
 //
 // HBM traffic per token: D*2 bytes read, 12 bytes written; the kernel is
-// bandwidth bound (the E x D weight is 20 KiB and stays in registers / L2).
+// bandwidth bound (the E x D weight is 20 KiB and stays in LDS / L2).
 #include "common.h"
 #include "numfmt.h"
 #include "quant.h"
@@ -196,14 +196,42 @@ struct GateQuant {
   float ln_eps;
 };
 
+// Token -> wave mapping of both kernels: block b owns tokens [b * tpb, (b + 1) * tpb), its waves take them in turn
+// (wave w: b * tpb + w, + WAVES_PER_BLOCK, ...). A block therefore knows the expert histogram of a contiguous token
+// range, which is the first pass of the dispatch's counting sort: when block_hist is not NULL, block b writes its E
+// counts to block_hist[b * E ..] and the dispatch needs no counting launch of its own.
+template <int E>
+__device__ __forceinline__ void write_block_hist(const int (&cnt)[E], int32_t* __restrict__ block_hist) {
+  __shared__ int32_t wave_cnt[WAVES_PER_BLOCK][E];
+  if (block_hist == nullptr) return;  // kernel argument: the same for every thread
+  const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  if (lane == 0) {
+#pragma unroll
+    for (int e = 0; e < E; ++e) wave_cnt[wv][e] = cnt[e];
+  }
+  __syncthreads();
+  if (threadIdx.x < E) {
+    int32_t sum = 0;
+#pragma unroll
+    for (int w = 0; w < WAVES_PER_BLOCK; ++w) sum += wave_cnt[w][threadIdx.x];
+    block_hist[(size_t)blockIdx.x * E + threadIdx.x] = sum;
+  }
+}
+
 template <int E, int NCHUNK, bool QUANT, bool LN = false>
 __global__ __launch_bounds__(WAVES_PER_BLOCK * 64, 3) void gate_top2_reg_kernel(
-    const uint4* __restrict__ x, const uint4* __restrict__ wg, int T, int32_t* __restrict__ idx,
-    uint16_t* __restrict__ wout, GateQuant q) {
+    const uint4* __restrict__ x, const uint4* __restrict__ wg, int T, int tpb, int32_t* __restrict__ idx,
+    uint16_t* __restrict__ wout, int32_t* __restrict__ block_hist, GateQuant q) {
   const int lane = threadIdx.x & 63;
-  const int wave = blockIdx.x * WAVES_PER_BLOCK + (threadIdx.x >> 6);
-  const int nwaves = gridDim.x * WAVES_PER_BLOCK;
   constexpr int ROW16 = NCHUNK * 64;  // 16-byte units per row
+  int t = blockIdx.x * tpb + (threadIdx.x >> 6);
+  const int t_end = min(T, (int)(blockIdx.x + 1) * tpb);
+  // the wave's first token is requested before the block copies the gate weight: the two latencies overlap
+  uint4 cur[NCHUNK], nxt[NCHUNK];
+  if (t < t_end) {
+#pragma unroll
+    for (int c = 0; c < NCHUNK; ++c) cur[c] = x[(size_t)t * ROW16 + c * 64 + lane];
+  }
   // The gate weight (E rows) sits in LDS, not in registers: 80 registers less per lane, i.e. four waves per SIMD
   // instead of two, which is what a kernel that only streams needs. A lane reads the same 16-byte units of every
   // row for every token (lane-contiguous, conflict-free).
@@ -211,8 +239,9 @@ __global__ __launch_bounds__(WAVES_PER_BLOCK * 64, 3) void gate_top2_reg_kernel(
   for (int i = threadIdx.x; i < E * ROW16; i += WAVES_PER_BLOCK * 64) w[i] = wg[i];
   __syncthreads();
 
-  int t = wave;
-  if (t >= T) return;
+  int cnt[E];
+#pragma unroll
+  for (int e = 0; e < E; ++e) cnt[e] = 0;
   // the 1/scale_input of every expert, read once: a load that depends on the routing inside the token loop
   // would make every token wait for its predecessor's stores (loads and stores retire in order)
   float inv_e[E], invs = -1.0f;
@@ -221,12 +250,9 @@ __global__ __launch_bounds__(WAVES_PER_BLOCK * 64, 3) void gate_top2_reg_kernel(
     for (int e = 0; e < E; ++e) inv_e[e] = hdmoe_q_inv_scale(q.scale_in.p[e]);
     invs = hdmoe_q_uniform(hdmoe_q_inv_scale(q.shared_scale));
   }
-  uint4 cur[NCHUNK], nxt[NCHUNK];
-#pragma unroll
-  for (int c = 0; c < NCHUNK; ++c) cur[c] = x[(size_t)t * ROW16 + c * 64 + lane];
-  for (; t < T; t += nwaves) {
-    const int tn = t + nwaves;
-    if (tn < T) {
+  for (; t < t_end; t += WAVES_PER_BLOCK) {
+    const int tn = t + WAVES_PER_BLOCK;
+    if (tn < t_end) {
 #pragma unroll
       for (int c = 0; c < NCHUNK; ++c) nxt[c] = x[(size_t)tn * ROW16 + c * 64 + lane];
     }
@@ -254,6 +280,8 @@ __global__ __launch_bounds__(WAVES_PER_BLOCK * 64, 3) void gate_top2_reg_kernel(
     }
     int i0, i1;
     finish_token<E>(logit, lane, t, idx, wout, i0, i1);
+#pragma unroll
+    for (int e = 0; e < E; ++e) cnt[e] += (i0 == e) + (i1 == e);
     if constexpr (QUANT) {
       float inv0 = inv_e[0], inv1 = inv_e[0];
 #pragma unroll
@@ -283,18 +311,21 @@ __global__ __launch_bounds__(WAVES_PER_BLOCK * 64, 3) void gate_top2_reg_kernel(
 #pragma unroll
     for (int c = 0; c < NCHUNK; ++c) cur[c] = nxt[c];
   }
+  write_block_hist<E>(cnt, block_hist);
 }
 
 // Any D that is a multiple of 8: Wg is re-read through the cache hierarchy.
 template <int E, bool QUANT>
 __global__ __launch_bounds__(WAVES_PER_BLOCK * 64) void gate_top2_generic_kernel(
-    const uint4* __restrict__ x, const uint4* __restrict__ wg, int T, int D, int32_t* __restrict__ idx,
-    uint16_t* __restrict__ wout, GateQuant q) {
+    const uint4* __restrict__ x, const uint4* __restrict__ wg, int T, int D, int tpb, int32_t* __restrict__ idx,
+    uint16_t* __restrict__ wout, int32_t* __restrict__ block_hist, GateQuant q) {
   const int lane = threadIdx.x & 63;
-  const int wave = blockIdx.x * WAVES_PER_BLOCK + (threadIdx.x >> 6);
-  const int nwaves = gridDim.x * WAVES_PER_BLOCK;
   const int row16 = D / 8;
-  for (int t = wave; t < T; t += nwaves) {
+  const int t_end = min(T, (int)(blockIdx.x + 1) * tpb);
+  int cnt[E];
+#pragma unroll
+  for (int e = 0; e < E; ++e) cnt[e] = 0;
+  for (int t = blockIdx.x * tpb + (threadIdx.x >> 6); t < t_end; t += WAVES_PER_BLOCK) {
     float logit[E];
 #pragma unroll
     for (int e = 0; e < E; ++e) logit[e] = 0.0f;
@@ -305,6 +336,8 @@ __global__ __launch_bounds__(WAVES_PER_BLOCK * 64) void gate_top2_generic_kernel
     }
     int i0, i1;
     finish_token<E>(logit, lane, t, idx, wout, i0, i1);
+#pragma unroll
+    for (int e = 0; e < E; ++e) cnt[e] += (i0 == e) + (i1 == e);
     if constexpr (QUANT) {
       const float inv0 = hdmoe_q_uniform(hdmoe_q_inv_scale(q.scale_in.p[i0]));
       const float inv1 = hdmoe_q_uniform(hdmoe_q_inv_scale(q.scale_in.p[i1]));
@@ -319,18 +352,15 @@ __global__ __launch_bounds__(WAVES_PER_BLOCK * 64) void gate_top2_generic_kernel
       }
     }
   }
+  write_block_hist<E>(cnt, block_hist);
 }
 
 template <int E>
 int launch_gate(const void* x, const void* wg, int T, int D, int32_t* idx, void* w, const GateQuant* quant,
-                hipStream_t s, const char* what) {
-  // at least two tokens per wave amortise the block's copy of the gate weight into LDS; at most three blocks per CU,
-  // which is what the register kernels' 12 waves per CU hold at once (the waves stride over the tokens)
-  constexpr int TOKENS_PER_WAVE = 2;
-  int blocks = (T + WAVES_PER_BLOCK * TOKENS_PER_WAVE - 1) / (WAVES_PER_BLOCK * TOKENS_PER_WAVE);
-  if (blocks < 1) blocks = 1;
-  if (blocks > HDMOE_NUM_CU * 3) blocks = HDMOE_NUM_CU * 3;
-  dim3 grid(blocks), block(WAVES_PER_BLOCK * 64);
+                int32_t* block_hist, hipStream_t s, const char* what) {
+  const int tpb = hdmoe_gate_tokens_per_block(T);
+  const int blocks = (T + tpb - 1) / tpb;
+  dim3 grid(blocks < 1 ? 1 : blocks), block(WAVES_PER_BLOCK * 64);
   const uint4* xp = static_cast<const uint4*>(x);
   const uint4* wp = static_cast<const uint4*>(wg);
   uint16_t* wo = static_cast<uint16_t*>(w);
@@ -340,22 +370,27 @@ int launch_gate(const void* x, const void* wg, int T, int D, int32_t* idx, void*
   constexpr int ER = E <= 4 ? E : 4;  // the register kernel is only instantiated for up to 4 experts
   if (E <= 4 && D == 2560) {
     if (quant && q.mod_scale != nullptr)
-      hipLaunchKernelGGL((gate_top2_reg_kernel<ER, 5, true, true>), grid, block, 0, s, xp, wp, T, idx, wo, q);
-    else if (quant) hipLaunchKernelGGL((gate_top2_reg_kernel<ER, 5, true>), grid, block, 0, s, xp, wp, T, idx, wo, q);
-    else hipLaunchKernelGGL((gate_top2_reg_kernel<ER, 5, false>), grid, block, 0, s, xp, wp, T, idx, wo, q);
+      hipLaunchKernelGGL((gate_top2_reg_kernel<ER, 5, true, true>), grid, block, 0, s, xp, wp, T, tpb, idx, wo, block_hist, q);
+    else if (quant)
+      hipLaunchKernelGGL((gate_top2_reg_kernel<ER, 5, true>), grid, block, 0, s, xp, wp, T, tpb, idx, wo, block_hist, q);
+    else
+      hipLaunchKernelGGL((gate_top2_reg_kernel<ER, 5, false>), grid, block, 0, s, xp, wp, T, tpb, idx, wo, block_hist, q);
   } else {
     if (q.mod_scale != nullptr) return hdmoe_fail(HDMOE_E_SHAPE, "%s: the LayerNorm variant needs D = 2560 and E <= 4", what);
-    if (quant) hipLaunchKernelGGL((gate_top2_generic_kernel<E, true>), grid, block, 0, s, xp, wp, T, D, idx, wo, q);
-    else hipLaunchKernelGGL((gate_top2_generic_kernel<E, false>), grid, block, 0, s, xp, wp, T, D, idx, wo, q);
+    if (quant)
+      hipLaunchKernelGGL((gate_top2_generic_kernel<E, true>), grid, block, 0, s, xp, wp, T, D, tpb, idx, wo, block_hist, q);
+    else
+      hipLaunchKernelGGL((gate_top2_generic_kernel<E, false>), grid, block, 0, s, xp, wp, T, D, tpb, idx, wo, block_hist, q);
   }
   return hdmoe_check_launch(what);
 }
 
 int dispatch_gate(const void* x_bf16, const void* gate_w_bf16, int T, int D, int E, int32_t* topk_idx,
-                  void* topk_weight_bf16, const GateQuant* quant, hipStream_t s, const char* what) {
+                  void* topk_weight_bf16, const GateQuant* quant, int32_t* block_hist, hipStream_t s,
+                  const char* what) {
   switch (E) {
 #define HDMOE_GATE_CASE(n) \
-  case n: return launch_gate<n>(x_bf16, gate_w_bf16, T, D, topk_idx, topk_weight_bf16, quant, s, what);
+  case n: return launch_gate<n>(x_bf16, gate_w_bf16, T, D, topk_idx, topk_weight_bf16, quant, block_hist, s, what);
     HDMOE_GATE_CASE(2) HDMOE_GATE_CASE(3) HDMOE_GATE_CASE(4) HDMOE_GATE_CASE(5) HDMOE_GATE_CASE(6)
     HDMOE_GATE_CASE(7) HDMOE_GATE_CASE(8) HDMOE_GATE_CASE(9) HDMOE_GATE_CASE(10) HDMOE_GATE_CASE(11)
     HDMOE_GATE_CASE(12) HDMOE_GATE_CASE(13) HDMOE_GATE_CASE(14) HDMOE_GATE_CASE(15) HDMOE_GATE_CASE(16)
@@ -426,8 +461,31 @@ extern "C" int hdmoe_gate_top2(const void* x_bf16, const void* gate_w_bf16, int 
   if (T < 0 || D <= 0 || D % 8 != 0)
     return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_gate_top2: T=%d D=%d (D must be a positive multiple of 8)", T, D);
   if (T == 0) return HDMOE_OK;
-  return dispatch_gate(x_bf16, gate_w_bf16, T, D, E, topk_idx, topk_weight_bf16, nullptr,
+  return dispatch_gate(x_bf16, gate_w_bf16, T, D, E, topk_idx, topk_weight_bf16, nullptr, nullptr,
                        static_cast<hipStream_t>(stream), "hdmoe_gate_top2");
+}
+
+// Tokens per block of the gate kernels, a pure function of T: a power of two between WAVES_PER_BLOCK and 128 (so
+// that the dispatch's chunks of 128 or 1024 tokens are whole numbers of blocks), the smallest that keeps the grid
+// at about three blocks per CU (the register kernels' 12 waves per CU) and gives a block's copy of the gate weight
+// into LDS at least two tokens per wave to pay for.
+int hdmoe_gate_tokens_per_block(int T) {
+  int tpb = WAVES_PER_BLOCK * 2;
+  while (tpb < 128 && (T + tpb - 1) / tpb > HDMOE_NUM_CU * 3) tpb *= 2;
+  return tpb;
+}
+
+// Bytes of the per-block expert histograms the gate kernels can leave for the dispatch.
+size_t hdmoe_gate_hist_bytes(int T, int E) {
+  const int tpb = hdmoe_gate_tokens_per_block(T);
+  const size_t blocks = T > 0 ? ((size_t)T + tpb - 1) / tpb : 1;
+  return hdmoe_align_up(blocks * (size_t)E * sizeof(int32_t), 256);
+}
+
+// The same gate for the one-call layer, which also takes the histograms.
+int hdmoe_launch_gate(const void* x_bf16, const void* gate_w_bf16, int T, int D, int E, int32_t* topk_idx,
+                      void* topk_weight_bf16, int32_t* block_hist, hipStream_t s, const char* what) {
+  return dispatch_gate(x_bf16, gate_w_bf16, T, D, E, topk_idx, topk_weight_bf16, nullptr, block_hist, s, what);
 }
 
 // The gate of the one-call layer with fp8 experts: routing plus the token's three fp8 rows in one pass over x.
@@ -438,7 +496,7 @@ int hdmoe_launch_gate_quant(const void* x_bf16, const void* gate_w_bf16, int T, 
                             void* topk_weight_bf16, const float* const* scale_input, const float* shared_scale,
                             void* xq_routed, void* xq_shared, hipStream_t s, const char* what,
                             const void* mod_scale = nullptr, const void* mod_shift = nullptr, int tokens_per_batch = 0,
-                            float ln_eps = 0.0f) {
+                            float ln_eps = 0.0f, int32_t* block_hist = nullptr) {
   GateQuant q;
   memset(&q, 0, sizeof(q));
   if (mod_scale != nullptr) {
@@ -451,7 +509,7 @@ int hdmoe_launch_gate_quant(const void* x_bf16, const void* gate_w_bf16, int T, 
   q.shared_scale = shared_scale;
   q.xq_routed = static_cast<uint2*>(xq_routed);
   q.xq_shared = static_cast<uint2*>(xq_shared);
-  return dispatch_gate(x_bf16, gate_w_bf16, T, D, E, topk_idx, topk_weight_bf16, &q, s, what);
+  return dispatch_gate(x_bf16, gate_w_bf16, T, D, E, topk_idx, topk_weight_bf16, &q, block_hist, s, what);
 }
 
 extern "C" int hdmoe_ln_modulate_bf16(const void* x_bf16, const void* scale_bf16, const void* shift_bf16, int T, int D,

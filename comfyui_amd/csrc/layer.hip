@@ -19,7 +19,12 @@ int hdmoe_launch_gate_quant(const void* x_bf16, const void* gate_w_bf16, int T, 
                             void* topk_weight_bf16, const float* const* scale_input, const float* shared_scale,
                             void* xq_routed, void* xq_shared, hipStream_t s, const char* what,
                             const void* mod_scale = nullptr, const void* mod_shift = nullptr, int tokens_per_batch = 0,
-                            float ln_eps = 0.0f);
+                            float ln_eps = 0.0f, int32_t* block_hist = nullptr);
+int hdmoe_launch_gate(const void* x_bf16, const void* gate_w_bf16, int T, int D, int E, int32_t* topk_idx,
+                      void* topk_weight_bf16, int32_t* block_hist, hipStream_t s, const char* what);
+int hdmoe_launch_dispatch_scatter(const int32_t* topk_idx, int T, int E, int32_t* counts, int32_t* offsets,
+                                  int32_t* perm, int32_t* inv_perm, const int32_t* block_hist, int tokens_per_hist,
+                                  hipStream_t s, const char* what);
 bool hdmoe_gate_quant_takes_ln(int D, int E);
 int hdmoe_launch_combine(const void* y_sorted_bf16, const int32_t* inv_perm, const void* topk_weight_bf16,
                          const void* shared_bf16, const void* gate_bf16, const void* residual_bf16, int tokens_per_batch,
@@ -51,7 +56,8 @@ extern "C" int hdmoe_layer_layout_get(int T, int D, int H, int Hs, int E, int we
   out->offsets = take((size_t)(E + 1) * 4);
   out->perm = take(n * 4);
   out->inv_perm = take(n * 4);
-  out->dispatch_ws = take(hdmoe_dispatch_workspace_bytes(T, E));
+  // per-block expert histograms of the gate kernel (the first pass of the dispatch)
+  out->dispatch_ws = take(hdmoe_gate_hist_bytes(T, E));
   // a: routed rows sorted by expert [2T,D], then (fp8 only) the token-order copy for the shared expert [T,D]
   out->a = take((n + ((fp8 && Hs > 0) ? (size_t)T : 0)) * D * eb);
   // h: routed [2T,H] then shared [T,Hs]
@@ -113,6 +119,7 @@ extern "C" int hdmoe_moe_ffn(const hdmoe_layer_args* p, hdmoe_stream_t stream) {
   int32_t* offsets = reinterpret_cast<int32_t*>(ws + l.offsets);
   int32_t* perm = reinterpret_cast<int32_t*>(ws + l.perm);
   int32_t* inv_perm = reinterpret_cast<int32_t*>(ws + l.inv_perm);
+  int32_t* hist = reinterpret_cast<int32_t*>(ws + l.dispatch_ws);
   uint8_t* a_routed = ws + l.a;
   uint8_t* a_shared = a_routed + (size_t)n * D * eb;  // fp8 only
   uint8_t* h_routed = ws + l.h;
@@ -177,14 +184,16 @@ extern "C" int hdmoe_moe_ffn(const hdmoe_layer_args* p, hdmoe_stream_t stream) {
                                          one_copy ? nullptr : a_routed, (Hs > 0 || one_copy) ? a_shared : nullptr, s,
                                          "hdmoe_moe_ffn (gate + quantise)",
                                          ln_in_gate ? p->mod_scale : nullptr, ln_in_gate ? p->mod_shift : nullptr,
-                                         p->tokens_per_batch, p->ln_eps))
+                                         p->tokens_per_batch, p->ln_eps, hist))
       return rc;
   } else {
-    if (int rc = hdmoe_gate_top2(xin, p->gate_w, T, D, E, idx, tw, stream)) return rc;
+    if (D % 8 != 0) return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_moe_ffn: D=%d must be a multiple of 8", D);
+    if (int rc = hdmoe_launch_gate(xin, p->gate_w, T, D, E, idx, tw, hist, s, "hdmoe_moe_ffn (gate)")) return rc;
   }
   mark();
-  if (int rc = hdmoe_dispatch(idx, T, E, counts, offsets, perm, inv_perm, ws + l.dispatch_ws,
-                              hdmoe_dispatch_workspace_bytes(T, E), stream))
+  // the gate kernel has left the expert histogram of each of its blocks: the dispatch is its second pass alone
+  if (int rc = hdmoe_launch_dispatch_scatter(idx, T, E, counts, offsets, perm, inv_perm, hist,
+                                             hdmoe_gate_tokens_per_block(T), s, "hdmoe_moe_ffn (dispatch)"))
     return rc;
   mark();
 

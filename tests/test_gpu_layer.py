@@ -248,3 +248,42 @@ def test_layer_casts_activations_in_the_gate_kernel_bit_exactly(dev, dim, E, sca
                 assert torch.equal(a[2 * sel + slot], want), (slot, e)
     want = cast(xc, scales.get("shared_experts") if scaled else None)
     assert torch.equal(a[2 * T:], want)
+
+
+@pytest.mark.parametrize("weights", ["fp8", "bf16"])
+@pytest.mark.parametrize("dim,E,T", [(256, 4, 1), (256, 4, 7), (256, 3, 129), (2560, 4, 333), (256, 8, 4097),
+                                     (2560, 4, 8192), (256, 4, 33000)])
+def test_layer_dispatch_from_gate_histograms(dev, weights, dim, E, T):
+    """Inside the one-call layer the gate kernel counts (one expert histogram per block of tokens) and the dispatch
+    runs its second pass alone. counts, offsets, perm and inv_perm in the layer's workspace: equal to the CPU
+    checker's stable sort of the same routing, at token counts around the block and chunk sizes (one token, a
+    partial block, more than one chunk, the large-chunk form above 32768 tokens), with 3, 4 and 8 experts and both
+    gate kernels (row in registers at D = 2560, generic otherwise)."""
+    from comfyui_amd import functional as HF
+    from comfyui_amd import _lib
+    hidden_arg = 512
+    master, g = synth.make_weights(11, dim=dim, hidden_arg=hidden_arg, num_experts=E)
+    sd = synth.to_state_dict(master, weights)
+    x = synth.make_input(g, T, dim=dim)
+    m = synth.build_module({k: v.to(dev) for k, v in sd.items()}, weights, dev, dim=dim, hidden_arg=hidden_arg,
+                           num_experts=E)
+    x2 = x.reshape(T, dim).to(dev)
+    wdt, experts, shared, keep = m._collect(x2)
+    H, Hs = m.experts[0].w1.weight.shape[0], m.shared_experts.w1.weight.shape[0]
+    code = _lib.W_E4M3FN if weights == "fp8" else _lib.W_BF16
+    lay = HF.layer_layout(T, dim, H, Hs, E, code)
+    ws = torch.full((lay.total,), 0xAB, dtype=torch.uint8, device=dev)   # stale bytes: nothing may rely on zeros
+    y, idx, _ = HF.moe_ffn(x2, m.gate.weight, experts, shared, H, Hs, wdt, workspace=ws, want_routing=True)
+    torch.cuda.synchronize()
+    assert not bool(torch.isnan(y.float()).any())
+
+    def ints(off, n):
+        return ws[off:off + 4 * n].cpu().view(torch.int32)
+    counts_r, offs_r, perm_r, inv_r = O.dispatch(idx.cpu(), E)
+    assert torch.equal(ints(lay.counts, E), counts_r.to(torch.int32))
+    assert torch.equal(ints(lay.offsets, E + 1), offs_r.to(torch.int32))
+    assert torch.equal(ints(lay.perm, 2 * T), perm_r.to(torch.int32))
+    assert torch.equal(ints(lay.inv_perm, 2 * T), inv_r.reshape(-1).to(torch.int32))
+    # the stand-alone stage (its own counting pass) agrees
+    for a, b in zip(HF.dispatch(idx, E), (counts_r, offs_r, perm_r, inv_r)):
+        assert torch.equal(a.cpu(), b)
