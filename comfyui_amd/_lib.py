@@ -15,6 +15,7 @@ LIB_PATH = os.path.join(_HERE, "libhdmoe.so")
 
 W_BF16 = 0
 W_E4M3FN = 1
+W_F16 = 2
 SRC_BF16 = 0
 SRC_F32 = 2
 ACT_NONE = 0
@@ -72,6 +73,7 @@ SIGNATURES = {
     "hdmoe_version": (c_int, []),
     "hdmoe_last_error": (ctypes.c_char_p, []),
     "hdmoe_gate_top2": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),
+    "hdmoe_gate_top2_f16": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),
     "hdmoe_renorm_top2_bf16": (c_int, [c_void_p, c_int, c_void_p, c_void_p]),
     "hdmoe_dispatch_workspace_bytes": (c_size_t, [c_int, c_int]),
     "hdmoe_dispatch": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t,
@@ -91,9 +93,13 @@ SIGNATURES = {
                                   c_void_p]),
     "hdmoe_silu_mul_bf16": (c_int, [c_void_p, c_void_p, c_int64, c_void_p, c_void_p]),
     "hdmoe_gelu_bf16": (c_int, [c_void_p, c_int64, c_void_p, c_void_p]),
+    "hdmoe_gelu_f16": (c_int, [c_void_p, c_int64, c_void_p, c_void_p]),
     "hdmoe_scale_to_bf16": (c_int, [c_int, c_void_p, c_int64, c_void_p, c_void_p, c_void_p]),
     "hdmoe_grouped_linear": (c_int, [c_void_p, c_void_p, c_int, c_int, ctypes.POINTER(LinearWeights), c_void_p, c_void_p,
                                      c_int, ctypes.POINTER(LinearWeights), c_void_p, c_int, c_int, c_int, c_void_p]),
+    "hdmoe_grouped_linear_f16": (c_int, [c_void_p, c_void_p, c_int, c_int, ctypes.POINTER(LinearWeights), c_void_p,
+                                         c_void_p, c_int, ctypes.POINTER(LinearWeights), c_void_p, c_int, c_int, c_int,
+                                         c_void_p]),
     "hdmoe_stochastic_round_e4m3fn": (c_int, [c_int, c_void_p, ctypes.c_int64, c_void_p, ctypes.c_uint64, c_void_p,
                                               c_void_p]),
     "hdmoe_ln_modulate_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, ctypes.c_float, c_void_p,
@@ -102,6 +108,7 @@ SIGNATURES = {
                                              c_int, c_void_p, c_void_p]),
     "hdmoe_gated_residual_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p]),
     "hdmoe_combine": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p]),
+    "hdmoe_combine_f16": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p]),
     "hdmoe_layer_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int, c_int]),
     "hdmoe_moe_ffn": (c_int, [ctypes.POINTER(LayerArgs), c_void_p]),
     "hdmoe_ffn_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),

@@ -122,14 +122,15 @@ __global__ __launch_bounds__(THREADS) void silu_mul_kernel(const uint4* __restri
 // (/root/reference/comfy/ldm/hunyuan3dv2_1/hunyuandit.py:14-26), for projections whose Linear is not the plain bf16 one.
 __device__ __forceinline__ float gelu1(float h) { return 0.5f * h * (1.0f + erff(h * 0.70710678118654752440f)); }
 
+template <class A>  // HdmoeBf16 or HdmoeF16: the tensor's element format
 __global__ __launch_bounds__(THREADS) void gelu_kernel(const uint4* __restrict__ x, int64_t n8, uint4* __restrict__ out) {
   for (int64_t i = blockIdx.x * (int64_t)THREADS + threadIdx.x; i < n8; i += (int64_t)gridDim.x * THREADS) {
     const uint4 v = x[i];
     uint4 o;
-    o.x = pack_bf16(gelu1(bf16_lo(v.x)), gelu1(bf16_hi(v.x)));
-    o.y = pack_bf16(gelu1(bf16_lo(v.y)), gelu1(bf16_hi(v.y)));
-    o.z = pack_bf16(gelu1(bf16_lo(v.z)), gelu1(bf16_hi(v.z)));
-    o.w = pack_bf16(gelu1(bf16_lo(v.w)), gelu1(bf16_hi(v.w)));
+    o.x = A::pack(gelu1(A::lo(v.x)), gelu1(A::hi(v.x)));
+    o.y = A::pack(gelu1(A::lo(v.y)), gelu1(A::hi(v.y)));
+    o.z = A::pack(gelu1(A::lo(v.z)), gelu1(A::hi(v.z)));
+    o.w = A::pack(gelu1(A::lo(v.w)), gelu1(A::hi(v.w)));
     out[i] = o;
   }
 }
@@ -159,20 +160,27 @@ struct CombineExtra {
   int tokens_per_batch;
 };
 
+// A: the element format of every tensor of the call (HdmoeBf16 or HdmoeF16); each "bf16(...)" above is a rounding to it.
+template <class A>
 __device__ __forceinline__ float comb1(float y0, float y1, float w0, float w1, float sh, bool has_shared, float g,
                                        float res, bool has_gate) {
-  float s = round_bf16(round_bf16(y0 * w0) + round_bf16(y1 * w1));
-  if (has_shared) s = has_gate ? round_bf16(s + sh) : s + sh;
-  if (has_gate) s = round_bf16(g * s) + res;
+  // no fused multiply-add: with fp16 the compiler narrows these fp32 operations between two roundings to fp16
+  // operations (exact) and would then fuse a product into the following sum, dropping the product's rounding
+#pragma clang fp contract(off)
+  float s = A::round(A::round(y0 * w0) + A::round(y1 * w1));
+  if (has_shared) s = has_gate ? A::round(s + sh) : s + sh;
+  if (has_gate) s = A::round(g * s) + res;
   return s;
 }
 
+template <class A>
 __device__ __forceinline__ uint32_t comb2(uint32_t y0, uint32_t y1, float w0, float w1, uint32_t sh, bool hs, uint32_t g,
                                           uint32_t res, bool hg) {
-  return pack_bf16(comb1(bf16_lo(y0), bf16_lo(y1), w0, w1, bf16_lo(sh), hs, bf16_lo(g), bf16_lo(res), hg),
-                   comb1(bf16_hi(y0), bf16_hi(y1), w0, w1, bf16_hi(sh), hs, bf16_hi(g), bf16_hi(res), hg));
+  return A::pack(comb1<A>(A::lo(y0), A::lo(y1), w0, w1, A::lo(sh), hs, A::lo(g), A::lo(res), hg),
+                 comb1<A>(A::hi(y0), A::hi(y1), w0, w1, A::hi(sh), hs, A::hi(g), A::hi(res), hg));
 }
 
+template <class A>
 __global__ __launch_bounds__(THREADS) void combine_kernel(const uint4* __restrict__ y, const int2* __restrict__ inv_perm,
                                                           const uint32_t* __restrict__ w, const uint4* __restrict__ shared,
                                                           int T, int row16, CombineExtra ex, uint4* __restrict__ out) {
@@ -184,7 +192,7 @@ __global__ __launch_bounds__(THREADS) void combine_kernel(const uint4* __restric
   for (int t = wave; t < T; t += nwaves) {
     const int2 r = inv_perm[t];
     const uint32_t wp = w[t];
-    const float w0 = bf16_lo(wp), w1 = bf16_hi(wp);
+    const float w0 = A::lo(wp), w1 = A::hi(wp);
     const uint4* y0 = y + (long)r.x * row16;
     const uint4* y1 = y + (long)r.y * row16;
     const long brow = hg ? (long)(t / ex.tokens_per_batch) * row16 : 0;
@@ -194,10 +202,10 @@ __global__ __launch_bounds__(THREADS) void combine_kernel(const uint4* __restric
       if (hs) sh = shared[(long)t * row16 + u];
       if (hg) { g = ex.gate[brow + u]; res = ex.residual[(long)t * row16 + u]; }
       uint4 o;
-      o.x = comb2(a.x, b.x, w0, w1, sh.x, hs, g.x, res.x, hg);
-      o.y = comb2(a.y, b.y, w0, w1, sh.y, hs, g.y, res.y, hg);
-      o.z = comb2(a.z, b.z, w0, w1, sh.z, hs, g.z, res.z, hg);
-      o.w = comb2(a.w, b.w, w0, w1, sh.w, hs, g.w, res.w, hg);
+      o.x = comb2<A>(a.x, b.x, w0, w1, sh.x, hs, g.x, res.x, hg);
+      o.y = comb2<A>(a.y, b.y, w0, w1, sh.y, hs, g.y, res.y, hg);
+      o.z = comb2<A>(a.z, b.z, w0, w1, sh.z, hs, g.z, res.z, hg);
+      o.w = comb2<A>(a.w, b.w, w0, w1, sh.w, hs, g.w, res.w, hg);
       out[(long)t * row16 + u] = o;
     }
   }
@@ -351,9 +359,22 @@ extern "C" int hdmoe_gelu_bf16(const void* x_bf16, int64_t n, void* out_bf16, hd
   const int64_t n8 = n / 8;
   int64_t blocks = (n8 + THREADS - 1) / THREADS;
   if (blocks > HDMOE_NUM_CU * 8) blocks = HDMOE_NUM_CU * 8;
-  hipLaunchKernelGGL(gelu_kernel, dim3((unsigned)blocks), dim3(THREADS), 0, static_cast<hipStream_t>(stream),
+  hipLaunchKernelGGL(gelu_kernel<HdmoeBf16>, dim3((unsigned)blocks), dim3(THREADS), 0, static_cast<hipStream_t>(stream),
                      static_cast<const uint4*>(x_bf16), n8, static_cast<uint4*>(out_bf16));
   return hdmoe_check_launch("hdmoe_gelu_bf16");
+}
+
+extern "C" int hdmoe_gelu_f16(const void* x_f16, int64_t n, void* out_f16, hdmoe_stream_t stream) {
+  HDMOE_REQUIRE_PTR(x_f16);
+  HDMOE_REQUIRE_PTR(out_f16);
+  if (n < 0 || n % 8 != 0) return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_gelu_f16: n=%lld must be a multiple of 8", (long long)n);
+  if (n == 0) return HDMOE_OK;
+  const int64_t n8 = n / 8;
+  int64_t blocks = (n8 + THREADS - 1) / THREADS;
+  if (blocks > HDMOE_NUM_CU * 8) blocks = HDMOE_NUM_CU * 8;
+  hipLaunchKernelGGL(gelu_kernel<HdmoeF16>, dim3((unsigned)blocks), dim3(THREADS), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const uint4*>(x_f16), n8, static_cast<uint4*>(out_f16));
+  return hdmoe_check_launch("hdmoe_gelu_f16");
 }
 
 extern "C" int hdmoe_renorm_top2_bf16(const void* topk_weight_bf16, int T, void* out_bf16, hdmoe_stream_t stream) {
@@ -370,15 +391,34 @@ extern "C" int hdmoe_renorm_top2_bf16(const void* topk_weight_bf16, int T, void*
 
 int hdmoe_launch_combine(const void* y_sorted_bf16, const int32_t* inv_perm, const void* topk_weight_bf16,
                          const void* shared_bf16, const void* gate_bf16, const void* residual_bf16, int tokens_per_batch,
-                         int T, int D, void* out_bf16, hipStream_t s, const char* what) {
+                         int T, int D, void* out_bf16, hipStream_t s, const char* what, bool f16 = false) {
   CombineExtra ex;
   ex.gate = static_cast<const uint4*>(gate_bf16);
   ex.residual = static_cast<const uint4*>(residual_bf16);
   ex.tokens_per_batch = tokens_per_batch > 0 ? tokens_per_batch : 1;
-  hipLaunchKernelGGL(combine_kernel, dim3(row_blocks(T)), dim3(THREADS), 0, s, static_cast<const uint4*>(y_sorted_bf16),
-                     reinterpret_cast<const int2*>(inv_perm), static_cast<const uint32_t*>(topk_weight_bf16),
-                     static_cast<const uint4*>(shared_bf16), T, D / 8, ex, static_cast<uint4*>(out_bf16));
+  if (f16)
+    hipLaunchKernelGGL(combine_kernel<HdmoeF16>, dim3(row_blocks(T)), dim3(THREADS), 0, s,
+                       static_cast<const uint4*>(y_sorted_bf16), reinterpret_cast<const int2*>(inv_perm),
+                       static_cast<const uint32_t*>(topk_weight_bf16), static_cast<const uint4*>(shared_bf16), T, D / 8,
+                       ex, static_cast<uint4*>(out_bf16));
+  else
+    hipLaunchKernelGGL(combine_kernel<HdmoeBf16>, dim3(row_blocks(T)), dim3(THREADS), 0, s,
+                       static_cast<const uint4*>(y_sorted_bf16), reinterpret_cast<const int2*>(inv_perm),
+                       static_cast<const uint32_t*>(topk_weight_bf16), static_cast<const uint4*>(shared_bf16), T, D / 8,
+                       ex, static_cast<uint4*>(out_bf16));
   return hdmoe_check_launch(what);
+}
+
+extern "C" int hdmoe_combine_f16(const void* y_sorted_f16, const int32_t* inv_perm, const void* topk_weight_f16,
+                                 const void* shared_f16, int T, int D, void* out_f16, hdmoe_stream_t stream) {
+  HDMOE_REQUIRE_PTR(y_sorted_f16);
+  HDMOE_REQUIRE_PTR(inv_perm);
+  HDMOE_REQUIRE_PTR(topk_weight_f16);
+  HDMOE_REQUIRE_PTR(out_f16);
+  if (T < 0 || D <= 0 || D % 8 != 0) return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_combine_f16: T=%d D=%d", T, D);
+  if (T == 0) return HDMOE_OK;
+  return hdmoe_launch_combine(y_sorted_f16, inv_perm, topk_weight_f16, shared_f16, nullptr, nullptr, 1, T, D, out_f16,
+                              static_cast<hipStream_t>(stream), "hdmoe_combine_f16", true);
 }
 
 extern "C" int hdmoe_combine(const void* y_sorted_bf16, const int32_t* inv_perm, const void* topk_weight_bf16,

@@ -46,15 +46,28 @@ __device__ __forceinline__ float exp_neg(float x) {
 __device__ __forceinline__ float bf16_lo(uint32_t u) { return __uint_as_float(u << 16); }
 __device__ __forceinline__ float bf16_hi(uint32_t u) { return __uint_as_float(u & 0xffff0000u); }
 
+// The element format of x, the gate weight and the routing weights: bf16 (HiDream, Hunyuan3D) or fp16 (the dtype
+// Hunyuan3D runs in where the device takes it). Logits and scores are rounded to that format between the steps.
+struct GateBf16 {
+  static __device__ __forceinline__ float lo(uint32_t u) { return bf16_lo(u); }
+  static __device__ __forceinline__ float hi(uint32_t u) { return bf16_hi(u); }
+  static __device__ __forceinline__ float round(float f) { return hdmoe_round_bf16(f); }
+  static __device__ __forceinline__ uint32_t pack(float a, float b) {
+    return (uint32_t)hdmoe_f32_to_bf16(a) | ((uint32_t)hdmoe_f32_to_bf16(b) << 16);
+  }
+};
+typedef HdmoeF16 GateF16;
+
+template <class A = GateBf16>
 __device__ __forceinline__ float dot8(const uint4& a, const uint4& b, float acc) {
-  acc = __builtin_fmaf(bf16_lo(a.x), bf16_lo(b.x), acc);
-  acc = __builtin_fmaf(bf16_hi(a.x), bf16_hi(b.x), acc);
-  acc = __builtin_fmaf(bf16_lo(a.y), bf16_lo(b.y), acc);
-  acc = __builtin_fmaf(bf16_hi(a.y), bf16_hi(b.y), acc);
-  acc = __builtin_fmaf(bf16_lo(a.z), bf16_lo(b.z), acc);
-  acc = __builtin_fmaf(bf16_hi(a.z), bf16_hi(b.z), acc);
-  acc = __builtin_fmaf(bf16_lo(a.w), bf16_lo(b.w), acc);
-  acc = __builtin_fmaf(bf16_hi(a.w), bf16_hi(b.w), acc);
+  acc = __builtin_fmaf(A::lo(a.x), A::lo(b.x), acc);
+  acc = __builtin_fmaf(A::hi(a.x), A::hi(b.x), acc);
+  acc = __builtin_fmaf(A::lo(a.y), A::lo(b.y), acc);
+  acc = __builtin_fmaf(A::hi(a.y), A::hi(b.y), acc);
+  acc = __builtin_fmaf(A::lo(a.z), A::lo(b.z), acc);
+  acc = __builtin_fmaf(A::hi(a.z), A::hi(b.z), acc);
+  acc = __builtin_fmaf(A::lo(a.w), A::lo(b.w), acc);
+  acc = __builtin_fmaf(A::hi(a.w), A::hi(b.w), acc);
   return acc;
 }
 
@@ -81,12 +94,12 @@ __device__ __forceinline__ float wave_sum(float v) {
   return v;
 }
 
-template <int E>
+template <int E, class A = GateBf16>
 __device__ __forceinline__ void finish_token(float (&logit)[E], int lane, int t, int32_t* idx,
                                              uint16_t* wout, int& first, int& second) {
 #pragma unroll
   for (int e = 0; e < E; ++e) {
-    logit[e] = hdmoe_round_bf16(wave_sum(logit[e]));  // F.linear output is a bf16 tensor
+    logit[e] = A::round(wave_sum(logit[e]));  // F.linear output is a tensor of the activation format
   }
   float mx = logit[0];
 #pragma unroll
@@ -100,7 +113,7 @@ __device__ __forceinline__ void finish_token(float (&logit)[E], int lane, int t,
   }
   float score[E];
 #pragma unroll
-  for (int e = 0; e < E; ++e) score[e] = hdmoe_round_bf16(__fdiv_rn(ex[e], sum));  // softmax output is bf16
+  for (int e = 0; e < E; ++e) score[e] = A::round(__fdiv_rn(ex[e], sum));  // so is the softmax output
   // first two of a stable descending sort: strict '>' keeps the lower index on ties
   int i0 = 0;
   float s0 = score[0];
@@ -118,8 +131,7 @@ __device__ __forceinline__ void finish_token(float (&logit)[E], int lane, int t,
   second = i1;
   if (lane == 0) {
     reinterpret_cast<int2*>(idx)[t] = make_int2(i0, i1);
-    reinterpret_cast<uint32_t*>(wout)[t] =
-        (uint32_t)hdmoe_f32_to_bf16(s0) | ((uint32_t)hdmoe_f32_to_bf16(s1) << 16);
+    reinterpret_cast<uint32_t*>(wout)[t] = A::pack(s0, s1);
   }
 }
 
@@ -315,7 +327,7 @@ __global__ __launch_bounds__(WAVES_PER_BLOCK * 64, 3) void gate_top2_reg_kernel(
 }
 
 // Any D that is a multiple of 8: Wg is re-read through the cache hierarchy.
-template <int E, bool QUANT>
+template <int E, bool QUANT, class A = GateBf16>
 __global__ __launch_bounds__(WAVES_PER_BLOCK * 64) void gate_top2_generic_kernel(
     const uint4* __restrict__ x, const uint4* __restrict__ wg, int T, int D, int tpb, int32_t* __restrict__ idx,
     uint16_t* __restrict__ wout, int32_t* __restrict__ block_hist, GateQuant q) {
@@ -332,10 +344,10 @@ __global__ __launch_bounds__(WAVES_PER_BLOCK * 64) void gate_top2_generic_kernel
     for (int u = lane; u < row16; u += 64) {
       uint4 xv = x[(size_t)t * row16 + u];
 #pragma unroll
-      for (int e = 0; e < E; ++e) logit[e] = dot8(xv, wg[(size_t)e * row16 + u], logit[e]);
+      for (int e = 0; e < E; ++e) logit[e] = dot8<A>(xv, wg[(size_t)e * row16 + u], logit[e]);
     }
     int i0, i1;
-    finish_token<E>(logit, lane, t, idx, wout, i0, i1);
+    finish_token<E, A>(logit, lane, t, idx, wout, i0, i1);
 #pragma unroll
     for (int e = 0; e < E; ++e) cnt[e] += (i0 == e) + (i1 == e);
     if constexpr (QUANT) {
@@ -357,7 +369,7 @@ __global__ __launch_bounds__(WAVES_PER_BLOCK * 64) void gate_top2_generic_kernel
 
 template <int E>
 int launch_gate(const void* x, const void* wg, int T, int D, int32_t* idx, void* w, const GateQuant* quant,
-                int32_t* block_hist, hipStream_t s, const char* what) {
+                int32_t* block_hist, hipStream_t s, const char* what, bool f16) {
   const int tpb = hdmoe_gate_tokens_per_block(T);
   const int blocks = (T + tpb - 1) / tpb;
   dim3 grid(blocks < 1 ? 1 : blocks), block(WAVES_PER_BLOCK * 64);
@@ -368,7 +380,11 @@ int launch_gate(const void* x, const void* wg, int T, int D, int32_t* idx, void*
   memset(&q, 0, sizeof(q));
   if (quant) q = *quant;
   constexpr int ER = E <= 4 ? E : 4;  // the register kernel is only instantiated for up to 4 experts
-  if (E <= 4 && D == 2560) {
+  if (f16) {
+    if (quant) return hdmoe_fail(HDMOE_E_SHAPE, "%s: the fp8 cast takes bf16 activations", what);
+    hipLaunchKernelGGL((gate_top2_generic_kernel<E, false, GateF16>), grid, block, 0, s, xp, wp, T, D, tpb, idx, wo,
+                       block_hist, q);
+  } else if (E <= 4 && D == 2560) {
     if (quant && q.mod_scale != nullptr)
       hipLaunchKernelGGL((gate_top2_reg_kernel<ER, 5, true, true>), grid, block, 0, s, xp, wp, T, tpb, idx, wo, block_hist, q);
     else if (quant)
@@ -387,10 +403,10 @@ int launch_gate(const void* x, const void* wg, int T, int D, int32_t* idx, void*
 
 int dispatch_gate(const void* x_bf16, const void* gate_w_bf16, int T, int D, int E, int32_t* topk_idx,
                   void* topk_weight_bf16, const GateQuant* quant, int32_t* block_hist, hipStream_t s,
-                  const char* what) {
+                  const char* what, bool f16 = false) {
   switch (E) {
 #define HDMOE_GATE_CASE(n) \
-  case n: return launch_gate<n>(x_bf16, gate_w_bf16, T, D, topk_idx, topk_weight_bf16, quant, block_hist, s, what);
+  case n: return launch_gate<n>(x_bf16, gate_w_bf16, T, D, topk_idx, topk_weight_bf16, quant, block_hist, s, what, f16);
     HDMOE_GATE_CASE(2) HDMOE_GATE_CASE(3) HDMOE_GATE_CASE(4) HDMOE_GATE_CASE(5) HDMOE_GATE_CASE(6)
     HDMOE_GATE_CASE(7) HDMOE_GATE_CASE(8) HDMOE_GATE_CASE(9) HDMOE_GATE_CASE(10) HDMOE_GATE_CASE(11)
     HDMOE_GATE_CASE(12) HDMOE_GATE_CASE(13) HDMOE_GATE_CASE(14) HDMOE_GATE_CASE(15) HDMOE_GATE_CASE(16)
@@ -463,6 +479,19 @@ extern "C" int hdmoe_gate_top2(const void* x_bf16, const void* gate_w_bf16, int 
   if (T == 0) return HDMOE_OK;
   return dispatch_gate(x_bf16, gate_w_bf16, T, D, E, topk_idx, topk_weight_bf16, nullptr, nullptr,
                        static_cast<hipStream_t>(stream), "hdmoe_gate_top2");
+}
+
+extern "C" int hdmoe_gate_top2_f16(const void* x_f16, const void* gate_w_f16, int T, int D, int E, int32_t* topk_idx,
+                                   void* topk_weight_f16, hdmoe_stream_t stream) {
+  HDMOE_REQUIRE_PTR(x_f16);
+  HDMOE_REQUIRE_PTR(gate_w_f16);
+  HDMOE_REQUIRE_PTR(topk_idx);
+  HDMOE_REQUIRE_PTR(topk_weight_f16);
+  if (T < 0 || D <= 0 || D % 8 != 0)
+    return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_gate_top2_f16: T=%d D=%d (D must be a positive multiple of 8)", T, D);
+  if (T == 0) return HDMOE_OK;
+  return dispatch_gate(x_f16, gate_w_f16, T, D, E, topk_idx, topk_weight_f16, nullptr, nullptr,
+                       static_cast<hipStream_t>(stream), "hdmoe_gate_top2_f16", true);
 }
 
 // Tokens per block of the gate kernels, a pure function of T: a power of two between WAVES_PER_BLOCK and 128 (so

@@ -43,6 +43,7 @@ typedef int v8i __attribute__((ext_vector_type(8)));
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 
 constexpr int BN = 256;        // weight rows per block tile
 constexpr int BK = 128;        // K bytes per stage
@@ -61,7 +62,10 @@ constexpr int GROUP_M = 4;     // m-tiles per raster band
 constexpr int NTHREADS = 512;
 constexpr int MAX_GROUPS = HDMOE_MAX_EXPERTS + 1;
 
-enum Mode { FP8_SWIGLU = 0, FP8_PLAIN = 1, BF16_SWIGLU = 2, BF16_PLAIN = 3, BF16_PLAIN_BIAS = 4, FP8_PLAIN_BIAS = 5 };
+// F16_PLAIN_BIAS: fp16 activations, weights, bias and outputs (the dtype the Hunyuan3D block runs in where the device
+// takes it); the bf16 kernel with the other 16-bit MFMA and the other rounding.
+enum Mode { FP8_SWIGLU = 0, FP8_PLAIN = 1, BF16_SWIGLU = 2, BF16_PLAIN = 3, BF16_PLAIN_BIAS = 4, FP8_PLAIN_BIAS = 5,
+            F16_PLAIN_BIAS = 6 };
 
 struct GemmGroup {
   const uint8_t* a;     // activations; row indices below are relative to this base
@@ -206,7 +210,9 @@ template <int MODE, int TT>
 __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs args) {
   constexpr bool FP8 = (MODE == FP8_SWIGLU || MODE == FP8_PLAIN || MODE == FP8_PLAIN_BIAS);
   constexpr bool SWIGLU = (MODE == FP8_SWIGLU || MODE == BF16_SWIGLU);
-  constexpr bool BIAS = (MODE == BF16_PLAIN_BIAS || MODE == FP8_PLAIN_BIAS);  // Linear with bias and optional GELU
+  constexpr bool BIAS = (MODE == BF16_PLAIN_BIAS || MODE == FP8_PLAIN_BIAS || MODE == F16_PLAIN_BIAS);  // Linear with bias and optional GELU
+  constexpr bool F16 = MODE == F16_PLAIN_BIAS;
+  using Act = std::conditional_t<F16, HdmoeF16, HdmoeBf16>;  // element format of activations, bias and outputs
   constexpr int WAVE_TOK = 32 * TT;        // tokens per wave row
   constexpr int BM = 2 * WAVE_TOK;         // tokens per block tile
   constexpr int A_SLABS = BM / 64;         // 64-row slabs of the token tile
@@ -410,22 +416,24 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
 #pragma unroll
       for (int ks = 0; ks < 4; ++ks) {
         const int c0 = ((ks * 2 + fr_grp) ^ fr_swz) * 16;
-        v8bf fa[TT], fb[2];
+        using frag_t = std::conditional_t<F16, v8h, v8bf>;
+        frag_t fa[TT], fb[2];
 #pragma unroll
         for (int tt = 0; tt < TT; ++tt) {
           if (!FULL && tt >= n_tt) continue;
-          fa[tt] = *reinterpret_cast<const v8bf*>(sa + tt * 32 * BK + c0);
+          fa[tt] = *reinterpret_cast<const frag_t*>(sa + tt * 32 * BK + c0);
         }
         if (!FULL && n_tt == 0) continue;
 #pragma unroll
         for (int ft = 0; ft < 2; ++ft)
-          fb[ft] = *reinterpret_cast<const v8bf*>(sb + ft * 128 * BK + c0);
+          fb[ft] = *reinterpret_cast<const frag_t*>(sb + ft * 128 * BK + c0);
 #pragma unroll
         for (int ft = 0; ft < 2; ++ft)
 #pragma unroll
           for (int tt = 0; tt < TT; ++tt) {
             if (!FULL && tt >= n_tt) continue;
-            acc[ft][tt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[ft], fa[tt], acc[ft][tt], 0, 0, 0);
+            if constexpr (F16) acc[ft][tt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[ft], fa[tt], acc[ft][tt], 0, 0, 0);
+            else acc[ft][tt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[ft], fa[tt], acc[ft][tt], 0, 0, 0);
           }
       }
     }
@@ -714,20 +722,20 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
 #pragma unroll
                   for (int i = 0; i < 4; ++i) v[i] = v[i] * sc;
                 }
-                v[0] = v[0] + __uint_as_float(bq.x << 16);
-                v[1] = v[1] + __uint_as_float(bq.x & 0xffff0000u);
-                v[2] = v[2] + __uint_as_float(bq.y << 16);
-                v[3] = v[3] + __uint_as_float(bq.y & 0xffff0000u);
+                v[0] = v[0] + Act::lo(bq.x);
+                v[1] = v[1] + Act::hi(bq.x);
+                v[2] = v[2] + Act::lo(bq.y);
+                v[3] = v[3] + Act::hi(bq.y);
               }
               if (gg.act == 1) {
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                  const float h = hdmoe_dev_round_bf16(v[i]);
+                  const float h = Act::round(v[i]);
                   v[i] = 0.5f * h * (1.0f + erff(h * 0.70710678118654752440f));
                 }
               }
-              pk.x = hdmoe_dev_pack_bf16(v[0], v[1]);
-              pk.y = hdmoe_dev_pack_bf16(v[2], v[3]);
+              pk.x = Act::pack(v[0], v[1]);
+              pk.y = Act::pack(v[2], v[3]);
             } else {
               pk.x = hdmoe_dev_pack_bf16(acc[ft][tt][q * 4 + 0] * sc, acc[ft][tt][q * 4 + 1] * sc);
               pk.y = hdmoe_dev_pack_bf16(acc[ft][tt][q * 4 + 2] * sc, acc[ft][tt][q * 4 + 3] * sc);
@@ -1116,7 +1124,7 @@ int hdmoe_down_parts(int rows_dyn, int n_dyn, int rows_static, int N, int K_dyn,
 int hdmoe_launch_linear_groups(const uint8_t* a_dyn, const int32_t* offsets, int rows_dyn, int n_dyn,
                                const hdmoe_linear_weights* experts, uint8_t* out_dyn, const uint8_t* a_static,
                                int rows_static, const hdmoe_linear_weights* shared, uint8_t* out_static, int K, int N,
-                               int act, hipStream_t s, const char* what) {
+                               int act, hipStream_t s, const char* what, bool f16 = false) {
   GemmArgs args;
   memset(&args, 0, sizeof(args));
   args.nparts = 1;
@@ -1153,7 +1161,8 @@ int hdmoe_launch_linear_groups(const uint8_t* a_dyn, const int32_t* offsets, int
     ++G;
   }
   args.G = G;
-  return launch_grouped<BF16_PLAIN_BIAS>(args, tile_bound, s, what);
+  return f16 ? launch_grouped<F16_PLAIN_BIAS>(args, tile_bound, s, what)
+             : launch_grouped<BF16_PLAIN_BIAS>(args, tile_bound, s, what);
 }
 
 // One Linear with an optional bias over all rows of `a` (either weight type): a single static group.
@@ -1178,6 +1187,7 @@ int hdmoe_launch_linear_bias(int weight_dtype, const uint8_t* a, int rows, int K
   gg.act = HDMOE_ACT_NONE;
   args.G = 1;
   const int tile_bound = ((rows + TileCfg<4>::BM - 1) / TileCfg<4>::BM) * (N / BN);
+  if (weight_dtype == HDMOE_W_F16) return launch_grouped<F16_PLAIN_BIAS>(args, tile_bound, s, what);
   return fp8 ? launch_grouped<FP8_PLAIN_BIAS>(args, tile_bound, s, what)
              : launch_grouped<BF16_PLAIN_BIAS>(args, tile_bound, s, what);
 }
@@ -1248,12 +1258,14 @@ extern "C" int hdmoe_linear(int weight_dtype, const void* a, int rows, int K, in
 extern "C" int hdmoe_linear_bias(int weight_dtype, const void* a, int rows, int K, int N, const void* w,
                                  const float* scale_w_dev, const float* scale_in_dev, const void* bias_bf16,
                                  void* out_bf16, hdmoe_stream_t stream) {
-  if (bias_bf16 == nullptr)
+  if (bias_bf16 == nullptr && weight_dtype != HDMOE_W_F16)
     return hdmoe_linear(weight_dtype, a, rows, K, N, w, scale_w_dev, scale_in_dev, out_bf16, stream);
   HDMOE_REQUIRE_PTR(a);
   HDMOE_REQUIRE_PTR(w);
   HDMOE_REQUIRE_PTR(out_bf16);
-  if (int rc = hdmoe_check_gemm_shape("hdmoe_linear_bias", weight_dtype, rows, K, N, BN)) return rc;
+  if (int rc = hdmoe_check_gemm_shape("hdmoe_linear_bias", weight_dtype == HDMOE_W_F16 ? HDMOE_W_BF16 : weight_dtype,
+                                      rows, K, N, BN))
+    return rc;
   if (weight_dtype == HDMOE_W_E4M3FN) HDMOE_REQUIRE_PTR(scale_w_dev);
   if (rows == 0) return HDMOE_OK;
   return hdmoe_launch_linear_bias(weight_dtype, static_cast<const uint8_t*>(a), rows, K, N,
@@ -1262,12 +1274,13 @@ extern "C" int hdmoe_linear_bias(int weight_dtype, const void* a, int rows, int 
                                   static_cast<hipStream_t>(stream), "hdmoe_linear_bias");
 }
 
-extern "C" int hdmoe_grouped_linear(const void* a_bf16, const int32_t* offsets, int rows_total, int E,
-                                    const hdmoe_linear_weights* experts, void* out_bf16, const void* a_static_bf16,
-                                    int rows_static, const hdmoe_linear_weights* shared, void* out_static_bf16, int K,
-                                    int N, int act, hdmoe_stream_t stream) {
-  if (E < 0 || E > HDMOE_MAX_EXPERTS) return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_grouped_linear: E=%d", E);
-  if (act != HDMOE_ACT_NONE && act != HDMOE_ACT_GELU) return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_grouped_linear: act=%d", act);
+namespace {
+int grouped_linear_entry(const char* what, bool f16, const void* a_bf16, const int32_t* offsets, int rows_total, int E,
+                         const hdmoe_linear_weights* experts, void* out_bf16, const void* a_static_bf16,
+                         int rows_static, const hdmoe_linear_weights* shared, void* out_static_bf16, int K, int N, int act,
+                         hdmoe_stream_t stream) {
+  if (E < 0 || E > HDMOE_MAX_EXPERTS) return hdmoe_fail(HDMOE_E_SHAPE, "%s: E=%d", what, E);
+  if (act != HDMOE_ACT_NONE && act != HDMOE_ACT_GELU) return hdmoe_fail(HDMOE_E_SHAPE, "%s: act=%d", what, act);
   if (E > 0) {
     HDMOE_REQUIRE_PTR(a_bf16);
     HDMOE_REQUIRE_PTR(offsets);
@@ -1279,12 +1292,29 @@ extern "C" int hdmoe_grouped_linear(const void* a_bf16, const int32_t* offsets, 
     HDMOE_REQUIRE_PTR(shared);
     HDMOE_REQUIRE_PTR(out_static_bf16);
   }
-  if (rows_static < 0) return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_grouped_linear: rows_static=%d", rows_static);
+  if (rows_static < 0) return hdmoe_fail(HDMOE_E_SHAPE, "%s: rows_static=%d", what, rows_static);
   const long rows_max = rows_total > rows_static ? rows_total : rows_static;
-  if (int rc = hdmoe_check_gemm_shape("hdmoe_grouped_linear", HDMOE_W_BF16, rows_max, K, N, BN)) return rc;
+  if (int rc = hdmoe_check_gemm_shape(what, HDMOE_W_BF16, rows_max, K, N, BN)) return rc;  // same sizes for fp16
   if ((E == 0 || rows_total == 0) && rows_static == 0) return HDMOE_OK;
   return hdmoe_launch_linear_groups(static_cast<const uint8_t*>(a_bf16), offsets, rows_total, rows_total > 0 ? E : 0,
                                     experts, static_cast<uint8_t*>(out_bf16), static_cast<const uint8_t*>(a_static_bf16),
                                     rows_static, shared, static_cast<uint8_t*>(out_static_bf16), K, N, act,
-                                    static_cast<hipStream_t>(stream), "hdmoe_grouped_linear");
+                                    static_cast<hipStream_t>(stream), what, f16);
+}
+}  // namespace
+
+extern "C" int hdmoe_grouped_linear(const void* a_bf16, const int32_t* offsets, int rows_total, int E,
+                                    const hdmoe_linear_weights* experts, void* out_bf16, const void* a_static_bf16,
+                                    int rows_static, const hdmoe_linear_weights* shared, void* out_static_bf16, int K,
+                                    int N, int act, hdmoe_stream_t stream) {
+  return grouped_linear_entry("hdmoe_grouped_linear", false, a_bf16, offsets, rows_total, E, experts, out_bf16,
+                              a_static_bf16, rows_static, shared, out_static_bf16, K, N, act, stream);
+}
+
+extern "C" int hdmoe_grouped_linear_f16(const void* a_f16, const int32_t* offsets, int rows_total, int E,
+                                        const hdmoe_linear_weights* experts, void* out_f16, const void* a_static_f16,
+                                        int rows_static, const hdmoe_linear_weights* shared, void* out_static_f16,
+                                        int K, int N, int act, hdmoe_stream_t stream) {
+  return grouped_linear_entry("hdmoe_grouped_linear_f16", true, a_f16, offsets, rows_total, E, experts, out_f16,
+                              a_static_f16, rows_static, shared, out_static_f16, K, N, act, stream);
 }

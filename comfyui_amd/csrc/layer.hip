@@ -28,7 +28,7 @@ int hdmoe_launch_dispatch_scatter(const int32_t* topk_idx, int T, int E, int32_t
 bool hdmoe_gate_quant_takes_ln(int D, int E);
 int hdmoe_launch_combine(const void* y_sorted_bf16, const int32_t* inv_perm, const void* topk_weight_bf16,
                          const void* shared_bf16, const void* gate_bf16, const void* residual_bf16, int tokens_per_batch,
-                         int T, int D, void* out_bf16, hipStream_t s, const char* what);
+                         int T, int D, void* out_bf16, hipStream_t s, const char* what, bool f16 = false);
 
 char* hdmoe_error_buffer() {
   static thread_local char buf[HDMOE_ERRBUF] = {0};

@@ -100,6 +100,30 @@ __device__ __forceinline__ float hdmoe_dev_round_bf16(float f) {
   return __uint_as_float(hdmoe_dev_pack_bf16(f, 0.0f) << 16);
 }
 
+// ---- the two 16-bit activation formats as one interface ------------------------------------------------
+// A kernel templated on the format reads packed pairs with lo()/hi(), rounds an fp32 value to the format with
+// round() and packs two with pack(); all conversions round to nearest even (v_cvt_f16_f32 follows the wave's
+// rounding mode, which no kernel here changes from the default). fp16 overflows to infinity and keeps its
+// subnormals, as torch's conversion does.
+typedef _Float16 hdmoe_f16x2 __attribute__((ext_vector_type(2)));
+
+struct HdmoeBf16 {
+  static __device__ __forceinline__ float lo(uint32_t u) { return __uint_as_float(u << 16); }
+  static __device__ __forceinline__ float hi(uint32_t u) { return __uint_as_float(u & 0xffff0000u); }
+  static __device__ __forceinline__ uint32_t pack(float a, float b) { return hdmoe_dev_pack_bf16(a, b); }
+  static __device__ __forceinline__ float round(float f) { return hdmoe_dev_round_bf16(f); }
+};
+
+struct HdmoeF16 {
+  static __device__ __forceinline__ float lo(uint32_t u) { return (float)(*reinterpret_cast<hdmoe_f16x2*>(&u))[0]; }
+  static __device__ __forceinline__ float hi(uint32_t u) { return (float)(*reinterpret_cast<hdmoe_f16x2*>(&u))[1]; }
+  static __device__ __forceinline__ uint32_t pack(float a, float b) {
+    hdmoe_f16x2 h = {(_Float16)a, (_Float16)b};
+    return *reinterpret_cast<uint32_t*>(&h);
+  }
+  static __device__ __forceinline__ float round(float f) { return (float)(_Float16)f; }
+};
+
 // e4m3fn conversion with the no-saturation rule (beyond the rounding midpoint above 448 -> NaN, 0x7F):
 // v_cvt_pk_fp8_f32 follows it when the FP16_OVFL bit of the wave's MODE register is clear and saturates to 448
 // when it is set. A wave starts with the bit its kernel descriptor holds (.amdhsa_fp16_overflow), which is 0 for

@@ -11,6 +11,15 @@ from ._lib import FfnWeights, LayerArgs, LayerLayout, LinearWeights, W_BF16, W_E
 
 FP8 = torch.float8_e4m3fn
 BF16 = torch.bfloat16
+F16 = torch.float16
+ACT_DTYPES = (BF16, F16)   # 16-bit activation formats; fp16 is served by the *_f16 entry points (Hunyuan3D block)
+
+
+def _act_dtype(t, what):
+    """The tensor's dtype if it is one of the two 16-bit activation formats."""
+    if t.dtype not in ACT_DTYPES:
+        raise TypeError(f"{what}: expected bfloat16 or float16, got {t.dtype}")
+    return t.dtype
 
 
 def _stream(t):
@@ -32,21 +41,25 @@ def weight_dtype_code(dtype):
         return W_BF16
     if dtype == FP8:
         return W_E4M3FN
+    if dtype == F16:
+        return _lib.W_F16      # hdmoe_linear_bias only
     raise TypeError(f"unsupported weight dtype {dtype}: the HIP path takes bfloat16 or float8_e4m3fn weights")
 
 
 def gate_top2(x2d, gate_w):
-    """MoEGate scoring + top-2 on the device. x2d [T,D] bf16, gate_w [E,D] bf16
-    -> topk_idx int32 [T,2], topk_weight bf16 [T,2]."""
-    _need_hip(x2d, "gate_top2 x", BF16)
-    _need_hip(gate_w, "gate_top2 gate weight", BF16)
+    """MoEGate scoring + top-2 on the device. x2d [T,D] bf16 (or fp16), gate_w [E,D] of the same dtype
+    -> topk_idx int32 [T,2], topk_weight [T,2] of that dtype."""
+    dt = _act_dtype(x2d, "gate_top2 x")
+    _need_hip(x2d, "gate_top2 x", dt)
+    _need_hip(gate_w, "gate_top2 gate weight", dt)
     T, D = x2d.shape
     E = gate_w.shape[0]
     if gate_w.shape[1] != D:
         raise ValueError(f"gate weight {tuple(gate_w.shape)} does not match hidden size {D}")
     idx = torch.empty((T, 2), dtype=torch.int32, device=x2d.device)
-    w = torch.empty((T, 2), dtype=BF16, device=x2d.device)
-    check(lib.hdmoe_gate_top2(ptr(x2d), ptr(gate_w), T, D, E, ptr(idx), ptr(w), _stream(x2d)))
+    w = torch.empty((T, 2), dtype=dt, device=x2d.device)
+    fn = lib.hdmoe_gate_top2 if dt == BF16 else lib.hdmoe_gate_top2_f16
+    check(fn(ptr(x2d), ptr(gate_w), T, D, E, ptr(idx), ptr(w), _stream(x2d)))
     return idx, w
 
 
@@ -109,16 +122,18 @@ def quant_permute_fp8(x2d, perm, offsets, scale_inputs):
 
 
 def permute_bf16(x2d, perm):
-    _need_hip(x2d, "permute_bf16 x", BF16)
+    """a[r] = x[perm[r] / 2]; rows are copied as bytes, so fp16 rows go through the same kernel."""
+    dt = _act_dtype(x2d, "permute_bf16 x")
+    _need_hip(x2d, "permute_bf16 x", dt)
     T, D = x2d.shape
-    out = torch.empty((2 * T, D), dtype=BF16, device=x2d.device)
+    out = torch.empty((2 * T, D), dtype=dt, device=x2d.device)
     check(lib.hdmoe_permute_bf16(ptr(x2d), ptr(perm), T, D, ptr(out), _stream(x2d)))
     return out
 
 
 def linear(a2d, weight, scale_weight=None, scale_input=None, bias=None):
-    """a2d [rows,K] (fp8 for fp8 weights, bf16 for bf16 weights) x weight [N,K]^T (+ bias [N] bf16) -> bf16 [rows,N];
-    the bias joins the fp32 result before the one rounding."""
+    """a2d [rows,K] (fp8 for fp8 weights, bf16 for bf16 weights, fp16 for fp16 weights) x weight [N,K]^T (+ bias [N])
+    -> [rows,N] bf16 (fp16 for fp16 weights); the bias joins the fp32 result before the one rounding."""
     code = weight_dtype_code(weight.dtype)
     _need_hip(a2d, "linear activations", weight.dtype)
     _need_hip(weight, "linear weight")
@@ -126,11 +141,12 @@ def linear(a2d, weight, scale_weight=None, scale_input=None, bias=None):
     N = weight.shape[0]
     if weight.shape[1] != K:
         raise ValueError(f"linear: activations [{rows},{K}] do not match weight {tuple(weight.shape)}")
+    out_dtype = F16 if weight.dtype == F16 else BF16
     if bias is not None:
-        _need_hip(bias, "linear bias", BF16)
+        _need_hip(bias, "linear bias", out_dtype)
         if bias.shape != (N,) or not bias.is_contiguous():
             raise ValueError(f"linear: bias {tuple(bias.shape)} does not match {N} output features")
-    out = torch.empty((rows, N), dtype=BF16, device=a2d.device)
+    out = torch.empty((rows, N), dtype=out_dtype, device=a2d.device)
     check(lib.hdmoe_linear_bias(code, ptr(a2d), rows, K, N, ptr(weight),
                                 _scale_ptr(scale_weight, a2d.device, "scale_weight"),
                                 _scale_ptr(scale_input, a2d.device, "scale_input"), ptr(bias), ptr(out), _stream(a2d)))
@@ -148,12 +164,12 @@ def silu_mul(a, b):
 
 
 def gelu(x):
-    """F.gelu (erf form) of a contiguous bf16 tensor."""
-    _need_hip(x, "gelu x", BF16)
-    if not x.is_contiguous():
-        raise ValueError("gelu: expected a contiguous tensor")
+    """F.gelu (erf form) of a contiguous bf16 or fp16 tensor."""
+    dt = _act_dtype(x, "gelu x")
+    _need_hip(x, "gelu x", dt)
     out = torch.empty_like(x)
-    check(lib.hdmoe_gelu_bf16(ptr(x), x.numel(), ptr(out), _stream(x)))
+    fn = lib.hdmoe_gelu_bf16 if dt == BF16 else lib.hdmoe_gelu_f16
+    check(fn(ptr(x), x.numel(), ptr(out), _stream(x)))
     return out
 
 
@@ -168,24 +184,27 @@ def scale_to_bf16(src, scale):
 
 
 def combine(y_sorted, inv_perm, topk_weight, shared):
-    _need_hip(y_sorted, "combine y", BF16)
-    _need_hip(topk_weight, "combine topk_weight", BF16)
+    dt = _act_dtype(y_sorted, "combine y")
+    _need_hip(y_sorted, "combine y", dt)
+    _need_hip(topk_weight, "combine topk_weight", dt)
+    if shared is not None:
+        _need_hip(shared, "combine shared", dt)
     T = topk_weight.shape[0]
     D = y_sorted.shape[1]
-    out = torch.empty((T, D), dtype=BF16, device=y_sorted.device)
-    check(lib.hdmoe_combine(ptr(y_sorted), ptr(inv_perm), ptr(topk_weight), ptr(shared), T, D, ptr(out),
-                            _stream(y_sorted)))
+    out = torch.empty((T, D), dtype=dt, device=y_sorted.device)
+    fn = lib.hdmoe_combine if dt == BF16 else lib.hdmoe_combine_f16
+    check(fn(ptr(y_sorted), ptr(inv_perm), ptr(topk_weight), ptr(shared), T, D, ptr(out), _stream(y_sorted)))
     return out
 
 
-def _linear_weights(weight, bias, K, N, what):
-    _need_hip(weight, f"{what} weight", BF16)
+def _linear_weights(weight, bias, K, N, what, dtype=BF16):
+    _need_hip(weight, f"{what} weight", dtype)
     if tuple(weight.shape) != (N, K):
         raise ValueError(f"{what}: weight shape {tuple(weight.shape)} != ({N}, {K})")
     lw = LinearWeights()
     lw.weight = ptr(weight)
     if bias is not None:
-        _need_hip(bias, f"{what} bias", BF16)
+        _need_hip(bias, f"{what} bias", dtype)
         if tuple(bias.shape) != (N,):
             raise ValueError(f"{what}: bias shape {tuple(bias.shape)} != ({N},)")
         lw.bias = ptr(bias)
@@ -197,20 +216,22 @@ def grouped_linear(a_sorted, offsets, experts, a_static=None, shared=None, act="
     one more (weight, bias) over all rows of `a_static`, in one launch. experts: list of (weight [N,K], bias [N] or
     None). Returns (out_sorted [rows, N], out_static [rows_static, N] or None)."""
     code = {"none": _lib.ACT_NONE, "gelu": _lib.ACT_GELU}[act]
-    _need_hip(a_sorted, "grouped_linear a", BF16)
+    dt = _act_dtype(a_sorted, "grouped_linear a")   # bf16, or fp16 throughout
+    _need_hip(a_sorted, "grouped_linear a", dt)
     rows, K = a_sorted.shape
     N = experts[0][0].shape[0] if experts else shared[0].shape[0]
     E = len(experts)
-    arr = (LinearWeights * max(E, 1))(*[_linear_weights(w, b, K, N, f"grouped_linear expert {i}")
+    arr = (LinearWeights * max(E, 1))(*[_linear_weights(w, b, K, N, f"grouped_linear expert {i}", dt)
                                         for i, (w, b) in enumerate(experts)])
-    out = torch.empty((rows, N), dtype=BF16, device=a_sorted.device)
+    out = torch.empty((rows, N), dtype=dt, device=a_sorted.device)
     out_static, sh, rows_static = None, None, 0
     if shared is not None:
-        _need_hip(a_static, "grouped_linear a_static", BF16)
+        _need_hip(a_static, "grouped_linear a_static", dt)
         rows_static = a_static.shape[0]
-        sh = _linear_weights(shared[0], shared[1], K, N, "grouped_linear shared")
-        out_static = torch.empty((rows_static, N), dtype=BF16, device=a_sorted.device)
-    check(lib.hdmoe_grouped_linear(ptr(a_sorted), ptr(offsets), rows, E, arr, ptr(out), ptr(a_static), rows_static,
+        sh = _linear_weights(shared[0], shared[1], K, N, "grouped_linear shared", dt)
+        out_static = torch.empty((rows_static, N), dtype=dt, device=a_sorted.device)
+    fn = lib.hdmoe_grouped_linear if dt == BF16 else lib.hdmoe_grouped_linear_f16
+    check(fn(ptr(a_sorted), ptr(offsets), rows, E, arr, ptr(out), ptr(a_static), rows_static,
                                    ctypes.byref(sh) if sh is not None else None, ptr(out_static), K, N, code,
                                    _stream(a_sorted)))
     return out, out_static

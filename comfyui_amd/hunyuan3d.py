@@ -10,11 +10,13 @@ and erf-GELU epilogue for the experts.
 
 Inference only (the reference's training branch and auxiliary loss are not part of this path). A token meets at
 most two experts, so the index_add_ accumulation bf16(bf16(w_a y_a) + bf16(w_b y_b)) is the same two-term sum the
-HiDream combine forms. Inputs must be bf16 HIP tensors: there is no CPU path.
+HiDream combine forms. Inputs must be bf16 or fp16 HIP tensors (fp16 is what model_management.unet_dtype picks for
+this model family on a device with fp16 support, supported_models_base.py:46): there is no CPU path. With fp16
+every tensor and every rounding point of the block is fp16; scaled-fp8 Linears take bf16 activations only.
 
 Two ways through the experts:
-  * every Linear a plain bf16 one resident on the device (no weight function, no scale_weight): two grouped launches
-    for all experts and the shared expert;
+  * every Linear a plain one of the activation dtype resident on the device (no weight function, no scale_weight):
+    two grouped launches for all experts and the shared expert;
   * anything else the `operations` argument brings (scaled-fp8 Linears with or without the fp8 matrix multiply,
     manual-cast or offloaded weights, weight functions): one expert at a time through the Linear modules' own
     forward, the GELU as an elementwise kernel, with the same gate, dispatch and combine kernels around them.
@@ -26,6 +28,7 @@ from . import functional as HF
 from . import ops as amd_ops
 
 BF16 = torch.bfloat16
+ACT_DTYPES = HF.ACT_DTYPES
 
 
 class _LinearWithBias(amd_ops.disable_weight_init.Linear):
@@ -33,8 +36,9 @@ class _LinearWithBias(amd_ops.disable_weight_init.Linear):
     grouped kernel with a single group."""
 
     def forward(self, x):
-        if not (x.is_cuda and x.dtype == BF16 and self.weight.dtype == BF16):
-            raise RuntimeError("comfyui_amd.hunyuan3d: expected bfloat16 HIP tensors and weights; there is no CPU path")
+        if not (x.is_cuda and x.dtype in ACT_DTYPES and self.weight.dtype == x.dtype):
+            raise RuntimeError("comfyui_amd.hunyuan3d: expected bfloat16 or float16 HIP tensors and weights of the same "
+                               "dtype; there is no CPU path")
         x2 = x.reshape(-1, x.shape[-1]).contiguous()
         _, y = HF.grouped_linear(x2[:0], None, [], a_static=x2, shared=(self.weight, self.bias), act="none")
         return y.view(*x.shape[:-1], self.weight.shape[0])
@@ -59,21 +63,21 @@ class GELU(nn.Module):
 
 
 def _need(x):
-    if not (x.is_cuda and x.dtype == BF16):
-        raise RuntimeError(f"comfyui_amd.hunyuan3d: expected bfloat16 HIP activations, got {x.dtype} on {x.device}; "
-                           "there is no CPU path")
+    if not (x.is_cuda and x.dtype in ACT_DTYPES):
+        raise RuntimeError(f"comfyui_amd.hunyuan3d: expected bfloat16 or float16 HIP activations, got {x.dtype} on "
+                           f"{x.device}; there is no CPU path")
 
 
 def _plain_bf16(lin, x):
-    """True when `lin` can join a grouped launch as it stands: bf16 weight (and bias) on x's device, nothing to
-    apply to them first."""
+    """True when `lin` can join a grouped launch as it stands: weight (and bias) of x's dtype (bf16 or fp16) on x's
+    device, nothing to apply to them first."""
     if getattr(lin, "weight_function", None) or getattr(lin, "bias_function", None):
         return False
     if getattr(lin, "scale_weight", None) is not None:
         return False
-    if lin.weight.dtype != BF16 or lin.weight.device != x.device:
+    if lin.weight.dtype != x.dtype or lin.weight.device != x.device:
         return False
-    return lin.bias is None or (lin.bias.dtype == BF16 and lin.bias.device == x.device)
+    return lin.bias is None or (lin.bias.dtype == x.dtype and lin.bias.device == x.device)
 
 
 class FeedForward(nn.Module):

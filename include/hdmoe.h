@@ -42,7 +42,7 @@
 extern "C" {
 #endif
 
-#define HDMOE_VERSION 111
+#define HDMOE_VERSION 112
 
 #define HDMOE_OK 0
 #define HDMOE_E_NULL (-1)      /* required pointer is NULL */
@@ -56,6 +56,8 @@ extern "C" {
 /* weight storage of the Linear layers */
 #define HDMOE_W_BF16 0
 #define HDMOE_W_E4M3FN 1
+/* fp16 weights with fp16 activations, bias and outputs: hdmoe_linear_bias only (and the *_f16 entry points below) */
+#define HDMOE_W_F16 2
 
 typedef void* hdmoe_stream_t;
 
@@ -72,6 +74,12 @@ const char* hdmoe_last_error(void);
  * D % 8 == 0, 2 <= E <= 16. The same gate serves comfy/ldm/hunyuan3dv2_1/hunyuandit.py:73-112 (E = 6 or 8). */
 int hdmoe_gate_top2(const void* x_bf16, const void* gate_w_bf16, int T, int D, int E,
                     int32_t* topk_idx, void* topk_weight_bf16, hdmoe_stream_t stream);
+
+/* The same gate on fp16 tensors (x, gate_w, topk_weight fp16; logits and scores rounded to fp16 between the steps):
+ * the dtype comfy/supported_models_base.py:46 lists first and model_management.unet_dtype picks for
+ * comfy/ldm/hunyuan3dv2_1/hunyuandit.py:73-112 on a device with fp16 support. */
+int hdmoe_gate_top2_f16(const void* x_f16, const void* gate_w_f16, int T, int D, int E,
+                        int32_t* topk_idx, void* topk_weight_f16, hdmoe_stream_t stream);
 
 /* Optional renormalisation of the two gate weights, comfy/ldm/hidream/model.py:277-280 (`norm_topk_prob`, off in
  * HiDream): out[t, s] = bf16( w[t, s] / bf16( bf16(w[t,0] + w[t,1]) + 1e-20 ) ), the rounding points of the three torch
@@ -116,7 +124,8 @@ int hdmoe_quant_permute_fp8(const void* x_bf16, const int32_t* perm, const int32
                             int T, int D, int E, const float* const* scale_input,
                             void* a_fp8, hdmoe_stream_t stream);
 
-/* bf16 gather of model.py:315,318 for bf16 weights: a[r] = x[perm[r] / 2]. */
+/* bf16 gather of model.py:315,318 for bf16 weights: a[r] = x[perm[r] / 2]. Rows are copied as bytes, so any 16-bit
+ * element type (fp16) goes through it unchanged. */
 int hdmoe_permute_bf16(const void* x_bf16, const int32_t* perm, int T, int D, void* a_bf16,
                        hdmoe_stream_t stream);
 
@@ -170,7 +179,8 @@ int hdmoe_linear(int weight_dtype, const void* a, int rows, int K, int N, const 
  * rounding, as F.linear does (ops.py:107-115) and as the scaled matrix multiply of fp8_linear does with its bias
  * argument (ops.py:345-346):
  *   fp8:  out = bf16( (a_fp8 . w_fp8^T) * scale_in * scale_w + bias )
- *   bf16: out = bf16( a_bf16 . w_bf16^T + bias ) */
+ *   bf16: out = bf16( a_bf16 . w_bf16^T + bias )
+ *   fp16: out = fp16( a_f16 . w_f16^T + bias )      (HDMOE_W_F16; bias fp16 or NULL) */
 int hdmoe_linear_bias(int weight_dtype, const void* a, int rows, int K, int N, const void* w,
                       const float* scale_w_dev, const float* scale_in_dev, const void* bias_bf16,
                       void* out_bf16, hdmoe_stream_t stream);
@@ -182,6 +192,8 @@ int hdmoe_silu_mul_bf16(const void* a_bf16, const void* b_bf16, int64_t n, void*
 /* F.gelu (erf form) of a bf16 tensor for the unfused Hunyuan3D expert, comfy/ldm/hunyuan3dv2_1/hunyuandit.py:14-26
  * (`gelu(proj(x))` when proj is not the plain bf16 Linear): out = bf16(gelu(fp32(x))). n % 8 == 0. */
 int hdmoe_gelu_bf16(const void* x_bf16, int64_t n, void* out_bf16, hdmoe_stream_t stream);
+/* the same on an fp16 tensor: out = fp16(gelu(fp32(x))) */
+int hdmoe_gelu_f16(const void* x_f16, int64_t n, void* out_f16, hdmoe_stream_t stream);
 
 /* `weight * scale_weight` or `input * scale_weight` of the scaled-fp8 Linear WITHOUT fp8
  * matmul (comfy/ops.py:407-410), after the operand was cast to bf16:
@@ -195,6 +207,10 @@ int hdmoe_scale_to_bf16(int src_dtype, const void* src, int64_t n, const float* 
  * Deterministic (a gather, no atomics). D % 8 == 0. */
 int hdmoe_combine(const void* y_sorted_bf16, const int32_t* inv_perm, const void* topk_weight_bf16,
                   const void* shared_bf16, int T, int D, void* out_bf16, hdmoe_stream_t stream);
+/* The same combine with every tensor and every rounding in fp16: the weighted index_add_ in expert order plus the shared
+ * expert of comfy/ldm/hunyuan3dv2_1/hunyuandit.py:176-187 at that dtype (a token meets at most two experts). */
+int hdmoe_combine_f16(const void* y_sorted_f16, const int32_t* inv_perm, const void* topk_weight_f16,
+                      const void* shared_f16, int T, int D, void* out_f16, hdmoe_stream_t stream);
 
 /* Linear with bias (and optional erf GELU) over the expert row segments of a dispatched batch, plus optionally one
  * more group over all rows of another input (a shared expert), in one launch: the two stages of the GELU
@@ -211,6 +227,12 @@ int hdmoe_grouped_linear(const void* a_bf16, const int32_t* offsets, int rows_to
                          const hdmoe_linear_weights* experts, void* out_bf16, const void* a_static_bf16,
                          int rows_static, const hdmoe_linear_weights* shared, void* out_static_bf16, int K, int N,
                          int act, hdmoe_stream_t stream);
+/* The same with fp16 activations, weights, biases and outputs (fp32 accumulation, one rounding to fp16 after the
+ * bias, GELU of the rounded value rounded again). */
+int hdmoe_grouped_linear_f16(const void* a_f16, const int32_t* offsets, int rows_total, int E,
+                             const hdmoe_linear_weights* experts, void* out_f16, const void* a_static_f16,
+                             int rows_static, const hdmoe_linear_weights* shared, void* out_static_f16, int K,
+                             int N, int act, hdmoe_stream_t stream);
 
 /* Weight maintenance of a scaled-fp8 Linear (comfy/ops.py:419-426 set_weight, comfy/float.py:14-67):
  * out[i] = stochastic_round_e4m3fn( float16( src[i] / *scale_dev ) ), scale_dev NULL = 1. Each value lands on one of

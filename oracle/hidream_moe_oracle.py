@@ -43,6 +43,9 @@ def _lib():
             raise RuntimeError(f"{path} missing: run `make -C oracle` (or __graft_entry__.build())")
         lib = ctypes.CDLL(path)
         lib.ref_gate_top2.restype = ctypes.c_int
+        lib.ref_gate_top2_f16.restype = ctypes.c_int
+        lib.ref_f16_decode.restype = None
+        lib.ref_f16_encode.restype = None
         lib.ref_dispatch.restype = ctypes.c_int
         lib.ref_combine.restype = None
         lib.ref_ln_modulate.restype = ctypes.c_int
@@ -93,6 +96,22 @@ def quantize_weight_per_tensor(w_f32):
 
 # -------------------------------------------------------------------------- gate
 
+def f16_decode(bits_u16):
+    """fp16 bit patterns (int16/uint16 tensor) -> fp32 by the format's definition (moe_ref.c f16_to_f32)."""
+    src = bits_u16.contiguous()
+    out = torch.empty(src.shape, dtype=torch.float32)
+    _lib().ref_f16_decode(_p(src), _p(out), ctypes.c_int64(src.numel()))
+    return out
+
+
+def f16_encode(values_f32):
+    """fp32 -> fp16 bit patterns (int16), round to nearest even, overflow to infinity (moe_ref.c f32_to_f16)."""
+    src = values_f32.float().contiguous()
+    out = torch.empty(src.shape, dtype=torch.int16)
+    _lib().ref_f16_encode(_p(src), _p(out), ctypes.c_int64(src.numel()))
+    return out
+
+
 def top2_lowest_index(scores):
     """First two columns of a stable descending sort: larger score first, ties -> lower index."""
     order = torch.sort(scores.float(), dim=-1, descending=True, stable=True).indices
@@ -112,17 +131,19 @@ def gate_torch(x2d, wg):
 def gate_fixed_order(x2d_bf16, wg_bf16):
     """Same computation with the one fixed fp32 summation order and exp() of moe_ref.c
     (what the HIP gate kernel is compared with bit for bit).
-    Returns idx int32 [T,2], weight bf16 [T,2], logits bf16 [T,E], scores bf16 [T,E]."""
+    Returns idx int32 [T,2], weight bf16 [T,2], logits bf16 [T,E], scores bf16 [T,E]. fp16 inputs: the same with
+    every tensor and the two roundings in fp16 (the Hunyuan3D block's other dtype)."""
     x = x2d_bf16.contiguous()
     wg = wg_bf16.contiguous()
-    assert x.dtype == torch.bfloat16 and wg.dtype == torch.bfloat16
+    assert x.dtype in (torch.bfloat16, torch.float16) and wg.dtype == x.dtype
     T, D = x.shape
     E = wg.shape[0]
     idx = torch.empty((T, 2), dtype=torch.int32)
-    w = torch.empty((T, 2), dtype=torch.bfloat16)
-    logits = torch.empty((T, E), dtype=torch.bfloat16)
-    scores = torch.empty((T, E), dtype=torch.bfloat16)
-    rc = _lib().ref_gate_top2(_p(x), _p(wg), T, D, E, _p(idx), _p(w), _p(logits), _p(scores))
+    w = torch.empty((T, 2), dtype=x.dtype)
+    logits = torch.empty((T, E), dtype=x.dtype)
+    scores = torch.empty((T, E), dtype=x.dtype)
+    fn = _lib().ref_gate_top2 if x.dtype == torch.bfloat16 else _lib().ref_gate_top2_f16
+    rc = fn(_p(x), _p(wg), T, D, E, _p(idx), _p(w), _p(logits), _p(scores))
     if rc != 0:
         raise ValueError("ref_gate_top2: bad arguments")
     return idx, w, logits, scores

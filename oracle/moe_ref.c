@@ -43,6 +43,40 @@ static uint16_t f32_to_bf16(float f) {
   return (uint16_t)keep;
 }
 
+/* IEEE binary16 <-> fp32 by the definition: 1 sign, 5 exponent (bias 15), 10 mantissa bits, subnormals m * 2^-24,
+ * exponent 31 = inf / NaN. Encode rounds to nearest even through ldexp/nearbyint arithmetic on the value (not bit
+ * tricks), overflows to infinity at 65520 and above. Pinned against torch's own conversion in the tests (all 65536
+ * patterns decoded, random and boundary values encoded). */
+static float f16_to_f32(uint16_t h) {
+  int s = h >> 15, e = (h >> 10) & 31, m = h & 1023;
+  float v;
+  if (e == 31) v = m ? NAN : INFINITY;
+  else if (e == 0) v = ldexpf((float)m, -24);
+  else v = ldexpf(1.0f + (float)m / 1024.0f, e - 15);
+  return s ? -v : v;
+}
+
+static uint16_t f32_to_f16(float f) {
+  uint16_t sign = (f32_bits(f) >> 31) ? 0x8000u : 0;
+  if (isnan(f)) return (uint16_t)(sign | 0x7e00u);
+  double a = fabs((double)f);
+  if (a >= 65520.0) return (uint16_t)(sign | 0x7c00u);          /* the midpoint above 65504 rounds to infinity */
+  if (a < ldexp(1.0, -14)) {                                    /* subnormal range: multiples of 2^-24 */
+    double q = nearbyint(ldexp(a, 24));                         /* default rounding mode: to nearest even */
+    return (uint16_t)(sign | (uint16_t)q);                      /* q == 1024 is the smallest normal, same bits */
+  }
+  int ex;
+  double fr = frexp(a, &ex);                                    /* a = fr * 2^ex, fr in [0.5, 1) */
+  double q = nearbyint(ldexp(fr, 11));                          /* 11 significant bits: 1024 .. 2048 */
+  if (q == 2048.0) { q = 1024.0; ex += 1; }
+  int e = ex - 1 + 15;
+  if (e >= 31) return (uint16_t)(sign | 0x7c00u);
+  return (uint16_t)(sign | (uint16_t)(e << 10) | (uint16_t)((int)q - 1024));
+}
+
+void ref_f16_decode(const uint16_t* in, float* out, int64_t n) { for (int64_t i = 0; i < n; ++i) out[i] = f16_to_f32(in[i]); }
+void ref_f16_encode(const float* in, uint16_t* out, int64_t n) { for (int64_t i = 0; i < n; ++i) out[i] = f32_to_f16(in[i]); }
+
 /* ---- float8_e4m3fn ---------------------------------------------------------- */
 
 /* closed form: (-1)^s * 2^(e-7) * (1 + m/8), e==0 -> m * 2^-9, 0x7F/0xFF NaN */
@@ -106,12 +140,14 @@ static float ref_exp_neg(float x) {
 /* x [T,D] bf16, wg [E,D] bf16 -> idx [T,2] int32 (slot 0 = larger score, ties to
  * the lower expert index), w [T,2] bf16 scores, optional logits/scores [T,E] bf16.
  * D must be a multiple of 8, 2 <= E <= 16. Returns 0, or -1 on bad arguments. */
-int ref_gate_top2(const uint16_t* x, const uint16_t* wg, int T, int D, int E,
-                  int32_t* idx, uint16_t* w, uint16_t* logits_out, uint16_t* scores_out) {
+static int gate_top2_fmt(const uint16_t* x, const uint16_t* wg, int T, int D, int E,
+                         int32_t* idx, uint16_t* w, uint16_t* logits_out, uint16_t* scores_out,
+                         float (*bf16_to_f32)(uint16_t), uint16_t (*f32_to_bf16)(float)) {
+  /* the two parameters shadow the bf16 conversions: the body below reads the same for either 16-bit format */
   if (D % 8 != 0 || E < 2 || E > 16 || T < 0) return -1;
   for (int t = 0; t < T; ++t) {
     const uint16_t* xr = x + (size_t)t * D;
-    float logit[16], score[16];
+    float logit[16] = {0}, score[16] = {0};
     for (int e = 0; e < E; ++e) {
       const uint16_t* wr = wg + (size_t)e * D;
       float lane[64];
@@ -141,6 +177,17 @@ int ref_gate_top2(const uint16_t* x, const uint16_t* wg, int T, int D, int E,
     if (scores_out) for (int e = 0; e < E; ++e) scores_out[(size_t)t * E + e] = f32_to_bf16(score[e]);
   }
   return 0;
+}
+
+int ref_gate_top2(const uint16_t* x, const uint16_t* wg, int T, int D, int E,
+                  int32_t* idx, uint16_t* w, uint16_t* logits_out, uint16_t* scores_out) {
+  return gate_top2_fmt(x, wg, T, D, E, idx, w, logits_out, scores_out, bf16_to_f32, f32_to_bf16);
+}
+
+/* the same gate on fp16 tensors: x, wg, w, logits and scores fp16, the two roundings to fp16 */
+int ref_gate_top2_f16(const uint16_t* x, const uint16_t* wg, int T, int D, int E,
+                      int32_t* idx, uint16_t* w, uint16_t* logits_out, uint16_t* scores_out) {
+  return gate_top2_fmt(x, wg, T, D, E, idx, w, logits_out, scores_out, f16_to_f32, f32_to_f16);
 }
 
 /* ---- dispatch --------------------------------------------------------------- */

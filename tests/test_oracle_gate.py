@@ -136,3 +136,76 @@ def test_renorm_topk_rounding_points_and_closed_forms():
     exact = w.double() / (w.double().sum(-1, keepdim=True) + 1e-20)
     ok = nz
     assert float(((r.double() - exact).abs()[ok] / exact[ok].clamp_min(1e-3)).max()) < 3 * 2.0 ** -8
+
+
+# ---- the same gate on fp16 tensors (the Hunyuan3D block's other dtype) ----------------------------------------
+
+F16 = torch.float16
+
+
+def test_f16_conversions_of_the_checker_equal_torch():
+    """The C checker's fp16 decode on all 65536 patterns and its encode on random values, every representable
+    value, every midpoint between neighbours (ties to even), the overflow boundary and the subnormal range, against
+    torch's own conversion."""
+    bits = torch.arange(65536, dtype=torch.int32).to(torch.int16)
+    dec = O.f16_decode(bits)
+    want = bits.view(F16).float()
+    nan = torch.isnan(want)
+    assert torch.equal(torch.isnan(dec), nan)
+    assert torch.equal(dec[~nan].view(torch.int32), want[~nan].view(torch.int32))      # incl. the sign of zero
+    g = torch.Generator().manual_seed(0)
+    finite = want[~nan & ~torch.isinf(want)]
+    pos = torch.sort(finite[finite >= 0]).values
+    mids = ((pos[:-1].double() + pos[1:].double()) / 2).float()                         # exact in fp32
+    vals = torch.cat([
+        torch.randn(200000, generator=g) * 10.0 ** torch.randint(-9, 6, (200000,), generator=g).float(),
+        finite, mids, -mids,
+        torch.tensor([65504.0, 65519.0, 65519.996, 65520.0, 65536.0, 1e9, float("inf"), -float("inf"), -65520.0,
+                      2.0 ** -24, 2.0 ** -25, 2.0 ** -25 * 1.0000001, 1.5 * 2.0 ** -24, 2.5 * 2.0 ** -24, 2.0 ** -14,
+                      0.0, -0.0, 1e-30]),
+    ])
+    enc = O.f16_encode(vals)
+    assert torch.equal(enc, vals.to(F16).view(torch.int16))
+    assert O.f16_encode(torch.tensor([float("nan")])).view(F16).isnan().all()
+
+
+def test_fixed_order_f16_vs_torch_and_fp64():
+    """fp16 gate: logits equal the fp16 rounding of the fp64 value except where that value sits on a rounding
+    midpoint to within what fp32 summation resolves; routing equal to torch's own fp16 kernels wherever logits and
+    scores agree bit for bit; small-integer inputs exact; ties to the lower index."""
+    T, D, E = 2048, 2048, 8
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn((T, D), generator=g).to(F16)
+    wg = (torch.randn((E, D), generator=g) / math.sqrt(D)).to(F16)
+    idx, w, logits, scores = O.gate_fixed_order(x, wg)
+    assert w.dtype == F16 and logits.dtype == F16
+    ti, tw, tl, ts = O.gate_torch(x, wg)
+    l64 = x.double() @ wg.double().t()
+    lo = l64.to(F16)
+    bits = lo.view(torch.int16).to(torch.int32)
+    up = (bits + 1).to(torch.int16).view(F16).double()
+    dn = (bits - 1).to(torch.int16).view(F16).double()
+    dist_to_mid = torch.minimum((l64 - (lo.double() + up) / 2).abs(), (l64 - (lo.double() + dn) / 2).abs())
+    sumabs = x.double().abs() @ wg.double().abs().t()
+    fragile = dist_to_mid <= sumabs * 2 ** -26             # observed <= 1e-8 of the sum of |terms|
+    assert float(fragile.float().mean()) < 2e-2            # fp16 has 8x finer steps than bf16: more midpoints nearby
+    bad = (logits.view(torch.int16) != lo.view(torch.int16)) & ~fragile
+    assert int(bad.sum()) == 0
+    tok_same = (logits.view(torch.int16) == tl.view(torch.int16)).all(dim=1) & \
+               (scores.view(torch.int16) == ts.view(torch.int16)).all(dim=1)
+    assert float(tok_same.float().mean()) > 0.9
+    assert torch.equal(idx[tok_same].long(), ti[tok_same])
+    assert torch.equal(w[tok_same].view(torch.int16), tw[tok_same].view(torch.int16))
+    sm = torch.softmax(logits.double(), dim=-1)
+    assert float((scores.double() - sm).abs().max()) <= 2 ** -12          # fp16 rounding of a value <= 1
+    assert torch.equal(w.view(torch.int16), torch.gather(scores, 1, idx.long()).view(torch.int16))
+    srt = torch.sort(scores.float(), dim=-1, descending=True, stable=True).indices[:, :2]
+    assert torch.equal(idx.long(), srt)
+    # small integers: exact whatever the order
+    xi = torch.randint(-3, 4, (100, 512), generator=g).float().to(F16)
+    wi = (torch.randint(-2, 3, (4, 512), generator=g).float() / 64).to(F16)
+    _, _, li, si = O.gate_fixed_order(xi, wi)
+    assert torch.equal(li.double(), (xi.double() @ wi.double().t()).to(F16).double())
+    # all-zero logits: scores 0.25 each, experts 0 and 1
+    i0, w0, _, s0 = O.gate_fixed_order(torch.zeros((2, 512), dtype=F16), torch.zeros((4, 512), dtype=F16))
+    assert i0.tolist() == [[0, 1], [0, 1]] and s0.float().tolist() == [[0.25] * 4] * 2
