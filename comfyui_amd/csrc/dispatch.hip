@@ -55,7 +55,7 @@ __global__ __launch_bounds__(THREADS) void dispatch_count_kernel(const int32_t* 
 
 template <int ITEMS>
 __global__ __launch_bounds__(THREADS) void dispatch_scatter_kernel(
-    const int32_t* __restrict__ flat, int n, int E, int nhist, int hist_per_chunk,
+    const int32_t* __restrict__ flat, int n, int E, int nhist, int hist_per_chunk, int chunk_slots,
     const int32_t* __restrict__ chunk_counts, int32_t* __restrict__ counts, int32_t* __restrict__ offsets,
     int32_t* __restrict__ perm, int32_t* __restrict__ inv_perm) {
   __shared__ int32_t total[HDMOE_MAX_EXPERTS];
@@ -92,12 +92,13 @@ __global__ __launch_bounds__(THREADS) void dispatch_scatter_kernel(
   }
   __syncthreads();
 
-  constexpr int CHUNK = THREADS * ITEMS;
-  const int base = blockIdx.x * CHUNK;
+  // a block's chunk: chunk_slots flat slots (at most THREADS * ITEMS; fewer when the histograms' granularity asks)
+  const int base = blockIdx.x * chunk_slots;
+  const int end = min(n, base + chunk_slots);
   const unsigned long long lt = (1ull << lane) - 1ull;
   for (int it = 0; it < ITEMS; ++it) {
     const int p = base + it * THREADS + threadIdx.x;
-    int e = p < n ? flat[p] : -1;
+    int e = p < end ? flat[p] : -1;
     if (e >= E) e = -1;  // never index the LDS tables with a bad id
     int32_t rank = 0;   // slots of my expert in lower lanes of my wave
     int32_t mine = 0;   // lane q holds the wave's count for expert q
@@ -147,37 +148,37 @@ int dispatch_enqueue(const char* what, const int32_t* topk_idx, int T, int E, in
   if (items == ITEMS_SMALL) {
     hipLaunchKernelGGL(dispatch_count_kernel<ITEMS_SMALL>, dim3(nchunks), dim3(THREADS), 0, s, topk_idx, n, E, cc);
     hipLaunchKernelGGL(dispatch_scatter_kernel<ITEMS_SMALL>, dim3(nchunks), dim3(THREADS), 0, s, topk_idx, n, E,
-                       nchunks, 1, cc, counts, offsets, perm, inv_perm);
+                       nchunks, 1, chunk, cc, counts, offsets, perm, inv_perm);
   } else {
     hipLaunchKernelGGL(dispatch_count_kernel<ITEMS_LARGE>, dim3(nchunks), dim3(THREADS), 0, s, topk_idx, n, E, cc);
     hipLaunchKernelGGL(dispatch_scatter_kernel<ITEMS_LARGE>, dim3(nchunks), dim3(THREADS), 0, s, topk_idx, n, E,
-                       nchunks, 1, cc, counts, offsets, perm, inv_perm);
+                       nchunks, 1, chunk, cc, counts, offsets, perm, inv_perm);
   }
   return hdmoe_check_launch(what);
 }
 
 // Second pass alone: the histograms come from the gate kernel, one per block of tokens_per_hist tokens
-// (hdmoe_gate_tokens_per_block: a power of two that divides a chunk's tokens).
+// (hdmoe_gate_tokens_per_block). A chunk is as many whole histograms as fit 128 tokens, or one histogram of up to
+// 1024 tokens.
 int dispatch_scatter_enqueue(const char* what, const int32_t* topk_idx, int T, int E, int32_t* counts,
                              int32_t* offsets, int32_t* perm, int32_t* inv_perm, const int32_t* block_hist,
                              int tokens_per_hist, hipStream_t s) {
   const int n = T * HDMOE_TOPK;
-  const int items = items_for((size_t)n);
-  const int chunk = THREADS * items;
-  const int chunk_tokens = chunk / HDMOE_TOPK;
-  if (tokens_per_hist < 1 || chunk_tokens % tokens_per_hist != 0)
-    return hdmoe_fail(HDMOE_E_SHAPE, "%s: histograms of %d tokens do not tile a chunk of %d", what, tokens_per_hist,
-                      chunk_tokens);
+  const int small_tokens = THREADS * ITEMS_SMALL / HDMOE_TOPK, large_tokens = THREADS * ITEMS_LARGE / HDMOE_TOPK;
+  if (tokens_per_hist < 1 || tokens_per_hist > large_tokens)
+    return hdmoe_fail(HDMOE_E_SHAPE, "%s: histograms of %d tokens (1 to %d)", what, tokens_per_hist, large_tokens);
+  const int per_chunk = tokens_per_hist <= small_tokens ? small_tokens / tokens_per_hist : 1;
+  const int chunk_tokens = per_chunk * tokens_per_hist;
+  const int chunk = chunk_tokens * HDMOE_TOPK;
   int nchunks = (n + chunk - 1) / chunk;
   if (nchunks < 1) nchunks = 1;
   const int nhist = T > 0 ? (T + tokens_per_hist - 1) / tokens_per_hist : 0;
-  const int per_chunk = chunk_tokens / tokens_per_hist;
-  if (items == ITEMS_SMALL)
+  if (chunk <= THREADS * ITEMS_SMALL)
     hipLaunchKernelGGL(dispatch_scatter_kernel<ITEMS_SMALL>, dim3(nchunks), dim3(THREADS), 0, s, topk_idx, n, E, nhist,
-                       per_chunk, block_hist, counts, offsets, perm, inv_perm);
+                       per_chunk, chunk, block_hist, counts, offsets, perm, inv_perm);
   else
     hipLaunchKernelGGL(dispatch_scatter_kernel<ITEMS_LARGE>, dim3(nchunks), dim3(THREADS), 0, s, topk_idx, n, E, nhist,
-                       per_chunk, block_hist, counts, offsets, perm, inv_perm);
+                       per_chunk, chunk, block_hist, counts, offsets, perm, inv_perm);
   return hdmoe_check_launch(what);
 }
 

@@ -494,13 +494,15 @@ extern "C" int hdmoe_gate_top2_f16(const void* x_f16, const void* gate_w_f16, in
                        static_cast<hipStream_t>(stream), "hdmoe_gate_top2_f16", true);
 }
 
-// Tokens per block of the gate kernels, a pure function of T: a power of two between WAVES_PER_BLOCK and 128 (so
-// that the dispatch's chunks of 128 or 1024 tokens are whole numbers of blocks), the smallest that keeps the grid
-// at about three blocks per CU (the register kernels' 12 waves per CU) and gives a block's copy of the gate weight
-// into LDS at least two tokens per wave to pay for.
+// Tokens per block of the gate kernels, a pure function of T: the grid is three blocks per CU, all resident at once
+// (the register kernels hold 12 waves per CU), unless that leaves a block fewer than two tokens per wave to pay for
+// its copy of the gate weight into LDS; very large T gets more blocks instead of more than 1024 tokens each (the
+// dispatch's scatter pass handles one or several whole blocks per chunk, at most 1024 tokens).
 int hdmoe_gate_tokens_per_block(int T) {
-  int tpb = WAVES_PER_BLOCK * 2;
-  while (tpb < 128 && (T + tpb - 1) / tpb > HDMOE_NUM_CU * 3) tpb *= 2;
+  const int resident = HDMOE_NUM_CU * 3;
+  int tpb = (T + resident - 1) / resident;
+  if (tpb < WAVES_PER_BLOCK * 2) tpb = WAVES_PER_BLOCK * 2;
+  if (tpb > 1024) tpb = 1024;
   return tpb;
 }
 
