@@ -57,7 +57,10 @@ extern "C" int hdmoe_layer_layout_get(int T, int D, int H, int Hs, int E, int we
   out->perm = take(n * 4);
   out->inv_perm = take(n * 4);
   // per-block expert histograms of the gate kernel (the first pass of the dispatch)
-  out->dispatch_ws = take(hdmoe_gate_hist_bytes(T, E));
+  {
+    const size_t a = hdmoe_gate_hist_bytes(T, E), b = hdmoe_dispatch_workspace_bytes(T, E);
+    out->dispatch_ws = take(a > b ? a : b);
+  }
   // a: routed rows sorted by expert [2T,D], then (fp8 only) the token-order copy for the shared expert [T,D]
   out->a = take((n + ((fp8 && Hs > 0) ? (size_t)T : 0)) * D * eb);
   // h: routed [2T,H] then shared [T,Hs]
@@ -119,7 +122,10 @@ extern "C" int hdmoe_moe_ffn(const hdmoe_layer_args* p, hdmoe_stream_t stream) {
   int32_t* offsets = reinterpret_cast<int32_t*>(ws + l.offsets);
   int32_t* perm = reinterpret_cast<int32_t*>(ws + l.perm);
   int32_t* inv_perm = reinterpret_cast<int32_t*>(ws + l.inv_perm);
-  int32_t* hist = reinterpret_cast<int32_t*>(ws + l.dispatch_ws);
+  // Up to 16384 tokens the gate kernel also counts (one expert histogram per block) and the dispatch is its scatter
+  // pass alone; above, the gate kernel's faster token order without histograms and the two-pass dispatch win.
+  int32_t* const dispatch_ws = reinterpret_cast<int32_t*>(ws + l.dispatch_ws);
+  int32_t* const hist = T <= 16384 ? dispatch_ws : nullptr;
   uint8_t* a_routed = ws + l.a;
   uint8_t* a_shared = a_routed + (size_t)n * D * eb;  // fp8 only
   uint8_t* h_routed = ws + l.h;
@@ -191,10 +197,15 @@ extern "C" int hdmoe_moe_ffn(const hdmoe_layer_args* p, hdmoe_stream_t stream) {
     if (int rc = hdmoe_launch_gate(xin, p->gate_w, T, D, E, idx, tw, hist, s, "hdmoe_moe_ffn (gate)")) return rc;
   }
   mark();
-  // the gate kernel has left the expert histogram of each of its blocks: the dispatch is its second pass alone
-  if (int rc = hdmoe_launch_dispatch_scatter(idx, T, E, counts, offsets, perm, inv_perm, hist,
-                                             hdmoe_gate_tokens_per_block(T), s, "hdmoe_moe_ffn (dispatch)"))
-    return rc;
+  if (hist != nullptr) {
+    if (int rc = hdmoe_launch_dispatch_scatter(idx, T, E, counts, offsets, perm, inv_perm, hist,
+                                               hdmoe_gate_tokens_per_block(T), s, "hdmoe_moe_ffn (dispatch)"))
+      return rc;
+  } else {
+    if (int rc = hdmoe_dispatch(idx, T, E, counts, offsets, perm, inv_perm, dispatch_ws,
+                                hdmoe_dispatch_workspace_bytes(T, E), stream))
+      return rc;
+  }
   mark();
 
   const uint8_t* a_static = nullptr;
