@@ -596,11 +596,16 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
       // The cast in front of the w2 Linear (ops.py:337-343) has three forms, fixed per tile: clamp to +-448 when
       // that Linear has no scale_input, nothing when 1/scale_input is 1, else multiply and round. The choice is
       // made once, outside the element loop.
-      auto swiglu_tile = [&](auto next_mode) {
+      // bf16 with the 320-token tile: 320 rows of 256 bytes are more than stage 1 holds, so the tile is staged and
+      // stored in two passes, the first three 32-token blocks of either wave row, then the last two.
+      constexpr bool TWO_PASS = !FP8 && TT == 5;
+      auto swiglu_tile = [&](auto next_mode, auto pass_c) {
         constexpr int NEXT = decltype(next_mode)::value;  // 0 clamp, 1 unit scale, 2 general scale
+        constexpr int PASS = decltype(pass_c)::value;     // -1: all blocks in one go; 0, 1: the passes of TWO_PASS
+        constexpr int TT0 = PASS == 1 ? 3 : 0, TT1 = PASS == 0 ? 3 : TT;
 #pragma unroll
-        for (int tt = 0; tt < TT; ++tt) {
-          const int tok = wt * WAVE_TOK + tt * 32 + tok32;
+        for (int tt = TT0; tt < TT1; ++tt) {
+          const int tok = PASS < 0 ? wt * WAVE_TOK + tt * 32 + tok32 : wt * ((TT1 - TT0) * 32) + (tt - TT0) * 32 + tok32;
           uint8_t* const row = stg + tok * ROWB;
 #pragma unroll
           for (int q = 0; q < 4; ++q) {
@@ -649,23 +654,43 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
           }
         }
       };
-      if constexpr (FP8) {
-        const int next = __builtin_amdgcn_readfirstlane(inv_next < 0.0f ? 0 : (inv_next == 1.0f ? 1 : 2));
-        if (next == 0) swiglu_tile(std::integral_constant<int, 0>{});
-        else if (next == 1) swiglu_tile(std::integral_constant<int, 1>{});
-        else swiglu_tile(std::integral_constant<int, 2>{});
-      } else {
-        swiglu_tile(std::integral_constant<int, 1>{});
-      }
-      __syncthreads();  // the tile's 256 x 128 outputs are staged
       constexpr int LANES_PER_ROW = ROWB / 16;
       constexpr int ROWS_PER_PASS = 64 / LANES_PER_ROW;
       const int c = lane % LANES_PER_ROW;
+      constexpr std::integral_constant<int, -1> all_blocks{};
+      if constexpr (TWO_PASS) {
+        auto store_pass = [&](auto pass_c) {
+          constexpr int PASS = decltype(pass_c)::value;
+          constexpr int TT0 = PASS == 1 ? 3 : 0, NTT = PASS == 0 ? 3 : TT - 3;
+          swiglu_tile(std::integral_constant<int, 1>{}, pass_c);
+          __syncthreads();  // this pass's 2 x NTT x 32 rows are staged
 #pragma unroll
-      for (int p = 0; p < (BM / 8) / ROWS_PER_PASS; ++p) {
-        const int r = wave * (BM / 8) + p * ROWS_PER_PASS + lane / LANES_PER_ROW;
-        const v4i v = *reinterpret_cast<const v4i*>(stg + r * ROWB + ((c ^ (r & 7)) << 4));
-        __builtin_amdgcn_raw_buffer_store_b128(v, ro, r * ldo + d.n0 * EB + c * 16, 0, 0);
+          for (int p = 0; p < (NTT * 8) / ROWS_PER_PASS; ++p) {
+            const int rl = wave * (NTT * 8) + p * ROWS_PER_PASS + lane / LANES_PER_ROW;    // staged row
+            const int r = (rl / (NTT * 32)) * WAVE_TOK + TT0 * 32 + rl % (NTT * 32);        // row of the tile
+            const v4i v = *reinterpret_cast<const v4i*>(stg + rl * ROWB + ((c ^ (rl & 7)) << 4));
+            __builtin_amdgcn_raw_buffer_store_b128(v, ro, r * ldo + d.n0 * EB + c * 16, 0, 0);
+          }
+        };
+        store_pass(std::integral_constant<int, 0>{});
+        __syncthreads();  // everyone has read the first pass's rows
+        store_pass(std::integral_constant<int, 1>{});
+      } else {
+        if constexpr (FP8) {
+          const int next = __builtin_amdgcn_readfirstlane(inv_next < 0.0f ? 0 : (inv_next == 1.0f ? 1 : 2));
+          if (next == 0) swiglu_tile(std::integral_constant<int, 0>{}, all_blocks);
+          else if (next == 1) swiglu_tile(std::integral_constant<int, 1>{}, all_blocks);
+          else swiglu_tile(std::integral_constant<int, 2>{}, all_blocks);
+        } else {
+          swiglu_tile(std::integral_constant<int, 1>{}, all_blocks);
+        }
+        __syncthreads();  // the tile's 256 x 128 outputs are staged
+#pragma unroll
+        for (int p = 0; p < (BM / 8) / ROWS_PER_PASS; ++p) {
+          const int r = wave * (BM / 8) + p * ROWS_PER_PASS + lane / LANES_PER_ROW;
+          const v4i v = *reinterpret_cast<const v4i*>(stg + r * ROWB + ((c ^ (r & 7)) << 4));
+          __builtin_amdgcn_raw_buffer_store_b128(v, ro, r * ldo + d.n0 * EB + c * 16, 0, 0);
+        }
       }
     } else {
       if constexpr (!BIAS) {
@@ -964,7 +989,8 @@ int hdmoe_launch_ffn_gemm(bool swiglu, int weight_dtype, const uint8_t* a_dyn, c
     return ((tiles + HDMOE_NUM_CU - 1) / HDMOE_NUM_CU) * (tt + 1);
   };
   const bool split = !swiglu && partial != nullptr && nparts > 1;  // split K runs on the 256-token tile
-  const bool tall = fp8 && !split && expected_cost(5) < expected_cost(4);
+  // (bf16: the gate/up kernel only; the down projection measured slower on the taller tile)
+  const bool tall = (fp8 || swiglu) && !split && expected_cost(5) < expected_cost(4);
   const int BM = tall ? TileCfg<5>::BM : TileCfg<4>::BM;  // tokens per block tile of the kernel that will run
   if (gather_dyn != nullptr && (unsigned long long)gather_rows * K_dyn * eb >= (1ull << 31))
     return hdmoe_fail(HDMOE_E_SHAPE, "%s: %d gathered rows of %d bytes exceed the 2 GiB offset range", what, gather_rows,
@@ -1080,6 +1106,7 @@ int hdmoe_launch_ffn_gemm(bool swiglu, int weight_dtype, const uint8_t* a_dyn, c
                                  : launch_grouped<FP8_PLAIN, 5>(args, tile_bound, s, what);
   if (fp8) return swiglu ? launch_grouped<FP8_SWIGLU>(args, tile_bound, s, what)
                          : launch_grouped<FP8_PLAIN>(args, tile_bound, s, what);
+  if (tall) return launch_grouped<BF16_SWIGLU, 5>(args, tile_bound, s, what);
   return swiglu ? launch_grouped<BF16_SWIGLU>(args, tile_bound, s, what)
                 : launch_grouped<BF16_PLAIN>(args, tile_bound, s, what);
 }

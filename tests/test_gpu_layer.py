@@ -171,16 +171,18 @@ def test_benchmark_configs(dev, name):
         assert torch.equal(a.cpu(), b)
 
 
-def test_production_row_counts_are_ragged(dev):
+@pytest.mark.parametrize("weights", ["fp8", "bf16"])
+def test_production_row_counts_are_ragged(dev, weights):
     """A single-stream block feeds image + text tokens: 2 x 4480 rows, not a multiple of any tile size, through the
-    full-size fp8 layer. Routing bit-exact on every token; outputs checked on a token subset that includes the
-    rows of the last, partial tile of every expert segment and of the shared expert."""
+    full-size layer (fp8, and bf16 weights, whose gate/up kernel takes its 320-token tile at this size). Routing
+    bit-exact on every token; outputs checked on a token subset that includes the rows of the last, partial tile of
+    every expert segment and of the shared expert."""
     from comfyui_amd import functional as HF
     cfg = synth.make_config("cfg2")
-    sd = synth.to_state_dict(cfg["master"], "fp8")
+    sd = synth.to_state_dict(cfg["master"], weights)
     g = torch.Generator().manual_seed(77)
     x = synth.make_input(g, 2 * 4480, batch=2)
-    y, idx, w, m = run_gpu(sd, x, "fp8", dev, synth.DIM)
+    y, idx, w, m = run_gpu(sd, x, weights, dev, synth.DIM)
     T = x.shape[0] * x.shape[1]
     xd = x.to(dev).reshape(T, -1)
     _, offsets, perm, _ = HF.dispatch(idx.to(dev), 4)
@@ -188,11 +190,18 @@ def test_production_row_counts_are_ragged(dev):
     picks = [torch.arange(T - 64, T), torch.arange(0, 32)]
     for e in range(4):
         seg_end = offsets[e + 1]
-        tail_start = offsets[e] + ((seg_end - offsets[e]) // 256) * 256      # first row of the segment's partial tile
-        rows = torch.arange(max(offsets[e], min(tail_start, seg_end - 16)), seg_end)
-        picks.append(perm[rows].long() // 2)
+        for tile in (256, 320):
+            tail_start = offsets[e] + ((seg_end - offsets[e]) // tile) * tile  # first row of the segment's partial tile
+            rows = torch.arange(max(offsets[e], min(tail_start, seg_end - 16)), seg_end)
+            picks.append(perm[rows].long() // 2)
+            # rows around the boundary between the two store passes of the bf16 320-token tile (blocks 0-2 | 3-4 of
+            # either wave row of 160 tokens)
+            first_tile = torch.arange(offsets[e], min(seg_end, offsets[e] + tile))
+            picks.append(perm[first_tile[88:104]].long() // 2)
+            picks.append(perm[first_tile[152:168]].long() // 2)
+            picks.append(perm[first_tile[248:264]].long() // 2)
     subset = torch.unique(torch.cat(picks))
-    check_layer(sd, x, "fp8", y, idx, w, 4, token_subset=subset)
+    check_layer(sd, x, weights, y, idx, w, 4, token_subset=subset)
 
 
 @pytest.mark.parametrize("dim,E,scaled", [(2560, 4, True), (512, 4, True), (512, 8, False), (2560, 2, True)])
