@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the HiDream MoE SwiGLU feed-forward layer on one MI355X.
 
-  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg3|cfg2|cfg1|cfg5-256|cfg5-4096|cfg3-branch|cfg4 [--layers L]] [--aux-kernels] [--no-cpu-baseline]
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg3|cfg2|cfg1|cfg5-256|cfg5-4096|cfg3-branch|cfg3-bf16|cfg4 [--layers L]] [--aux-kernels] [--no-cpu-baseline]
 
 A step is one forward of comfyui_amd.hidream.MOEFeedForwardSwiGLU (gate, dispatch, quantise,
 grouped fp8 GEMMs, combine, shared expert) over one synthetic batch that is already resident in
@@ -34,14 +34,17 @@ PEAK_HBM_GBPS = 8000.0      # MI355X HBM3E
 
 
 
-def gate_up_kernel_name(T, H, Hs, E, cus=256):
-    """Which kernel the library's launcher runs for the fp8 gate/up contraction of a layer (the rule of
+def gate_up_kernel_name(T, H, Hs, E, cus=256, fp8=True):
+    """Which kernel the library's launcher runs for the gate/up contraction of a layer (the rule of
     hdmoe_launch_ffn_gemm in comfyui_amd/csrc/gemm.hip, with HDMOE_SWIGLU4W unset): 320-token tiles in the 8-wave
-    kernel when they do not add a round of tiles to the persistent blocks, else 256-token tiles in the 4-wave one."""
+    kernel when they do not add a round of tiles to the persistent blocks, else 256-token tiles (fp8: in the 4-wave
+    kernel)."""
     def cost(tt):
         bm = 64 * tt
         tiles = E * (-(-(2 * T // E) // bm)) * (H // 128) + (-(-T // bm)) * (Hs // 128)
         return -(-tiles // cus) * (tt + 1)
+    if not fp8:
+        return "grouped_gemm_kernel<BF16_SWIGLU, %d>" % (5 if cost(5) < cost(4) else 4)
     return "grouped_gemm_kernel<FP8_SWIGLU, 5>" if cost(5) < cost(4) else "swiglu4w_kernel"
 
 
@@ -165,7 +168,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="cfg3", choices=["cfg1", "cfg2", "cfg3", "cfg5-256", "cfg5-4096", "cfg3-branch", "cfg4"])
+    ap.add_argument("--workload", default="cfg3", choices=["cfg1", "cfg2", "cfg3", "cfg5-256", "cfg5-4096", "cfg3-branch", "cfg3-bf16", "cfg4"])
     ap.add_argument("--layers", type=int, default=48, help="cfg4 only: number of stacked layers")
     ap.add_argument("--cpu-sample-tokens", type=int, default=8192)
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -202,7 +205,10 @@ def main():
         cfg, sd, module = dict(weights="fp8", x=None), None, modules[0]
         args.no_cpu_baseline = True              # the CPU baseline is quoted on the headline workload
     else:
-        cfg = synth.make_config(args.workload.replace("-branch", ""))
+        cfg = synth.make_config(args.workload.replace("-branch", "").replace("-bf16", ""))
+        if args.workload.endswith("-bf16"):      # the headline tokens and weights with the weights kept in bf16
+            cfg["weights"] = "bf16"
+            args.no_cpu_baseline = True
         sd = synth.to_state_dict(cfg["master"], cfg["weights"])
         cfg["master"] = None
         module = synth.build_module({k: v.to(dev) for k, v in sd.items()}, cfg["weights"], dev)
@@ -349,6 +355,7 @@ def main():
                          "cfg3-branch": "cfg3 tokens and weights through the block's whole feed-forward branch: x + gate_mlp * "
                                         "layer(LayerNorm(x) * (1 + scale_mlp) + shift_mlp), one enqueue (stage 'gate' "
                                         "includes the LayerNorm kernel, stage 'combine' the gated residual)",
+                         "cfg3-bf16": "cfg3 tokens (2x4096 = 8192, 1% outlier channels x20) with bf16 weights",
                          "cfg3": "cfg3 (headline): 2x4096 = 8192 tokens x 2560, scaled fp8 e4m3fn weights "
                                  "(scale_weight = amax/448, scale_input = 1.0), bf16 gate, x ~ N(0,1) with 1% "
                                  "outlier channels x20, 4 routed experts (hidden 6912) top-2 + shared expert (hidden 3584)"}[args.workload],
@@ -364,7 +371,7 @@ def main():
         "stage_ms": stage_ms,
         "gemm_down_tflops": gemm2_tflops,
         "roofline": {
-            "kernel": gate_up_kernel_name(T, H, Hs, E) if fp8 else "grouped_gemm_kernel<BF16_SWIGLU, 4>",
+            "kernel": gate_up_kernel_name(T, H, Hs, E, fp8=fp8),
             "bound": "mfma",
             "achieved": gemm1_tflops,
             "peak": peak,
