@@ -323,9 +323,9 @@ def main():
     gate_bytes = T * D * 2 + E * D * 2 + T * 2 * (4 + 2)
     # dispatch as built: index sort (the gate kernel counts, so the 2T ids are read once; write perm + inv_perm). fp8: the gate kernel also writes the
     # token's e4m3fn row, once, because every scale_input of these configurations is the same value (it would be three
-    # rows, two routed slots + shared expert, with differing scales), and nothing is permuted; bf16: the routed rows
-    # are materialised in expert order (read + write 2T rows).
-    dispatch_bytes = (2 * T * 4) + 2 * (2 * T * 4) + (T * D if fp8 else 2 * (2 * T * D * 2))
+    # rows, two routed slots + shared expert, with differing scales). Nothing is permuted for either weight type: the
+    # gate/up GEMM reads the routed rows through the permutation.
+    dispatch_bytes = (2 * T * 4) + 2 * (2 * T * 4) + (T * D if fp8 else 0)
     combine_bytes = 2 * T * D * 2 + T * D * 2 + T * D * 2 + T * 2 * 2 + 2 * T * 4
 
     traffic_bytes, traffic_entry = measured_traffic(args.workload)

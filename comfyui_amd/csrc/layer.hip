@@ -61,8 +61,9 @@ extern "C" int hdmoe_layer_layout_get(int T, int D, int H, int Hs, int E, int we
     const size_t a = hdmoe_gate_hist_bytes(T, E), b = hdmoe_dispatch_workspace_bytes(T, E);
     out->dispatch_ws = take(a > b ? a : b);
   }
-  // a: routed rows sorted by expert [2T,D], then (fp8 only) the token-order copy for the shared expert [T,D]
-  out->a = take((n + ((fp8 && Hs > 0) ? (size_t)T : 0)) * D * eb);
+  // a (fp8 only; bf16 weights multiply the tokens themselves): the tokens' e4m3fn rows per flat slot [2T,D], then
+  // the token-order copy for the shared expert [T,D]
+  out->a = take(fp8 ? (n + (Hs > 0 ? (size_t)T : 0)) * D * eb : 0);
   // h: routed [2T,H] then shared [T,Hs]
   out->h = take((n * H + (size_t)T * Hs) * eb);
   // y: routed [2T,D] then shared [T,D], bf16
@@ -208,20 +209,23 @@ extern "C" int hdmoe_moe_ffn(const hdmoe_layer_args* p, hdmoe_stream_t stream) {
   }
   mark();
 
+  // bf16 weights: the GEMM reads the tokens themselves, the routed rows through the permutation (row perm[r] / 2
+  // of x), so no permuted copy is written
   const uint8_t* a_static = nullptr;
   if (fp8) {
     if (Hs > 0) a_static = a_shared;
   } else {
-    if (int rc = hdmoe_permute_bf16(xin, perm, T, D, a_routed, stream)) return rc;
     a_static = static_cast<const uint8_t*>(xin);
   }
 
   mark();
   // gate/up projections + SiLU*mul, routed experts and shared expert in one launch
-  if (int rc = hdmoe_launch_ffn_gemm(true, wd, one_copy ? a_shared : a_routed, offsets, (int)n, E, p->experts, h_routed,
+  const bool per_token = one_copy || !fp8;  // the routed operand holds one row per token (else one per flat slot)
+  const uint8_t* const a_dyn = !fp8 ? static_cast<const uint8_t*>(xin) : (one_copy ? a_shared : a_routed);
+  if (int rc = hdmoe_launch_ffn_gemm(true, wd, a_dyn, offsets, (int)n, E, p->experts, h_routed,
                                      a_static, Hs > 0 ? T : 0, p->shared, h_shared, D, H, D, Hs, s,
-                                     "hdmoe_moe_ffn (gate/up)", fp8 ? perm : nullptr, one_copy ? T : (int)n, nullptr, 1,
-                                     one_copy ? 1 : 0))
+                                     "hdmoe_moe_ffn (gate/up)", perm, per_token ? T : (int)n, nullptr, 1,
+                                     per_token ? 1 : 0))
     return rc;
   mark();
   // down projections, both in one launch
