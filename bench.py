@@ -155,7 +155,23 @@ def aux_kernels(dev, module, x):
         ms = e0.elapsed_time(e1) / reps
         return {"ms": ms, "bytes": nbytes, "GBps": nbytes / ms / 1e6, "frac_of_hbm_peak": nbytes / ms / 1e6 / PEAK_HBM_GBPS}
 
+    def hunyuan_block(dtype, tokens=8192, dim=2048, inner=8192, E=8):
+        """The sibling model's MoE block (Hunyuan3D-2.1: width 2048, 8 GELU experts of hidden 8192, top-2, shared
+        expert) at 2 x 4096 latent tokens, random weights; TFLOP/s over the 6 Linears a token goes through."""
+        from comfyui_amd import hunyuan3d as H
+        m = H.MoEBlock(dim, num_experts=E, moe_top_k=2, ff_inner_dim=inner, dtype=dtype, device=dev).eval()
+        gg = torch.Generator(device=dev).manual_seed(3)
+        with torch.no_grad():
+            for prm in m.parameters():
+                prm.copy_((torch.randn(prm.shape, generator=gg, device=dev) / (prm.shape[-1] ** 0.5 if prm.dim() > 1 else 5.0)).to(dtype))
+            xh = torch.randn((2, tokens // 2, dim), generator=gg, device=dev).to(dtype)
+            r = timed(lambda: m(xh), 0, reps=20)
+        flop = tokens * 3 * 2 * 2 * dim * inner
+        return {"ms": r["ms"], "tokens": tokens, "TFLOPs": flop / r["ms"] / 1e9, "frac_of_mfma_peak": flop / r["ms"] / 1e9 / PEAK_BF16_TFLOPS}
+
     return {
+        "hunyuan3d_moe_block_bf16": hunyuan_block(torch.bfloat16),
+        "hunyuan3d_moe_block_fp16": hunyuan_block(torch.float16),
         "ln_modulate": timed(lambda: HF.ln_modulate(x2, scale, shift, S), 2 * T * D * 2),
         "combine": timed(lambda: HF.combine(y, inv, w, sh), 4 * T * D * 2 + T * 12),
         "combine_gated_residual": timed(lambda: HF.combine_gated_residual(y, inv, w, sh, gate, x2, S), 5 * T * D * 2 + T * 12),
