@@ -31,6 +31,7 @@
 // from its index and exits if its index is past the real tile count. Block ids are
 // remapped so that each XCD (ids congruent mod 8) walks a contiguous range of tiles,
 // 4 m-tiles deep, and its L2 sees each operand tile reused by neighbouring blocks.
+#include <cmath>
 #include <cstdlib>
 #include <type_traits>
 
@@ -1174,7 +1175,19 @@ int hdmoe_launch_linear_groups(const uint8_t* a_dyn, const int32_t* offsets, int
     gg.dyn = e;
     if (!gg.b0) return hdmoe_fail(HDMOE_E_NULL, "%s: expert %d has a NULL weight", what, e);
   }
-  constexpr int BM = TileCfg<4>::BM;
+  // tile height by the rule of the feed-forward GEMMs: the 320-token tile when it saves a round of tiles
+  auto expected_cost = [&](int tt) {
+    const int bm = 64 * tt;
+    long tiles = 0;
+    // a segment taken one standard deviation of an even routing above the mean: at a mean that is a multiple of the
+    // tile height half the segments need one tile more
+    const int seg = n_dyn > 0 ? rows_dyn / n_dyn + (int)sqrtf((float)(rows_dyn / n_dyn)) : 0;
+    if (n_dyn > 0) tiles += (long)n_dyn * ((seg + bm - 1) / bm) * (N / BN);
+    if (shared != nullptr && rows_static > 0) tiles += (long)((rows_static + bm - 1) / bm) * (N / BN);
+    return ((tiles + HDMOE_NUM_CU - 1) / HDMOE_NUM_CU) * (tt + 1);
+  };
+  const bool tall = expected_cost(5) < expected_cost(4);
+  const int BM = tall ? TileCfg<5>::BM : TileCfg<4>::BM;
   if (n_dyn > 0) tile_bound += (rows_dyn / BM + n_dyn) * (N / BN);
   if (shared != nullptr && rows_static > 0) {
     GemmGroup& gg = args.g[G];
@@ -1188,6 +1201,8 @@ int hdmoe_launch_linear_groups(const uint8_t* a_dyn, const int32_t* offsets, int
     ++G;
   }
   args.G = G;
+  if (tall) return f16 ? launch_grouped<F16_PLAIN_BIAS, 5>(args, tile_bound, s, what)
+                       : launch_grouped<BF16_PLAIN_BIAS, 5>(args, tile_bound, s, what);
   return f16 ? launch_grouped<F16_PLAIN_BIAS>(args, tile_bound, s, what)
              : launch_grouped<BF16_PLAIN_BIAS>(args, tile_bound, s, what);
 }

@@ -21,7 +21,8 @@ def close_bf16(got, ref, frac_exact=0.97, rel=6e-3):
 
 
 @pytest.mark.parametrize("act", ["none", "gelu"])
-@pytest.mark.parametrize("rows,K,N,bias", [(1, 256, 256, True), (300, 512, 768, True), (1025, 2048, 512, False)])
+@pytest.mark.parametrize("rows,K,N,bias", [(1, 256, 256, True), (300, 512, 768, True), (1025, 2048, 512, False),
+                                          (10000, 256, 2048, True)])   # the last: 320-token tiles, partial last tile
 def test_single_linear_with_bias_and_gelu(dev, act, rows, K, N, bias):
     from comfyui_amd import functional as HF
     g = torch.Generator().manual_seed(rows + K)
@@ -182,3 +183,25 @@ def test_training_mode_and_cpu_are_refused(dev):
         m.train()(torch.zeros((1, 4, 256), dtype=BF16, device=dev))
     with pytest.raises(RuntimeError):
         m.eval()(torch.zeros((1, 4, 256), dtype=BF16))
+
+
+def test_grouped_linear_on_320_token_tiles(dev):
+    """Segment sizes at which the launcher takes the 320-token tile (232 tiles in one round instead of 288 in two):
+    ragged segments, an empty expert, partial last tiles, a static group."""
+    from comfyui_amd import functional as HF
+    g = torch.Generator().manual_seed(11)
+    K, N, E = 256, 2048, 7
+    counts = [1500, 0, 1280, 1300, 1290, 1310, 1060]
+    rows = sum(counts)
+    offsets = torch.tensor([0] + torch.tensor(counts).cumsum(0).tolist(), dtype=torch.int32)
+    a = torch.randn((rows, K), generator=g).to(BF16)
+    ws = [((torch.randn((N, K), generator=g) / 16).to(BF16), torch.randn((N,), generator=g).to(BF16)) for _ in range(E)]
+    xs = torch.randn((90, K), generator=g).to(BF16)
+    wsh = ((torch.randn((N, K), generator=g) / 16).to(BF16), torch.randn((N,), generator=g).to(BF16))
+    out, out_sh = HF.grouped_linear(a.to(dev), offsets.to(dev), [(w.to(dev), b.to(dev)) for w, b in ws],
+                                    a_static=xs.to(dev), shared=(wsh[0].to(dev), wsh[1].to(dev)), act="gelu")
+    for e in range(E):
+        lo, hi = int(offsets[e]), int(offsets[e + 1])
+        if hi > lo:
+            close_bf16(out[lo:hi].cpu(), torch.nn.functional.gelu(O.linear_bias(a[lo:hi], *ws[e])), frac_exact=0.93)
+    close_bf16(out_sh.cpu(), torch.nn.functional.gelu(O.linear_bias(xs, *wsh)), frac_exact=0.93)

@@ -41,7 +41,8 @@ def test_gate_f16_bit_exact(dev, T, D, E):
 
 
 @pytest.mark.parametrize("act", ["none", "gelu"])
-@pytest.mark.parametrize("rows,K,N,bias", [(1, 256, 256, True), (300, 512, 768, True), (1025, 2048, 512, False)])
+@pytest.mark.parametrize("rows,K,N,bias", [(1, 256, 256, True), (300, 512, 768, True), (1025, 2048, 512, False),
+                                          (10000, 256, 2048, True)])   # the last: 320-token tiles, partial last tile
 def test_single_linear_with_bias_and_gelu_f16(dev, act, rows, K, N, bias):
     from comfyui_amd import functional as HF
     g = torch.Generator().manual_seed(rows + K)
@@ -198,3 +199,26 @@ def test_f32_activations_are_refused(dev):
     m = H.MoEBlock(256, num_experts=6, moe_top_k=2, ff_inner_dim=1024, dtype=torch.float32, device=dev).eval()
     with pytest.raises(RuntimeError):
         m(torch.zeros((1, 8, 256), dtype=torch.float32, device=dev))
+
+
+def test_grouped_linear_on_320_token_tiles_f16(dev):
+    """Segment sizes at which the launcher takes the 320-token tile (232 tiles in one round instead of 288 in two):
+    ragged segments, an empty expert, partial last tiles, a static group."""
+    from comfyui_amd import functional as HF
+    g = torch.Generator().manual_seed(11)
+    K, N, E = 256, 2048, 7
+    counts = [1500, 0, 1280, 1300, 1290, 1310, 1060]
+    rows = sum(counts)
+    offsets = torch.tensor([0] + torch.tensor(counts).cumsum(0).tolist(), dtype=torch.int32)
+    a = torch.randn((rows, K), generator=g).to(F16)
+    ws = [((torch.randn((N, K), generator=g) / 16).to(F16), torch.randn((N,), generator=g).to(F16)) for _ in range(E)]
+    xs = torch.randn((90, K), generator=g).to(F16)
+    wsh = ((torch.randn((N, K), generator=g) / 16).to(F16), torch.randn((N,), generator=g).to(F16))
+    out, out_sh = HF.grouped_linear(a.to(dev), offsets.to(dev), [(w.to(dev), b.to(dev)) for w, b in ws],
+                                    a_static=xs.to(dev), shared=(wsh[0].to(dev), wsh[1].to(dev)), act="gelu")
+    gelu = lambda t: torch.nn.functional.gelu(t.float()).to(F16)
+    for e in range(E):
+        lo, hi = int(offsets[e]), int(offsets[e + 1])
+        if hi > lo:
+            close_f16(out[lo:hi].cpu(), gelu(O.linear_bias(a[lo:hi], *ws[e])), frac_exact=0.93)
+    close_f16(out_sh.cpu(), gelu(O.linear_bias(xs, *wsh)), frac_exact=0.93)
