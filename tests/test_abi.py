@@ -86,6 +86,19 @@ def test_argument_errors_are_reported_without_a_device():
     assert L.hdmoe_linear(7, p, 4, 128, 256, p, p, None, p, None) == _lib.E_SHAPE
     assert L.hdmoe_linear(_lib.W_BF16, p, 0, 64, 256, p, None, None, p, None) == 0
     assert L.hdmoe_silu_mul_bf16(p, p, 12, p, None) == _lib.E_SHAPE
+    # the fp16 entry points and the fp16 weight code
+    assert L.hdmoe_gate_top2_f16(None, p, 4, 2048, 8, p, p, None) == _lib.E_NULL
+    assert b"x_f16" in L.hdmoe_last_error()
+    assert L.hdmoe_gate_top2_f16(p, p, 4, 2049, 8, p, p, None) == _lib.E_SHAPE
+    assert L.hdmoe_gate_top2_f16(p, p, 0, 2048, 8, p, p, None) == 0
+    assert L.hdmoe_combine_f16(p, p, p, None, 4, 12, p, None) == _lib.E_SHAPE
+    assert L.hdmoe_gelu_f16(p, 12, p, None) == _lib.E_SHAPE
+    assert L.hdmoe_grouped_linear_f16(p, p, 8, 17, None, p, None, 0, None, None, 256, 256, 0, None) == _lib.E_SHAPE
+    assert L.hdmoe_grouped_linear_f16(p, p, 8, 2, None, p, None, 0, None, None, 256, 256, 0, None) == _lib.E_NULL
+    assert L.hdmoe_linear(_lib.W_F16, p, 4, 128, 256, p, None, None, p, None) == _lib.E_SHAPE    # fp16: hdmoe_linear_bias only
+    assert L.hdmoe_linear_bias(_lib.W_F16, p, 4, 100, 256, p, None, None, None, p, None) == _lib.E_SHAPE
+    assert L.hdmoe_linear_bias(_lib.W_F16, p, 0, 128, 256, p, None, None, None, p, None) == 0
+    assert L.hdmoe_layer_workspace_bytes(16, 2560, 6912, 3584, 4, _lib.W_F16) == 0               # the layer takes bf16 / fp8
     assert L.hdmoe_moe_ffn(None, None) == _lib.E_NULL
     args = _lib.LayerArgs()
     args.T, args.D, args.H, args.Hs, args.E, args.weight_dtype = 16, 2560, 6912, 3584, 4, _lib.W_E4M3FN
