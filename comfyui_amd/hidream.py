@@ -92,6 +92,35 @@ def _fusable_dtype(ffns):
     return wdt
 
 
+def _lin_tensors(l):
+    """(weight, bias, scale_weight, scale_input) of a Linear, read from the module's own dictionaries: nn.Module's
+    __getattr__ costs about as much per access as everything else here together."""
+    d = l.__dict__
+    p = d["_parameters"]
+    sw = p["scale_weight"] if "scale_weight" in p else d.get("scale_weight")
+    si = p["scale_input"] if "scale_input" in p else d.get("scale_input")
+    return p["weight"], p.get("bias"), sw, si
+
+
+def _pack_key(ffns, dev):
+    """Everything the packed pointer structures of `ffns` depend on, or None when they cannot be reused from one call
+    to the next (weights that are cast, moved or patched per call). Values of scale_input enter through the version
+    counters and ops.invalidate_scale_cache(), as they do for ops.scale_value."""
+    key = [dev, amd_ops._scale_epoch]
+    for f in ffns:
+        mods = f.__dict__["_modules"]
+        for l in (mods["w1"], mods["w2"], mods["w3"]):
+            w, b, sw, si = _lin_tensors(l)
+            if w.device != dev or getattr(l, "weight_function", None) or getattr(l, "bias_function", None):
+                return None
+            if (sw is not None and sw.device != dev) or (si is not None and si.device != dev):
+                return None
+            key.append((type(l), l.training, w.data_ptr(), w.dtype, b is None, getattr(l, "hdmoe_fp8_matrix_mult", None),
+                        None if sw is None else (sw.data_ptr(), sw._version),
+                        None if si is None else (si.data_ptr(), si._version)))
+    return tuple(key)
+
+
 class FeedForwardSwiGLU(nn.Module):
     def __init__(self, dim: int, hidden_dim: int, multiple_of: int = 256,
                  ffn_dim_multiplier: Optional[float] = None, dtype=None, device=None, operations=None):
@@ -190,6 +219,14 @@ class MOEFeedForwardSwiGLU(nn.Module):
         """Device pointers of all 15 Linears for the one-call path, or None when the layer
         needs the per-Linear composition. Returned tensors are kept alive by the caller."""
         ffns = list(self.experts) + [self.shared_experts]
+        # resident, unpatched weights: the structures of the previous call hold as long as nothing they were built
+        # from has changed
+        key = _pack_key(ffns, x.device)
+        cached = self.__dict__.get("_packed")
+        if key is not None and cached is not None and cached[0] == key:
+            self.__dict__["_uniform_scale_in"] = cached[2]
+            return cached[1]
+        self.__dict__["_packed"] = None
         wdt = _fusable_dtype(ffns)
         if wdt is None:
             return None
@@ -201,14 +238,19 @@ class MOEFeedForwardSwiGLU(nn.Module):
                 return None
             packed.append(fw)
         # one scale_input value for every Linear that reads the tokens: they are cast to fp8 once
-        self._uniform_scale_in = False
+        uniform = False
         if wdt == FP8:
             sis = [getattr(f.w1, "scale_input", None) for f in ffns]
             if all(si is None for si in sis):
-                self._uniform_scale_in = True
+                uniform = True
             elif all(si is not None for si in sis):
                 v0 = amd_ops.scale_value(sis[0])
-                self._uniform_scale_in = all(amd_ops.scale_value(si) == v0 for si in sis[1:])
+                uniform = all(amd_ops.scale_value(si) == v0 for si in sis[1:])
+        self.__dict__["_uniform_scale_in"] = uniform
+        if key is not None:
+            # the structures hold raw pointers of tensors the module owns and the key was read from: no tensor is
+            # referenced from the cache (an offloaded or replaced weight must be free to go)
+            self.__dict__["_packed"] = (key, (wdt, packed[:-1], packed[-1], ()), uniform)
         return wdt, packed[:-1], packed[-1], keep
 
     def forward(self, x, stage_events=None):

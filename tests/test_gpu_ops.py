@@ -371,3 +371,48 @@ def test_checkpoint_file_onto_the_device_and_forward(dev, tmp_path):
     y = m(x.to(dev))
     idx, w = HF.gate_top2(x.to(dev).reshape(-1, 512), m.gate.weight)
     check_layer(sd, x, "fp8", y.cpu(), idx.cpu(), w.cpu(), 4)
+
+
+def test_packed_pointers_are_reused_only_while_nothing_changed(dev):
+    """The module keeps the pointer structures of the previous call while every weight and scale is the same tensor
+    at the same address. It must notice: a Parameter's storage swapped under it (`p.data = ...`), a scale_input
+    changed in place (after ops.invalidate_scale_cache(), as for ops.scale_value), train/eval of fp8_ops Linears;
+    and it must not keep a replaced weight alive."""
+    import gc
+    import weakref
+    from comfyui_amd import ops
+    dim = 256
+    sd, x = small_layer(seed=5, dim=dim, tokens=90, weights="fp8")
+    m = synth.build_module({k: v.to(dev) for k, v in sd.items()}, "fp8", dev, dim=dim)
+    xd = x.to(dev)
+    base = m(xd).cpu()
+    assert torch.equal(m(xd).cpu(), base) and m.__dict__.get("_packed") is not None
+    idx, w, _, _ = O.gate_fixed_order(x.reshape(-1, dim), sd["gate.weight"])
+
+    def oracle(state):
+        return O.moe_forward(x, oracle_params(state, 4), "fp8mm", gate_result=(idx, w))
+    # (a) storage swapped in place
+    lin = m.experts[1].w3
+    old = weakref.ref(lin.weight.data)
+    lin.weight.data = sd["experts.0.w3.weight"].to(dev).clone()
+    sd2 = dict(sd)
+    sd2["experts.1.w3.weight"] = sd["experts.0.w3.weight"]
+    got = m(xd).cpu()
+    close(got, oracle(sd2), 1e-2)
+    assert not torch.equal(got, base)
+    gc.collect()
+    assert old() is None, "the replaced weight is still referenced"
+    # (b) a scale_input value changed in place: visible after the documented invalidation
+    with torch.no_grad():
+        for e in range(4):
+            m.experts[e].w2.scale_input.data.fill_(0.5)
+        m.shared_experts.w2.scale_input.data.fill_(0.5)
+    ops.invalidate_scale_cache()
+    sd3 = dict(sd2)
+    for k in sd3:
+        if k.endswith("w2.scale_input"):
+            sd3[k] = torch.tensor(0.5)
+    close(m(xd).cpu(), oracle(sd3), 1e-2)
+    # (c) another device tensor for x's device is the same key; a CPU-resident Linear drops the cache
+    m.experts[0].w1.to("cpu")
+    assert torch.equal(m(xd).cpu(), m(xd).cpu()) and m.__dict__.get("_packed") is None
