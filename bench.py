@@ -38,7 +38,10 @@ def gate_up_kernel_name(T, H, Hs, E, cus=256, fp8=True):
     """Which kernel the library's launcher runs for the gate/up contraction of a layer (the rule of
     hdmoe_launch_ffn_gemm in comfyui_amd/csrc/gemm.hip, with HDMOE_SWIGLU4W unset): 320-token tiles in the 8-wave
     kernel when they do not add a round of tiles to the persistent blocks, else 256-token tiles (fp8: in the 4-wave
-    kernel)."""
+    kernel; with one tile per segment and the experts' half empty on average, in the form of the 8-wave kernel that
+    skips the token blocks without rows)."""
+    if fp8 and 2 * T <= 128 * E and T <= 256:
+        return "grouped_gemm_kernel<FP8_SWIGLU, 4, LIGHT>"
     def cost(tt):
         bm = 64 * tt
         tiles = E * (-(-(2 * T // E) // bm)) * (H // 128) + (-(-T // bm)) * (Hs // 128)

@@ -18,12 +18,17 @@
  *   - the only state the library keeps between calls: the thread-local error message, and per device one flag per
  *     GEMM kernel variant recording that hipFuncSetAttribute (the opt-in for more than 64 KiB of dynamic LDS) has
  *     been called for it on that device, plus the device address of the built-in buffer of hdmoe_dispatch_static;
- *   - one environment variable is read, at every call that runs the fp8 gate/up contraction: HDMOE_SWIGLU4W. That
- *     contraction has two kernels with the same results bit for bit: the 8-wave one (256- or 320-token tiles) and a
- *     4-wave one (one wave per SIMD, 256-token tiles, a tile's SiLU*mul epilogue issued between the MFMAs of the next
- *     tile; needs K a multiple of 256 and at least 2048, and scale_in2). Unset: the 4-wave kernel runs where the
- *     320-token tile would not be used (up to about 5000 tokens for HiDream's sizes; it is 2-3 % faster there and
- *     1-2 % slower above). "0": never. Anything else: whenever the shapes allow;
+ *   - two environment variables are read, at every call that runs an fp8 feed-forward contraction. Both choose
+ *     between kernels with the same results bit for bit.
+ *     HDMOE_SWIGLU4W: the gate/up contraction has an 8-wave kernel (256- or 320-token tiles) and a 4-wave one (one
+ *     wave per SIMD, 256-token tiles, a tile's SiLU*mul epilogue issued between the MFMAs of the next tile; needs K a
+ *     multiple of 256 and at least 2048, and scale_in2). Unset: the 4-wave kernel runs where the 320-token tile would
+ *     not be used (up to about 5000 tokens for HiDream's sizes; it is 2-3 % faster there and 1-2 % slower above).
+ *     "0": never. Anything else: whenever the shapes allow.
+ *     HDMOE_LIGHT: the 8-wave kernels (gate/up and down) have a form whose K loop skips the 32-token blocks of a tile
+ *     that hold no rows. Unset: it runs when every segment is one tile and the experts' tiles are half empty on
+ *     average (rows per expert <= 128 and shared rows <= 256: up to 256 tokens for HiDream's sizes; 3-12 % faster
+ *     there, slower above). "0": never. Anything else: always;
  *   - return value 0 = enqueued; negative = HDMOE_E_* and nothing was enqueued;
  *     hdmoe_last_error() gives a thread-local message for the last failure;
  *   - scale pointers (float*, device) address the fp32 scalar Parameters

@@ -1,0 +1,166 @@
+"""The fp8 contractions of launches with few rows per segment run in the form of the tile kernel whose K loop skips
+the 32-token blocks without rows (csrc/gemm.hip, LIGHT; HDMOE_LIGHT in the environment forces it on or off). Same MFMA,
+same operand layout, same order over K and same epilogue as the assembly loop, so the same bytes out."""
+import os
+
+import pytest
+import torch
+
+from comfyui_amd import synth
+from oracle import hidream_moe_oracle as O
+from tests.helpers import oracle_params, small_layer
+
+pytestmark = pytest.mark.gpu
+BF16 = torch.bfloat16
+
+
+@pytest.fixture
+def light_env():
+    old = {k: os.environ.get(k) for k in ("HDMOE_LIGHT", "HDMOE_SWIGLU4W")}
+    yield
+    for k, v in old.items():
+        if v is None:
+            os.environ.pop(k, None)
+        else:
+            os.environ[k] = v
+
+
+def grouped_swiglu(T, D, H, E, seed, dev, s_next):
+    """h of hdmoe_grouped_swiglu on random routed rows: assembly loop, then the loop that skips padding."""
+    from comfyui_amd import _lib, functional as HF
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn((T, D), generator=g).to(BF16)
+    ws = []
+    for _ in range(E):
+        w1, s1 = synth.quantize_per_tensor(torch.randn((H, D), generator=g) * 0.03)
+        w3, s3 = synth.quantize_per_tensor(torch.randn((H, D), generator=g) * 0.03)
+        ws.append((w1.to(dev), s1.to(dev).float().reshape(()), w3.to(dev), s3.to(dev).float().reshape(())))
+    if E >= 2:
+        idx = torch.stack([torch.randperm(E, generator=g)[:2] for _ in range(T)]).to(torch.int32)
+    else:
+        idx = torch.zeros((T, 2), dtype=torch.int32)
+    _, offsets, perm, _ = HF.dispatch(idx.to(dev), E)
+    s_in = torch.tensor(1.0, device=dev)
+    s_nx = torch.tensor(s_next, device=dev)
+    xs = HF.quant_fp8(x.to(dev), s_in)[(perm // 2).long()].contiguous()
+
+    def weights(w):
+        f = _lib.FfnWeights()
+        f.w1, f.w3, f.scale_w1, f.scale_w3 = w[0].data_ptr(), w[2].data_ptr(), w[1].data_ptr(), w[3].data_ptr()
+        f.scale_in1 = f.scale_in3 = s_in.data_ptr()
+        f.scale_in2 = s_nx.data_ptr()
+        return f
+    arr = (_lib.FfnWeights * E)(*[weights(w) for w in ws])
+    out = []
+    os.environ["HDMOE_SWIGLU4W"] = "0"
+    for form in ("0", "1"):
+        os.environ["HDMOE_LIGHT"] = form
+        h = torch.full((2 * T, H), 0x55, dtype=torch.uint8, device=dev)
+        _lib.check(_lib.lib.hdmoe_grouped_swiglu(_lib.W_E4M3FN, xs.data_ptr(), offsets.data_ptr(), 2 * T, E, D, H, arr,
+                                                 h.data_ptr(), None))
+        torch.cuda.synchronize()
+        out.append(h.cpu())
+    return out
+
+
+@pytest.mark.parametrize("T,D,H,E,s_next", [
+    (1, 2048, 128, 1, 1.0),         # one row, one tile
+    (64, 2048, 128, 4, 1.0),        # a token block or two per expert
+    (128, 2560, 6912, 4, 0.37),     # the layer's shapes at 128 tokens: 54 feature tiles per expert
+    (300, 2048, 256, 2, 0.5),       # more than one 256-row tile in a segment
+    (40, 2304, 256, 16, 1.0),       # 16 experts, most of them empty or a few rows; 18 K steps
+    (200, 384, 128, 3, 2.0),        # 3 K steps (odd)
+    (97, 512, 384, 5, 0.25),        # 4 K steps, an odd number of feature tiles
+    (500, 6912, 256, 2, 1.0),       # the down projection's K as the contraction length
+])
+def test_same_bytes_from_both_kernels(dev, light_env, T, D, H, E, s_next):
+    base, light = grouped_swiglu(T, D, H, E, seed=T + H, dev=dev, s_next=s_next)
+    assert not bool((base == 0x55).all())
+    assert torch.equal(base, light)
+
+
+@pytest.mark.parametrize("tokens", [1, 7, 64, 256, 300, 700])
+@pytest.mark.parametrize("scale_in", [None, 0.5])
+def test_layer_through_the_light_form(dev, light_env, tokens, scale_in):
+    """The whole layer: gate/up (rows gathered through the dispatch permutation, shared expert in the same launch)
+    and the down projection (split over K into fp32 partial sums, or unsplit) against the tile kernels, bit for bit,
+    and against the oracle."""
+    dim = 2048
+    sd, x = small_layer(seed=300 + tokens, dim=dim, tokens=tokens, weights="fp8", scale_in=scale_in)
+    m = synth.build_module({k: v.to(dev) for k, v in sd.items()}, "fp8", dev, dim=dim)
+    os.environ["HDMOE_SWIGLU4W"] = "0"
+    os.environ["HDMOE_LIGHT"] = "0"
+    base = m(x.to(dev)).cpu()
+    os.environ["HDMOE_LIGHT"] = "1"
+    light = m(x.to(dev)).cpu()
+    assert torch.equal(base.view(torch.int16), light.view(torch.int16))
+    idx, w, _, _ = O.gate_fixed_order(x.reshape(-1, dim), sd["gate.weight"])
+    ref = O.moe_forward(x, oracle_params(sd, 4), "fp8mm", gate_result=(idx, w))
+    d = O.error_metrics(light, ref)
+    assert d["rel_rms"] <= 1e-2, d
+
+
+def test_dense_feed_forward_through_both_kernels(dev, light_env):
+    """hdmoe_ffn_swiglu (the shared expert / text feed-forward on its own: one static group, no gather)."""
+    from comfyui_amd import hidream, ops
+    FP8 = torch.float8_e4m3fn
+    dim, hidden = 2048, 1536
+    g = torch.Generator().manual_seed(5)
+    cls = ops.scaled_fp8_ops(fp8_matrix_mult=True, scale_input=True, override_dtype=FP8)
+    ff = hidream.FeedForwardSwiGLU(dim, hidden, dtype=BF16, device=dev, operations=cls).eval()
+    for lin in (ff.w1, ff.w2, ff.w3):
+        w8, sw = synth.quantize_per_tensor(torch.randn(tuple(lin.weight.shape), generator=g) * 0.03)
+        lin.weight = torch.nn.Parameter(w8.to(dev), requires_grad=False)
+        with torch.no_grad():
+            lin.scale_weight.copy_(sw)
+            lin.scale_input.fill_(0.5)
+    for shape in ((1, 77, dim), (2, 450, dim)):
+        x = torch.randn(shape, generator=g).to(BF16).to(dev)
+        os.environ["HDMOE_LIGHT"] = "0"
+        base = ff(x).cpu()
+        os.environ["HDMOE_LIGHT"] = "1"
+        light = ff(x).cpu()
+        assert bool(torch.isfinite(base.float()).all()) and float(base.float().abs().max()) > 0
+        assert torch.equal(base.view(torch.int16), light.view(torch.int16))
+
+
+def test_layer_with_the_light_form_in_a_graph(dev, light_env):
+    """Capture and replay of a layer whose contractions take the light form (nothing allocated, the kernel attribute
+    set before the capture)."""
+    os.environ["HDMOE_LIGHT"] = "1"
+    dim = 2048
+    sd, x = small_layer(seed=17, dim=dim, tokens=200, weights="fp8")
+    m = synth.build_module({k: v.to(dev) for k, v in sd.items()}, "fp8", dev, dim=dim)
+    xs = [x.to(dev), (x * 0.5).to(dev), x.flip(1).contiguous().to(dev)]
+    eager = [m(v).clone() for v in xs]
+    torch.cuda.synchronize()
+    static_x = xs[0].clone()
+    side = torch.cuda.Stream()                  # default priority
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        m(static_x)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_y = m(static_x)
+    for rep in range(2):
+        for v, want in zip(xs, eager):
+            static_x.copy_(v)
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(static_y, want)
+            assert torch.equal(m(v), want)      # eager work between replays
+
+
+def test_random_shapes_same_bytes(dev, light_env):
+    """A seeded walk over token counts, widths, expert counts and cast scales."""
+    import random
+    rnd = random.Random(11)
+    for it in range(12):
+        E = rnd.choice([1, 2, 3, 4, 6, 8])
+        D = 128 * rnd.choice([3, 4, 5, 8, 16, 18, 20, 32])
+        H = 128 * rnd.randint(1, 12)
+        T = rnd.choice([1, 7, 33, 100, 257, 511, 1000])
+        s_next = rnd.choice([1.0, 0.5, 0.37, 2.0])
+        base, light = grouped_swiglu(T, D, H, E, seed=900 + it, dev=dev, s_next=s_next)
+        assert torch.equal(base, light), (T, D, H, E, s_next)
