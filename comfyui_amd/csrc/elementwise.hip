@@ -211,6 +211,80 @@ __global__ __launch_bounds__(THREADS) void combine_kernel(const uint4* __restric
   }
 }
 
+// The combine of a layer whose down projection was cut along K: the rows come as fp32 partial sums
+// [nparts][rows_dyn + T][D] (routed rows in expert order, then the shared expert's), and this kernel first does what
+// splitk_reduce_kernel (gemm.hip) does for a row, bf16((sum over the parts in ascending order) * scale of the row's
+// Linear), then what combine_kernel does with the three rows of a token. Same operations in the same order as the two
+// kernels it replaces, so the same bytes; one launch and one bf16 round trip of the rows less.
+struct CombinePartialArgs {
+  const float* partial;
+  long long part_stride;   // floats between two parts
+  int nparts, rows_dyn, n_dyn, fp8, has_shared;
+  const int32_t* offsets;  // segment bounds of the routed rows, n_dyn + 1 entries
+  const float* sw[HDMOE_MAX_EXPERTS + 1];   // scale_weight of the down Linear per expert (fp8); the shared expert is entry n_dyn
+  const float* sin[HDMOE_MAX_EXPERTS + 1];  // its scale_input or NULL
+};
+
+template <class A>
+__global__ __launch_bounds__(THREADS) void combine_partials_kernel(const CombinePartialArgs pa, const int2* __restrict__ inv_perm,
+                                                                   const uint32_t* __restrict__ w, int T, int row16,
+                                                                   CombineExtra ex, uint4* __restrict__ out) {
+  const int lane = threadIdx.x & 63;
+  const int wave = blockIdx.x * WAVES + (threadIdx.x >> 6);
+  const int nwaves = gridDim.x * WAVES;
+  const bool hs = pa.has_shared != 0;
+  const bool hg = ex.gate != nullptr;
+  const int chunks = (row16 + 63) / 64;   // a wave takes 64 x 8 features of one token at a time
+  const int n_out = row16 * 8;
+  auto scale_of = [&](int g) -> float { return pa.fp8 ? (pa.sin[g] ? *pa.sin[g] : 1.0f) * *pa.sw[g] : 1.0f; };
+  auto group_of = [&](int r) {
+    int g = 0;
+    while (g + 1 < pa.n_dyn && r >= pa.offsets[g + 1]) ++g;
+    return g;
+  };
+  // the 8 features of row r at column c, as splitk_reduce_kernel leaves them (values of the 16-bit format)
+  auto row_vals = [&](int r, int c, float sc, float (&v)[8]) {
+    const float* src = pa.partial + (size_t)r * n_out + c;
+    float4 s0 = *reinterpret_cast<const float4*>(src), s1 = *reinterpret_cast<const float4*>(src + 4);
+    for (int p = 1; p < pa.nparts; ++p) {
+      const float* q = src + (size_t)p * (size_t)pa.part_stride;
+      const float4 t0 = *reinterpret_cast<const float4*>(q), t1 = *reinterpret_cast<const float4*>(q + 4);
+      s0.x += t0.x; s0.y += t0.y; s0.z += t0.z; s0.w += t0.w;
+      s1.x += t1.x; s1.y += t1.y; s1.z += t1.z; s1.w += t1.w;
+    }
+    v[0] = A::round(s0.x * sc); v[1] = A::round(s0.y * sc); v[2] = A::round(s0.z * sc); v[3] = A::round(s0.w * sc);
+    v[4] = A::round(s1.x * sc); v[5] = A::round(s1.y * sc); v[6] = A::round(s1.z * sc); v[7] = A::round(s1.w * sc);
+  };
+  const float sc_sh = hs ? scale_of(pa.n_dyn) : 1.0f;
+  for (int unit = wave; unit < T * chunks; unit += nwaves) {
+    const int t = unit / chunks;
+    const int u = (unit - t * chunks) * 64 + lane;
+    if (u >= row16) continue;
+    const int2 r = inv_perm[t];
+    const uint32_t wp = w[t];
+    const float w0 = A::lo(wp), w1 = A::hi(wp);
+    float y0[8], y1[8], sh[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    row_vals(r.x, u * 8, scale_of(group_of(r.x)), y0);
+    row_vals(r.y, u * 8, scale_of(group_of(r.y)), y1);
+    if (hs) row_vals(pa.rows_dyn + t, u * 8, sc_sh, sh);
+    uint4 g = make_uint4(0, 0, 0, 0), res = g;
+    if (hg) {
+      g = ex.gate[(long)(t / ex.tokens_per_batch) * row16 + u];
+      res = ex.residual[(long)t * row16 + u];
+    }
+    auto two = [&](int i, uint32_t gg, uint32_t rr) {
+      return A::pack(comb1<A>(y0[i], y1[i], w0, w1, sh[i], hs, A::lo(gg), A::lo(rr), hg),
+                     comb1<A>(y0[i + 1], y1[i + 1], w0, w1, sh[i + 1], hs, A::hi(gg), A::hi(rr), hg));
+    };
+    uint4 o;
+    o.x = two(0, g.x, res.x);
+    o.y = two(2, g.y, res.y);
+    o.z = two(4, g.z, res.z);
+    o.w = two(6, g.w, res.w);
+    out[(long)t * row16 + u] = o;
+  }
+}
+
 // out[t] = bf16( bf16(gate[b] * y[t]) + residual[t] ), b = t / tokens_per_batch: the gate and residual behind a dense
 // feed-forward (/root/reference/comfy/ldm/hidream/model.py:519-523, text stream).
 __global__ __launch_bounds__(THREADS) void gated_residual_kernel(const uint4* __restrict__ y, const uint4* __restrict__ gate,
@@ -387,6 +461,38 @@ extern "C" int hdmoe_renorm_top2_bf16(const void* topk_weight_bf16, int T, void*
   hipLaunchKernelGGL(renorm_top2_kernel, dim3(blocks), dim3(THREADS), 0, static_cast<hipStream_t>(stream),
                      static_cast<const uint32_t*>(topk_weight_bf16), T, static_cast<uint32_t*>(out_bf16));
   return hdmoe_check_launch("hdmoe_renorm_top2_bf16");
+}
+
+// The combine of a layer over the fp32 partial sums of a down projection cut along K (combine_partials_kernel).
+// experts[e].scale_w2 / scale_in2 and the shared expert's are the scales of the rows (fp8 weights only).
+int hdmoe_launch_combine_partials(const float* partial, long long part_stride, int nparts, int rows_dyn, int n_dyn,
+                                  const int32_t* offsets, bool fp8, const hdmoe_ffn_weights* experts,
+                                  const hdmoe_ffn_weights* shared, const int32_t* inv_perm, const void* topk_weight_bf16,
+                                  const void* gate_bf16, const void* residual_bf16, int tokens_per_batch, int T, int D,
+                                  void* out_bf16, hipStream_t s, const char* what) {
+  if (n_dyn < 0 || n_dyn > HDMOE_MAX_EXPERTS) return hdmoe_fail(HDMOE_E_SHAPE, "%s: %d experts", what, n_dyn);
+  CombinePartialArgs pa;
+  memset(&pa, 0, sizeof(pa));
+  pa.partial = partial;
+  pa.part_stride = part_stride;
+  pa.nparts = nparts;
+  pa.rows_dyn = rows_dyn;
+  pa.n_dyn = n_dyn;
+  pa.fp8 = fp8 ? 1 : 0;
+  pa.has_shared = shared != nullptr ? 1 : 0;
+  pa.offsets = offsets;
+  for (int e = 0; e < n_dyn; ++e) { pa.sw[e] = experts[e].scale_w2; pa.sin[e] = experts[e].scale_in2; }
+  if (shared != nullptr) { pa.sw[n_dyn] = shared->scale_w2; pa.sin[n_dyn] = shared->scale_in2; }
+  CombineExtra ex;
+  ex.gate = static_cast<const uint4*>(gate_bf16);
+  ex.residual = static_cast<const uint4*>(residual_bf16);
+  ex.tokens_per_batch = tokens_per_batch > 0 ? tokens_per_batch : 1;
+  const int row16 = D / 8;
+  const long units = (long)T * ((row16 + 63) / 64);
+  hipLaunchKernelGGL(combine_partials_kernel<HdmoeBf16>, dim3(row_blocks(units)), dim3(THREADS), 0, s, pa,
+                     reinterpret_cast<const int2*>(inv_perm), static_cast<const uint32_t*>(topk_weight_bf16), T, row16, ex,
+                     static_cast<uint4*>(out_bf16));
+  return hdmoe_check_launch(what);
 }
 
 int hdmoe_launch_combine(const void* y_sorted_bf16, const int32_t* inv_perm, const void* topk_weight_bf16,

@@ -1007,7 +1007,7 @@ int hdmoe_launch_ffn_gemm(bool swiglu, int weight_dtype, const uint8_t* a_dyn, c
                           int rows_static, const hdmoe_ffn_weights* shared, uint8_t* out_static, int K_dyn, int N_dyn,
                           int K_static, int N_static, hipStream_t s, const char* what,
                           const int32_t* gather_dyn = nullptr, int gather_rows = 0, float* partial = nullptr,
-                          int nparts = 1, int gather_shift = 0) {
+                          int nparts = 1, int gather_shift = 0, bool reduce = true) {
   const int eb = elem_bytes(weight_dtype);
   const bool fp8 = weight_dtype == HDMOE_W_E4M3FN;
   const int feat_per_tile = swiglu ? BN / 2 : BN;
@@ -1105,6 +1105,7 @@ int hdmoe_launch_ffn_gemm(bool swiglu, int weight_dtype, const uint8_t* a_dyn, c
                    : fp8 ? launch_grouped<FP8_PLAIN>(args, tile_bound, s, what)
                          : launch_grouped<BF16_PLAIN>(args, tile_bound, s, what);
     if (rc != HDMOE_OK) return rc;
+    if (!reduce) return HDMOE_OK;  // the caller's next kernel adds the parts up (hdmoe_launch_combine_partials)
     SplitKReduceArgs ra;
     memset(&ra, 0, sizeof(ra));
     ra.partial = partial;

@@ -9,7 +9,12 @@ int hdmoe_launch_ffn_gemm(bool swiglu, int weight_dtype, const uint8_t* a_dyn, c
                           int rows_static, const hdmoe_ffn_weights* shared, uint8_t* out_static, int K_dyn, int N_dyn,
                           int K_static, int N_static, hipStream_t s, const char* what,
                           const int32_t* gather_dyn = nullptr, int gather_rows = 0, float* partial = nullptr,
-                          int nparts = 1, int gather_shift = 0);
+                          int nparts = 1, int gather_shift = 0, bool reduce = true);
+int hdmoe_launch_combine_partials(const float* partial, long long part_stride, int nparts, int rows_dyn, int n_dyn,
+                                  const int32_t* offsets, bool fp8, const hdmoe_ffn_weights* experts,
+                                  const hdmoe_ffn_weights* shared, const int32_t* inv_perm, const void* topk_weight_bf16,
+                                  const void* gate_bf16, const void* residual_bf16, int tokens_per_batch, int T, int D,
+                                  void* out_bf16, hipStream_t s, const char* what);
 int hdmoe_down_parts(int rows_dyn, int n_dyn, int rows_static, int N, int K_dyn, int K_static, int weight_dtype);
 int hdmoe_check_gemm_shape(const char* what, int weight_dtype, long rows, int K, int N, int feat_per_tile);
 int hdmoe_launch_quant_dispatch(const void* x_bf16, const int32_t* perm, const int32_t* offsets, int T, int D, int E,
@@ -232,12 +237,20 @@ extern "C" int hdmoe_moe_ffn(const hdmoe_layer_args* p, hdmoe_stream_t stream) {
   const int parts = hdmoe_down_parts((int)n, E, Hs > 0 ? T : 0, D, H, Hs, wd);
   if (int rc = hdmoe_launch_ffn_gemm(false, wd, h_routed, offsets, (int)n, E, p->experts, y_routed, h_shared,
                                      Hs > 0 ? T : 0, p->shared, y_shared, H, D, Hs, D, s, "hdmoe_moe_ffn (down)",
-                                     nullptr, 0, parts > 1 ? reinterpret_cast<float*>(ws + l.partials) : nullptr, parts))
+                                     nullptr, 0, parts > 1 ? reinterpret_cast<float*>(ws + l.partials) : nullptr, parts,
+                                     0, /*reduce=*/false))
     return rc;
   mark();
-  const int rc = hdmoe_launch_combine(y_routed, inv_perm, tw, Hs > 0 ? y_shared : nullptr,
+  // cut along K: the combine adds the parts up itself (no launch and no bf16 copy of the rows in between)
+  const int rc = parts > 1
+      ? hdmoe_launch_combine_partials(reinterpret_cast<const float*>(ws + l.partials),
+                                      (long long)(n + (Hs > 0 ? (size_t)T : 0)) * D, parts, (int)n, E, offsets, fp8,
+                                      p->experts, Hs > 0 ? p->shared : nullptr, inv_perm, tw,
                                       fused_block ? p->mod_gate : nullptr, fused_block ? p->x : nullptr,
-                                      fused_block ? p->tokens_per_batch : 1, T, D, p->out, s, "hdmoe_moe_ffn (combine)");
+                                      fused_block ? p->tokens_per_batch : 1, T, D, p->out, s, "hdmoe_moe_ffn (combine)")
+      : hdmoe_launch_combine(y_routed, inv_perm, tw, Hs > 0 ? y_shared : nullptr,
+                             fused_block ? p->mod_gate : nullptr, fused_block ? p->x : nullptr,
+                             fused_block ? p->tokens_per_batch : 1, T, D, p->out, s, "hdmoe_moe_ffn (combine)");
   mark();
   if (rc == HDMOE_OK && ev_err != hipSuccess)
     return hdmoe_fail(HDMOE_E_LAUNCH, "hdmoe_moe_ffn: hipEventRecord on a stage event: %s", hipGetErrorString(ev_err));

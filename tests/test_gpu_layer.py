@@ -346,3 +346,48 @@ def test_random_layers(dev, case):
         sel = torch.unique(torch.cat([torch.randperm(T, generator=g)[:600], torch.arange(T - 64, T), torch.arange(0, 32)]))
     # the fp32-intermediate comparison measures the e4m3 noise of the dataflow itself at these small widths: reported only
     check_layer(sd, x, weights, y, idx, w, E, token_subset=sel, gate_f32=False)
+
+
+@pytest.mark.parametrize("weights,tokens,scale_in", [("fp8", 64, None), ("fp8", 256, 0.5), ("fp8", 700, 0.5), ("bf16", 300, None)])
+def test_combine_over_the_partial_sums_of_a_cut_down_projection(dev, weights, tokens, scale_in):
+    """Small token counts: the down projection is cut along K and the layer's last kernel adds the fp32 partial sums
+    up, scales and rounds the rows and combines them. Its output against the same steps taken apart: torch's fp32
+    adds over the parts left in the workspace (ascending), the row's scale, the rounding to bf16, then the combine
+    kernel (itself bit-exact against the oracle, tests/test_gpu_stages.py): the same bytes."""
+    from comfyui_amd import functional as HF
+    dim = 2048
+    sd, x = small_layer(seed=40 + tokens, dim=dim, tokens=tokens, weights=weights, scale_in=scale_in)
+    m = synth.build_module({k: v.to(dev) for k, v in sd.items()}, weights, dev, dim=dim)
+    x2 = x.to(dev).reshape(-1, dim).contiguous()
+    T, E = x2.shape[0], len(m.experts)
+    wdt, experts, shared, keep = m._collect(x2)
+    H, Hs = m.experts[0].w1.weight.shape[0], m.shared_experts.w1.weight.shape[0]
+    code = HF.weight_dtype_code(wdt)
+    lay = HF.layer_layout(T, dim, H, Hs, E, code)
+    rows = 3 * T
+    parts = (lay.total - lay.partials) // (rows * dim * 4)
+    assert parts > 1, "this size no longer cuts the down projection: pick a smaller one"
+    ws = torch.zeros(lay.total, dtype=torch.uint8, device=dev)
+    out, idx, tw = HF.moe_ffn(x2, m.gate.device_weight(x2), experts, shared, H, Hs, wdt, workspace=ws, want_routing=True,
+                              uniform_scale_in=m._uniform_scale_in)
+    torch.cuda.synchronize()
+    P = ws[lay.partials:lay.partials + parts * rows * dim * 4].view(torch.float32).view(parts, rows, dim)
+    s = P[0].clone()
+    for p in range(1, parts):
+        s += P[p]
+    offsets = ws[lay.offsets:lay.offsets + 4 * (E + 1)].view(torch.int32).cpu().tolist()
+    inv_perm = ws[lay.inv_perm:lay.inv_perm + 8 * T].view(torch.int32)
+    scale = torch.ones(rows, dtype=torch.float32, device=dev)
+    if weights == "fp8":
+        def sc(ffn):
+            s_in = ffn.w2.scale_input
+            one = torch.ones((), dtype=torch.float32, device=dev)
+            return (one if s_in is None else s_in.float().reshape(())) * ffn.w2.scale_weight.float().reshape(())
+        for e in range(E):
+            scale[offsets[e]:offsets[e + 1]] = sc(m.experts[e])
+        scale[2 * T:] = sc(m.shared_experts)
+    y = (s * scale[:, None]).to(torch.bfloat16)
+    want = HF.combine(y[:2 * T].contiguous(), inv_perm, tw, y[2 * T:].contiguous())
+    assert bool(torch.isfinite(out.float()).all()) and float(out.float().abs().max()) > 0
+    assert torch.equal(out.view(torch.int16), want.view(torch.int16))
+    del keep
