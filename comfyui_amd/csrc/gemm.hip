@@ -57,7 +57,8 @@ constexpr int MAX_SLABS = 5;  // 64-row slabs of the largest token tile (arrays 
 template <int TT>
 struct TileCfg {
   static constexpr int BM = 64 * TT;                      // tokens per block tile
-  static constexpr int SMEM = STAGES * (BM + 256) * 128;  // dynamic LDS of a block
+  // dynamic LDS of a block; the 128-token tile (TT = 2) has room for a third stage
+  static constexpr int SMEM = (TT == 2 ? 3 : STAGES) * (BM + 256) * 128;
 };
 constexpr int GROUP_M = 4;     // m-tiles per raster band
 constexpr int NTHREADS = 512;
@@ -229,7 +230,17 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
   constexpr int A_OFF1 = FP8 ? A_BYTES : STAGE_BYTES;
   constexpr int B_OFF0 = FP8 ? 2 * A_BYTES : A_BYTES;
   constexpr int B_OFF1 = FP8 ? 2 * A_BYTES + B_BYTES : STAGE_BYTES + A_BYTES;
+  // RING3 (the light form on the 128-token tile; split K only): three stages [A | B] one after the other, K steps
+  // requested two ahead. With few rows a K step lasts as long as its loads take to arrive, not as long as its MFMAs.
+  constexpr bool RING3 = LIGHT && TT == 2;
+  static_assert(!RING3 || (FP8 && !SWIGLU && !BIAS), "the three-stage ring is built for the fp8 split-K down projection");
+  static_assert(TT != 2 || RING3, "the 128-token tile exists only with the three-stage ring");
+  auto a_off = [](int stage) { return RING3 ? stage * STAGE_BYTES : (stage ? A_OFF1 : 0); };
+  auto b_off = [](int stage) { return RING3 ? stage * STAGE_BYTES + A_BYTES : (stage ? B_OFF1 : B_OFF0); };
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+  if constexpr (RING3) {
+    if (args.nparts <= 1) return;  // its epilogue is the partial-sum store only (kernel argument: uniform)
+  }
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -384,8 +395,8 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
   // requested before the tile becomes current, so the count is never below 1.
   int kt_real = 1;
   auto issue_loads = [&](int stage, int kt) {
-    uint8_t* sa = smem + (stage ? A_OFF1 : 0);
-    uint8_t* sb = smem + (stage ? B_OFF1 : B_OFF0);
+    uint8_t* sa = smem + a_off(stage);
+    uint8_t* sb = smem + b_off(stage);
     const int k0 = k_base + kt * BK;
     const __amdgpu_buffer_rsrc_t empty = make_rsrc(nullptr, 0);
     const bool pad = kt >= kt_real;
@@ -414,8 +425,8 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
   // m-tile of a segment); the others are neither read from LDS nor multiplied.
   [[maybe_unused]] auto compute = [&](int stage, auto full_c, int n_tt) {
     constexpr bool FULL = decltype(full_c)::value;
-    const uint8_t* sa = smem + (stage ? A_OFF1 : 0) + a_base;
-    const uint8_t* sb = smem + (stage ? B_OFF1 : B_OFF0) + b_base;
+    const uint8_t* sa = smem + a_off(stage) + a_base;
+    const uint8_t* sb = smem + b_off(stage) + b_base;
     if constexpr (!FP8) {
 #pragma unroll
       for (int ks = 0; ks < 4; ++ks) {
@@ -822,7 +833,11 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
   for (int j = 0; j < A_SLABS; ++j) gi_nxt[j] = -1;
   load_gather(cur, gi_cur);
   set_src(cur, gi_cur);
+  kt_real = cur.nkt;
   issue_loads(0, 0);
+  if constexpr (RING3) {
+    if (cur.nkt > 1) issue_loads(1, 1);
+  }
   for (int i = 0; cur.g >= 0; ++i) {
     const int KT = cur.nkt;
     kt_real = KT;
@@ -888,8 +903,30 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
         }
       }
     };
+    // Three stages: steps kt and kt + 1 are on their way when step kt is waited for (a wave's loads return in
+    // order: its loads of step kt have landed when at most those of step kt + 1 are outstanding); behind the barrier
+    // everyone has read stage (kt + 2) % 3, which held step kt - 1, and step kt + 2 is requested into it.
+    [[maybe_unused]] auto k_loop3 = [&](auto full_c, int n_tt) {
+      constexpr int PER_STEP = A_SLABS + 4;  // global->LDS loads of a wave per K step
+      auto step = [&](int kt, int stage, int stage_next2) {
+        // wait and barrier as one assembly statement: __syncthreads() carries a fence that waits for every
+        // outstanding global->LDS load, the ones of step kt + 1 included
+        if (kt + 1 < KT) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" : : "n"(PER_STEP) : "memory");
+        else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" : : : "memory");
+        if (kt + 2 < KT) issue_loads(stage_next2, kt + 2);
+        compute(stage, full_c, n_tt);
+      };
+      for (int kt = 0; kt < KT; kt += 3) {
+        step(kt, 0, 2);
+        if (kt + 1 < KT) step(kt + 1, 1, 0);
+        if (kt + 2 < KT) step(kt + 2, 2, 1);
+      }
+    };
     const int my_rows = __builtin_amdgcn_readfirstlane(cur.rows_here) - wt * WAVE_TOK;  // rows of the tile in this wave's half
-    if constexpr (FP8 && !LIGHT) {
+    if constexpr (RING3) {
+      if (my_rows > 32 * (TT - 1)) k_loop3(std::true_type{}, TT);
+      else k_loop3(std::false_type{}, my_rows <= 0 ? 0 : (my_rows + 31) / 32);
+    } else if constexpr (FP8 && !LIGHT) {
       k_loop_fp8();
     } else {
       if (my_rows > 32 * (TT - 1)) k_loop(std::true_type{}, TT);
@@ -900,7 +937,11 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
     __syncthreads();
     if (nxt.g >= 0) {
       set_src(nxt, gi_nxt);
+      kt_real = nxt.nkt;
       issue_loads(0, 0);
+      if constexpr (RING3) {
+        if (nxt.nkt > 1) issue_loads(1, 1);
+      }
     }
     epilogue(cur);
     cur = nxt;
@@ -1101,7 +1142,14 @@ int hdmoe_launch_ffn_gemm(bool swiglu, int weight_dtype, const uint8_t* a_dyn, c
     for (int g = 0; g < G; ++g)
       args.g[g].pout = partial + (args.g[g].row_begin < 0 ? 0 : (size_t)(n_dyn > 0 ? rows_dyn : 0) * N);
     tile_bound *= nparts;
-    const int rc = light ? launch_grouped<FP8_PLAIN, 4, true>(args, tile_bound, s, what)
+    int tb_light = 0;  // the light form cut along K runs on 128-token tiles with a three-stage ring
+    if (light) {
+      constexpr int BM2 = TileCfg<2>::BM;
+      if (n_dyn > 0) tb_light += (rows_dyn / BM2 + n_dyn) * (N_dyn / feat_per_tile);
+      if (shared != nullptr && rows_static > 0) tb_light += ((rows_static + BM2 - 1) / BM2) * (N_static / feat_per_tile);
+      tb_light *= nparts;
+    }
+    const int rc = light ? launch_grouped<FP8_PLAIN, 2, true>(args, tb_light, s, what)
                    : fp8 ? launch_grouped<FP8_PLAIN>(args, tile_bound, s, what)
                          : launch_grouped<BF16_PLAIN>(args, tile_bound, s, what);
     if (rc != HDMOE_OK) return rc;
@@ -1164,6 +1212,32 @@ int hdmoe_launch_ffn_gemm(bool swiglu, int weight_dtype, const uint8_t* a_dyn, c
 // sizes, about 10 TB/s; one step is about 1.4 us).
 int hdmoe_down_parts(int rows_dyn, int n_dyn, int rows_static, int N, int K_dyn, int K_static, int weight_dtype) {
   const int eb = elem_bytes(weight_dtype);
+  // fp8 with few rows per segment (the rule of the light form in hdmoe_launch_ffn_gemm): the launch runs on 128-token
+  // tiles with K steps requested two ahead, and is bound by how fast the weights arrive, not by its K loops. About 150
+  // blocks keep enough loads in flight; more parts only add partial sums. The routing is not known here and the
+  // mean segment sits near the tile height, so segments are taken 1.5 times the mean: an expert that needs a second
+  // m-tile must not push the launch into a second round of blocks. (Whole layer, uniform / skewed routing, 256
+  // tokens: 2 parts 99 / 102 us, 3 parts 95 / 110 us; 128 tokens: 2 parts 88, 3 parts 81, 5 parts 96 us.)
+  if (weight_dtype == HDMOE_W_E4M3FN && (n_dyn <= 0 || rows_dyn <= 128 * n_dyn) && rows_static <= 256) {
+    const int bm2 = TileCfg<2>::BM;
+    long t2 = 0;
+    int kt2 = 0;
+    if (n_dyn > 0 && rows_dyn > 0) {
+      const long seg = ((long)rows_dyn * 3 / 2 + n_dyn - 1) / n_dyn;
+      t2 += (long)n_dyn * ((seg + bm2 - 1) / bm2) * (N / BN);
+      kt2 = K_dyn * eb / BK;
+    }
+    if (rows_static > 0) {
+      t2 += (long)((rows_static + bm2 - 1) / bm2) * (N / BN);
+      if (K_static * eb / BK > kt2) kt2 = K_static * eb / BK;
+    }
+    if (t2 <= 0 || kt2 <= 0) return 1;
+    long parts = (150 + t2 - 1) / t2;
+    if (parts > HDMOE_NUM_CU / t2) parts = HDMOE_NUM_CU / t2;
+    if (parts > 6) parts = 6;
+    while (parts > 1 && kt2 / parts < 6) --parts;
+    return parts < 1 ? 1 : (int)parts;
+  }
   const int bm = TileCfg<4>::BM;
   double tiles = 0;
   int kt = 0;
