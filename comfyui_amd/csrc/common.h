@@ -50,3 +50,27 @@ size_t hdmoe_gate_hist_bytes(int T, int E);
 
 constexpr int HDMOE_NUM_CU = 256;   // MI355X
 constexpr int HDMOE_NUM_XCD = 8;
+
+// ---- K cuts of a down projection (split K) ---------------------------------------------------------------------
+// The host does not know the routing, and whether a cut pays depends on how many tiles the experts' segments really
+// make: a cut whose tiles fit one round of blocks beats every other, one tile more and it needs a second round. So the
+// host lists candidate cuts (most parts first, each expected to fit under favourable routing) and a last entry that is
+// taken when none fits; the GEMM kernel and the kernel that adds the parts up both evaluate hdmoe_plan_pick on the
+// segment bounds the dispatch left on the device, and so agree without the host ever seeing them.
+constexpr int HDMOE_PLAN_MAX = 12;
+struct HdmoeSplitPlan {
+  int n;                     // entries in use; 1 = a fixed cut
+  int pd[HDMOE_PLAN_MAX];    // K parts of a tile of the experts' groups
+  int ps[HDMOE_PLAN_MAX];    // K parts of a tile of the static group (the shared expert)
+  int bm;                    // tile height (tokens) the launch runs with
+  int max_tiles;             // an entry before the last is taken only if its tiles number at most this
+};
+
+// mt_dyn / mt_static: m-tiles (tile height plan.bm) of all experts' segments / of the static group; ntiles_n: tiles
+// along the output features. Returns the index of the entry to run.
+__host__ __device__ inline int hdmoe_plan_pick(const HdmoeSplitPlan& plan, int mt_dyn, int mt_static, int ntiles_n) {
+  for (int i = 0; i + 1 < plan.n; ++i)
+    if ((mt_dyn * plan.pd[i] + mt_static * plan.ps[i]) * ntiles_n <= plan.max_tiles) return i;
+  return plan.n - 1;
+}
+

@@ -219,7 +219,8 @@ __global__ __launch_bounds__(THREADS) void combine_kernel(const uint4* __restric
 struct CombinePartialArgs {
   const float* partial;
   long long part_stride;   // floats between two parts
-  int nparts, rows_dyn, n_dyn, fp8, has_shared;
+  HdmoeSplitPlan plan;     // the candidate cuts of the down projection; the entry that ran is chosen as its kernel chose
+  int rows_dyn, n_dyn, fp8, has_shared;
   const int32_t* offsets;  // segment bounds of the routed rows, n_dyn + 1 entries
   const float* sw[HDMOE_MAX_EXPERTS + 1];   // scale_weight of the down Linear per expert (fp8); the shared expert is entry n_dyn
   const float* sin[HDMOE_MAX_EXPERTS + 1];  // its scale_input or NULL
@@ -243,10 +244,10 @@ __global__ __launch_bounds__(THREADS) void combine_partials_kernel(const Combine
     return g;
   };
   // the 8 features of row r at column c, as splitk_reduce_kernel leaves them (values of the 16-bit format)
-  auto row_vals = [&](int r, int c, float sc, float (&v)[8]) {
+  auto row_vals = [&](int r, int c, float sc, int nparts, float (&v)[8]) {
     const float* src = pa.partial + (size_t)r * n_out + c;
     float4 s0 = *reinterpret_cast<const float4*>(src), s1 = *reinterpret_cast<const float4*>(src + 4);
-    for (int p = 1; p < pa.nparts; ++p) {
+    for (int p = 1; p < nparts; ++p) {
       const float* q = src + (size_t)p * (size_t)pa.part_stride;
       const float4 t0 = *reinterpret_cast<const float4*>(q), t1 = *reinterpret_cast<const float4*>(q + 4);
       s0.x += t0.x; s0.y += t0.y; s0.z += t0.z; s0.w += t0.w;
@@ -256,6 +257,19 @@ __global__ __launch_bounds__(THREADS) void combine_partials_kernel(const Combine
     v[4] = A::round(s1.x * sc); v[5] = A::round(s1.y * sc); v[6] = A::round(s1.z * sc); v[7] = A::round(s1.w * sc);
   };
   const float sc_sh = hs ? scale_of(pa.n_dyn) : 1.0f;
+  // which cut the down projection ran with (the same function of the segment bounds as in its kernel)
+  int nparts = pa.plan.pd[0], nparts_static = pa.plan.ps[0];
+  if (pa.plan.n > 1) {
+    // the bounds as one vector load (at most 17 entries), then lane reads
+    const int off_lane = lane <= pa.n_dyn ? pa.offsets[lane] : 0;
+    int mt_dyn = 0;
+    for (int e = 0; e < pa.n_dyn; ++e)
+      mt_dyn += (__builtin_amdgcn_readlane(off_lane, e + 1) - __builtin_amdgcn_readlane(off_lane, e) + pa.plan.bm - 1) / pa.plan.bm;
+    const int mt_static = hs ? (T + pa.plan.bm - 1) / pa.plan.bm : 0;
+    const int idx = hdmoe_plan_pick(pa.plan, mt_dyn, mt_static, n_out / 256);
+    nparts = pa.plan.pd[idx];
+    nparts_static = pa.plan.ps[idx];
+  }
   for (int unit = wave; unit < T * chunks; unit += nwaves) {
     const int t = unit / chunks;
     const int u = (unit - t * chunks) * 64 + lane;
@@ -264,9 +278,9 @@ __global__ __launch_bounds__(THREADS) void combine_partials_kernel(const Combine
     const uint32_t wp = w[t];
     const float w0 = A::lo(wp), w1 = A::hi(wp);
     float y0[8], y1[8], sh[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-    row_vals(r.x, u * 8, scale_of(group_of(r.x)), y0);
-    row_vals(r.y, u * 8, scale_of(group_of(r.y)), y1);
-    if (hs) row_vals(pa.rows_dyn + t, u * 8, sc_sh, sh);
+    row_vals(r.x, u * 8, scale_of(group_of(r.x)), nparts, y0);
+    row_vals(r.y, u * 8, scale_of(group_of(r.y)), nparts, y1);
+    if (hs) row_vals(pa.rows_dyn + t, u * 8, sc_sh, nparts_static, sh);
     uint4 g = make_uint4(0, 0, 0, 0), res = g;
     if (hg) {
       g = ex.gate[(long)(t / ex.tokens_per_batch) * row16 + u];
@@ -465,7 +479,8 @@ extern "C" int hdmoe_renorm_top2_bf16(const void* topk_weight_bf16, int T, void*
 
 // The combine of a layer over the fp32 partial sums of a down projection cut along K (combine_partials_kernel).
 // experts[e].scale_w2 / scale_in2 and the shared expert's are the scales of the rows (fp8 weights only).
-int hdmoe_launch_combine_partials(const float* partial, long long part_stride, int nparts, int rows_dyn, int n_dyn,
+int hdmoe_launch_combine_partials(const float* partial, long long part_stride, const HdmoeSplitPlan& plan,
+                                  int rows_dyn, int n_dyn,
                                   const int32_t* offsets, bool fp8, const hdmoe_ffn_weights* experts,
                                   const hdmoe_ffn_weights* shared, const int32_t* inv_perm, const void* topk_weight_bf16,
                                   const void* gate_bf16, const void* residual_bf16, int tokens_per_batch, int T, int D,
@@ -475,7 +490,8 @@ int hdmoe_launch_combine_partials(const float* partial, long long part_stride, i
   memset(&pa, 0, sizeof(pa));
   pa.partial = partial;
   pa.part_stride = part_stride;
-  pa.nparts = nparts;
+  if (plan.n < 1 || plan.n > HDMOE_PLAN_MAX) return hdmoe_fail(HDMOE_E_SHAPE, "%s: split plan with %d entries", what, plan.n);
+  pa.plan = plan;
   pa.rows_dyn = rows_dyn;
   pa.n_dyn = n_dyn;
   pa.fp8 = fp8 ? 1 : 0;

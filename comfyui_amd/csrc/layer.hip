@@ -9,13 +9,16 @@ int hdmoe_launch_ffn_gemm(bool swiglu, int weight_dtype, const uint8_t* a_dyn, c
                           int rows_static, const hdmoe_ffn_weights* shared, uint8_t* out_static, int K_dyn, int N_dyn,
                           int K_static, int N_static, hipStream_t s, const char* what,
                           const int32_t* gather_dyn = nullptr, int gather_rows = 0, float* partial = nullptr,
-                          int nparts = 1, int gather_shift = 0, bool reduce = true);
-int hdmoe_launch_combine_partials(const float* partial, long long part_stride, int nparts, int rows_dyn, int n_dyn,
+                          int nparts = 1, int gather_shift = 0, bool reduce = true,
+                          const HdmoeSplitPlan* plan = nullptr);
+int hdmoe_launch_combine_partials(const float* partial, long long part_stride, const HdmoeSplitPlan& plan,
+                                  int rows_dyn, int n_dyn,
                                   const int32_t* offsets, bool fp8, const hdmoe_ffn_weights* experts,
                                   const hdmoe_ffn_weights* shared, const int32_t* inv_perm, const void* topk_weight_bf16,
                                   const void* gate_bf16, const void* residual_bf16, int tokens_per_batch, int T, int D,
                                   void* out_bf16, hipStream_t s, const char* what);
-int hdmoe_down_parts(int rows_dyn, int n_dyn, int rows_static, int N, int K_dyn, int K_static, int weight_dtype);
+int hdmoe_down_parts(int rows_dyn, int n_dyn, int rows_static, int N, int K_dyn, int K_static, int weight_dtype,
+                     HdmoeSplitPlan* plan = nullptr);
 int hdmoe_check_gemm_shape(const char* what, int weight_dtype, long rows, int K, int N, int feat_per_tile);
 int hdmoe_launch_quant_dispatch(const void* x_bf16, const int32_t* perm, const int32_t* offsets, int T, int D, int E,
                                 const float* const* scale_input, const float* shared_scale, bool with_shared,
@@ -234,17 +237,18 @@ extern "C" int hdmoe_moe_ffn(const hdmoe_layer_args* p, hdmoe_stream_t stream) {
     return rc;
   mark();
   // down projections, both in one launch
-  const int parts = hdmoe_down_parts((int)n, E, Hs > 0 ? T : 0, D, H, Hs, wd);
+  HdmoeSplitPlan plan;  // candidate cuts; the kernels pick one by the real segment sizes
+  const int parts = hdmoe_down_parts((int)n, E, Hs > 0 ? T : 0, D, H, Hs, wd, &plan);
   if (int rc = hdmoe_launch_ffn_gemm(false, wd, h_routed, offsets, (int)n, E, p->experts, y_routed, h_shared,
                                      Hs > 0 ? T : 0, p->shared, y_shared, H, D, Hs, D, s, "hdmoe_moe_ffn (down)",
                                      nullptr, 0, parts > 1 ? reinterpret_cast<float*>(ws + l.partials) : nullptr, parts,
-                                     0, /*reduce=*/false))
+                                     0, /*reduce=*/false, &plan))
     return rc;
   mark();
   // cut along K: the combine adds the parts up itself (no launch and no bf16 copy of the rows in between)
   const int rc = parts > 1
       ? hdmoe_launch_combine_partials(reinterpret_cast<const float*>(ws + l.partials),
-                                      (long long)(n + (Hs > 0 ? (size_t)T : 0)) * D, parts, (int)n, E, offsets, fp8,
+                                      (long long)(n + (Hs > 0 ? (size_t)T : 0)) * D, plan, (int)n, E, offsets, fp8,
                                       p->experts, Hs > 0 ? p->shared : nullptr, inv_perm, tw,
                                       fused_block ? p->mod_gate : nullptr, fused_block ? p->x : nullptr,
                                       fused_block ? p->tokens_per_batch : 1, T, D, p->out, s, "hdmoe_moe_ffn (combine)")
