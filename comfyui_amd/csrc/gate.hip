@@ -511,13 +511,14 @@ extern "C" int hdmoe_gate_top2_f16(const void* x_f16, const void* gate_w_f16, in
 }
 
 // Tokens per block of the gate kernels, a pure function of T: the grid is three blocks per CU, all resident at once
-// (the register kernels hold 12 waves per CU), unless that leaves a block fewer than two tokens per wave to pay for
-// its copy of the gate weight into LDS; very large T gets more blocks instead of more than 1024 tokens each (the
+// (the register kernels hold 12 waves per CU), with at least one token per wave (a few hundred tokens then spread over
+// more blocks: 2 us off the 256-token gate against two tokens per wave, nothing lost at 4096 tokens, where a block
+// holds 6 tokens instead of 8); very large T gets more blocks instead of more than 1024 tokens each (the
 // dispatch's scatter pass handles one or several whole blocks per chunk, at most 1024 tokens).
 int hdmoe_gate_tokens_per_block(int T) {
   const int resident = HDMOE_NUM_CU * 3;
   int tpb = (T + resident - 1) / resident;
-  if (tpb < WAVES_PER_BLOCK * 2) tpb = WAVES_PER_BLOCK * 2;
+  if (tpb < WAVES_PER_BLOCK) tpb = WAVES_PER_BLOCK;
   if (tpb > 1024) tpb = 1024;
   return tpb;
 }
