@@ -91,7 +91,7 @@ def make_config(name, seed=0):
         return dict(name=name, master=master, weights="fp8", x=make_input(g, 4096))
     if name == "cfg3":      # fp8 weights, 2 x 4096 tokens, 1% outlier channels x20  (headline)
         return dict(name=name, master=master, weights="fp8", x=make_input(g, 8192, batch=2, outlier_frac=0.01))
-    if name in ("cfg5-256", "cfg5-4096"):
+    if name.startswith("cfg5-") and name[5:].isdigit():   # cfg5-256 and cfg5-4096 are the benchmark lines
         tokens = int(name.split("-")[1])
         x = make_input(g, tokens)
         master, x = apply_routing_skew(master, x)

@@ -145,7 +145,9 @@ def test_composed_path_matches_fused(dev):
     assert diff["rel_rms"] < 2e-3
 
 
-@pytest.mark.parametrize("name", ["cfg1", "cfg2", "cfg3", "cfg5-256", "cfg5-4096"])
+# cfg5-1024 is not a benchmark line: it is the size where the cut of the down projection is chosen on the device, with
+# a routing (one expert nearly empty, one heavy) under which no candidate cut fits one round of blocks
+@pytest.mark.parametrize("name", ["cfg1", "cfg2", "cfg3", "cfg5-256", "cfg5-1024", "cfg5-4096"])
 def test_benchmark_configs(dev, name):
     """The benchmark configurations at their full size: EVERY token of the output is compared with the oracle (an
     unwritten or misplaced output tile anywhere would show), routing and permutation bit-exact on every token."""
