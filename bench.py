@@ -41,7 +41,7 @@ def gate_up_kernel_name(T, H, Hs, E, cus=256, fp8=True):
     kernel; with one tile per segment and the experts' half empty on average, in the form of the 8-wave kernel that
     skips the token blocks without rows)."""
     if fp8 and 2 * T <= 128 * E and T <= 256:
-        return "grouped_gemm_kernel<FP8_SWIGLU, 4, LIGHT>"
+        return "grouped_gemm_kernel<FP8_SWIGLU, %d, LIGHT>" % (2 if (T <= 128 and 2 * T <= 64 * E) else 4)
     def cost(tt):
         bm = 64 * tt
         tiles = E * (-(-(2 * T // E) // bm)) * (H // 128) + (-(-T // bm)) * (Hs // 128)

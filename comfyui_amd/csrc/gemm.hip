@@ -235,13 +235,13 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
   // RING3 (the light form on the 128-token tile; split K only): three stages [A | B] one after the other, K steps
   // requested two ahead. With few rows a K step lasts as long as its loads take to arrive, not as long as its MFMAs.
   constexpr bool RING3 = LIGHT && TT == 2;
-  static_assert(!RING3 || (FP8 && !SWIGLU && !BIAS), "the three-stage ring is built for the fp8 split-K down projection");
+  static_assert(!RING3 || (FP8 && !BIAS), "the three-stage ring is built for the fp8 feed-forward contractions");
   static_assert(TT != 2 || RING3, "the 128-token tile exists only with the three-stage ring");
   auto a_off = [](int stage) { return RING3 ? stage * STAGE_BYTES : (stage ? A_OFF1 : 0); };
   auto b_off = [](int stage) { return RING3 ? stage * STAGE_BYTES + A_BYTES : (stage ? B_OFF1 : B_OFF0); };
   extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
-  if constexpr (RING3) {
-    if (args.nparts <= 1) return;  // its epilogue is the partial-sum store only (kernel argument: uniform)
+  if constexpr (RING3 && !SWIGLU) {
+    if (args.nparts <= 1) return;  // its plain epilogue is the partial-sum store only (kernel argument: uniform)
   }
 
   const int tid = threadIdx.x;
@@ -606,7 +606,8 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
   // Staging room for the outputs once the K loop is over: whatever is not stage 0 (which takes the next tile's
   // first K step meanwhile). fp8: the token tile of stage 1 (BM x 128 bytes: exactly the SwiGLU tile) and the
   // weight tile of stage 1; bf16: stage 1 as a whole.
-  uint8_t* const stg = smem + (FP8 ? A_OFF1 : STAGE_BYTES);
+  // (three-stage ring: the token tile of stage 2; the next tile's first two K steps go to stages 0 and 1 meanwhile)
+  uint8_t* const stg = smem + (RING3 ? 2 * STAGE_BYTES : FP8 ? A_OFF1 : STAGE_BYTES);
   auto wave_sync = [] {
     // orders this wave's LDS writes before its LDS reads of other lanes' data (LDS executes a wave's requests
     // in order; this only stops the compiler from moving them)
@@ -1232,6 +1233,16 @@ int hdmoe_launch_ffn_gemm(bool swiglu, int weight_dtype, const uint8_t* a_dyn, c
   // The 4-wave form of the gate/up kernel (swiglu4w.h) has the 256-token tile; it takes the launch whenever the
   // 8-wave kernel would not use its 320-token tile (2-3 % faster there: part of its epilogue hides in the K loop).
   // HDMOE_SWIGLU4W in the environment overrides: "0" = never, anything else = whenever the shapes allow.
+  // Light form, gate/up: with every segment inside one 128-token tile (up to 128 tokens in a top-2 layer of 4 experts)
+  // the three-stage ring of the down projection pays here too (whole layer 78 -> 73 us at 16 tokens, 80 -> 75 at 128;
+  // at 256 tokens the shared expert's second m-tile costs more than the ring gains: 93 -> 105 us).
+  if (light && swiglu && rows_static <= TileCfg<2>::BM && (n_dyn <= 0 || rows_dyn <= TileCfg<2>::BM / 2 * n_dyn)) {
+    constexpr int BM2 = TileCfg<2>::BM;
+    int tb = 0;
+    if (n_dyn > 0) tb += (rows_dyn / BM2 + n_dyn) * (N_dyn / feat_per_tile);
+    if (shared != nullptr && rows_static > 0) tb += ((rows_static + BM2 - 1) / BM2) * (N_static / feat_per_tile);
+    return launch_grouped<FP8_SWIGLU, 2, true>(args, tb, s, what);
+  }
   if (light) return swiglu ? launch_grouped<FP8_SWIGLU, 4, true>(args, tile_bound, s, what)
                            : launch_grouped<FP8_PLAIN, 4, true>(args, tile_bound, s, what);
   const bool want4w = env4w != nullptr ? env4w[0] != '0' : !tall;
