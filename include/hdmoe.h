@@ -47,7 +47,7 @@
 extern "C" {
 #endif
 
-#define HDMOE_VERSION 112
+#define HDMOE_VERSION 113
 
 #define HDMOE_OK 0
 #define HDMOE_E_NULL (-1)      /* required pointer is NULL */
