@@ -235,7 +235,7 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
   // RING3 (the light form on the 128-token tile; split K only): three stages [A | B] one after the other, K steps
   // requested two ahead. With few rows a K step lasts as long as its loads take to arrive, not as long as its MFMAs.
   constexpr bool RING3 = LIGHT && TT == 2;
-  static_assert(!RING3 || (FP8 && !BIAS), "the three-stage ring is built for the fp8 feed-forward contractions");
+  static_assert(!RING3 || !BIAS, "the three-stage ring is built for the feed-forward contractions");
   static_assert(TT != 2 || RING3, "the 128-token tile exists only with the three-stage ring");
   auto a_off = [](int stage) { return RING3 ? stage * STAGE_BYTES : (stage ? A_OFF1 : 0); };
   auto b_off = [](int stage) { return RING3 ? stage * STAGE_BYTES + A_BYTES : (stage ? B_OFF1 : B_OFF0); };
@@ -1094,6 +1094,9 @@ int hdmoe_launch_ffn_gemm(bool swiglu, int weight_dtype, const uint8_t* a_dyn, c
   const char* const env4w = getenv("HDMOE_SWIGLU4W");  // forcing the 4-wave kernel also keeps the default off
   const bool light = fp8 && (env_light != nullptr ? env_light[0] != '0'
                                                   : few_rows && !(swiglu && env4w != nullptr && env4w[0] != '0'));
+  // 16-bit weights: their K loop skips empty token blocks anyway; what the small sizes take from the light form is the
+  // three-stage ring on 128-token tiles (HDMOE_LIGHT=0 keeps it off here too)
+  const bool ring16 = !fp8 && few_rows && !(env_light != nullptr && env_light[0] == '0');
   // (bf16: the gate/up kernel only; the down projection measured slower on the taller tile)
   const bool tall = (fp8 || swiglu) && !split && !light && expected_cost(5) < expected_cost(4);
   const int BM = tall ? TileCfg<5>::BM : TileCfg<4>::BM;  // tokens per block tile of the kernel that will run
@@ -1173,7 +1176,7 @@ int hdmoe_launch_ffn_gemm(bool swiglu, int weight_dtype, const uint8_t* a_dyn, c
     } else {
       args.plan.n = 1;
       args.plan.pd[0] = args.plan.ps[0] = nparts;
-      args.plan.bm = light ? BM2 : BM;
+      args.plan.bm = (light || ring16) ? BM2 : BM;
       args.plan.max_tiles = HDMOE_NUM_CU;
     }
     if (reduce && args.plan.n > 1) {  // splitk_reduce_kernel takes a fixed cut: the plan's last entry
@@ -1191,7 +1194,7 @@ int hdmoe_launch_ffn_gemm(bool swiglu, int weight_dtype, const uint8_t* a_dyn, c
     for (int i = 0; i < args.plan.n; ++i) {
       const int tb = tb_dyn * args.plan.pd[i] + tb_static * args.plan.ps[i];
       if (tb > tile_bound) tile_bound = tb;
-      if (light) {
+      if (light || ring16) {
         int tl = 0;
         if (n_dyn > 0) tl += (rows_dyn / BM2 + n_dyn) * (N_dyn / feat_per_tile) * args.plan.pd[i];
         if (shared != nullptr && rows_static > 0)
@@ -1200,6 +1203,7 @@ int hdmoe_launch_ffn_gemm(bool swiglu, int weight_dtype, const uint8_t* a_dyn, c
       }
     }
     const int rc = light ? launch_grouped<FP8_PLAIN, 2, true>(args, tb_light, s, what)
+                   : ring16 ? launch_grouped<BF16_PLAIN, 2, true>(args, tb_light, s, what)
                    : fp8 ? launch_grouped<FP8_PLAIN>(args, tile_bound, s, what)
                          : launch_grouped<BF16_PLAIN>(args, tile_bound, s, what);
     if (rc != HDMOE_OK) return rc;
@@ -1236,12 +1240,14 @@ int hdmoe_launch_ffn_gemm(bool swiglu, int weight_dtype, const uint8_t* a_dyn, c
   // Light form, gate/up: with every segment inside one 128-token tile (up to 128 tokens in a top-2 layer of 4 experts)
   // the three-stage ring of the down projection pays here too (whole layer 78 -> 73 us at 16 tokens, 80 -> 75 at 128;
   // at 256 tokens the shared expert's second m-tile costs more than the ring gains: 93 -> 105 us).
-  if (light && swiglu && rows_static <= TileCfg<2>::BM && (n_dyn <= 0 || rows_dyn <= TileCfg<2>::BM / 2 * n_dyn)) {
+  if ((light || ring16) && swiglu && rows_static <= TileCfg<2>::BM &&
+      (n_dyn <= 0 || rows_dyn <= TileCfg<2>::BM / 2 * n_dyn)) {
     constexpr int BM2 = TileCfg<2>::BM;
     int tb = 0;
     if (n_dyn > 0) tb += (rows_dyn / BM2 + n_dyn) * (N_dyn / feat_per_tile);
     if (shared != nullptr && rows_static > 0) tb += ((rows_static + BM2 - 1) / BM2) * (N_static / feat_per_tile);
-    return launch_grouped<FP8_SWIGLU, 2, true>(args, tb, s, what);
+    return fp8 ? launch_grouped<FP8_SWIGLU, 2, true>(args, tb, s, what)
+               : launch_grouped<BF16_SWIGLU, 2, true>(args, tb, s, what);
   }
   if (light) return swiglu ? launch_grouped<FP8_SWIGLU, 4, true>(args, tile_bound, s, what)
                            : launch_grouped<FP8_PLAIN, 4, true>(args, tile_bound, s, what);
@@ -1291,13 +1297,13 @@ int hdmoe_down_parts(int rows_dyn, int n_dyn, int rows_static, int N, int K_dyn,
   const int ktd = dyn ? K_dyn * eb / BK : 0, kts = rows_static > 0 ? K_static * eb / BK : 0;
   if ((!dyn && rows_static <= 0) || nt <= 0 || (ktd <= 0 && kts <= 0)) return fixed(1);
 
-  // fp8 with few rows per segment (the rule of the light form in hdmoe_launch_ffn_gemm): the launch runs on 128-token
+  // Few rows per segment (the rule of the light form in hdmoe_launch_ffn_gemm): the launch runs on 128-token
   // tiles with K steps requested two ahead, and is bound by how fast the weights arrive, not by its K loops. About 150
   // blocks keep enough loads in flight; more parts only add partial sums. The mean segment sits near the tile height,
   // so segments are counted 1.5 times the mean: an expert that needs a second m-tile must not push the launch into a
   // second round of blocks. (Whole layer, uniform / skewed routing, 256 tokens: 2 parts 99 / 102 us, 3 parts 95 / 110
   // us; 128 tokens: 2 parts 88, 3 parts 81, 5 parts 96 us.)
-  if (weight_dtype == HDMOE_W_E4M3FN && (n_dyn <= 0 || rows_dyn <= 128 * n_dyn) && rows_static <= 256) {
+  if ((n_dyn <= 0 || rows_dyn <= 128 * n_dyn) && rows_static <= 256) {
     const int bm2 = TileCfg<2>::BM;
     pl.bm = bm2;
     long t2 = 0;

@@ -28,7 +28,8 @@
  *     HDMOE_LIGHT: the 8-wave kernels (gate/up and down) have a form whose K loop skips the 32-token blocks of a tile
  *     that hold no rows. Unset: it runs when every segment is one tile and the experts' tiles are half empty on
  *     average (rows per expert <= 128 and shared rows <= 256: up to 256 tokens for HiDream's sizes; 3-12 % faster
- *     there, slower above). "0": never. Anything else: always;
+ *     there, slower above). "0": never (also keeps 16-bit weights off the three-stage kernels those sizes take).
+ *     Anything else: always (fp8);
  *   - return value 0 = enqueued; negative = HDMOE_E_* and nothing was enqueued;
  *     hdmoe_last_error() gives a thread-local message for the last failure;
  *   - scale pointers (float*, device) address the fp32 scalar Parameters

@@ -164,3 +164,22 @@ def test_random_shapes_same_bytes(dev, light_env):
         s_next = rnd.choice([1.0, 0.5, 0.37, 2.0])
         base, light = grouped_swiglu(T, D, H, E, seed=900 + it, dev=dev, s_next=s_next)
         assert torch.equal(base, light), (T, D, H, E, s_next)
+
+
+@pytest.mark.parametrize("tokens", [1, 64, 128, 200, 256])
+def test_bf16_layer_on_the_three_stage_ring(dev, light_env, tokens):
+    """bf16 weights at small token counts: gate/up (up to 128 tokens) and the down projection cut along K run on
+    128-token tiles with K steps requested two ahead; HDMOE_LIGHT=0 keeps them on the two-stage 256-token tiles. Same
+    bytes, and within the oracle's bound."""
+    dim = 2048
+    sd, x = small_layer(seed=500 + tokens, dim=dim, tokens=tokens, weights="bf16")
+    m = synth.build_module({k: v.to(dev) for k, v in sd.items()}, "bf16", dev, dim=dim)
+    os.environ["HDMOE_LIGHT"] = "0"
+    base = m(x.to(dev)).cpu()
+    os.environ.pop("HDMOE_LIGHT")
+    ring = m(x.to(dev)).cpu()
+    assert torch.equal(base.view(torch.int16), ring.view(torch.int16))
+    idx, w, _, _ = O.gate_fixed_order(x.reshape(-1, dim), sd["gate.weight"])
+    ref = O.moe_forward(x, oracle_params(sd, 4), "plain", gate_result=(idx, w))
+    d = O.error_metrics(ring, ref)
+    assert d["rel_rms"] <= 5e-3, d
