@@ -40,8 +40,12 @@ def gate_up_kernel_name(T, H, Hs, E, cus=256, fp8=True):
     kernel when they do not add a round of tiles to the persistent blocks, else 256-token tiles (fp8: in the 4-wave
     kernel; with one tile per segment and the experts' half empty on average, in the form of the 8-wave kernel that
     skips the token blocks without rows)."""
-    if fp8 and 2 * T <= 128 * E and T <= 256:
-        return "grouped_gemm_kernel<FP8_SWIGLU, %d, LIGHT>" % (2 if (T <= 128 and 2 * T <= 64 * E) else 4)
+    if 2 * T <= 128 * E and T <= 256:
+        ring = T <= 128 and 2 * T <= 64 * E      # every segment inside one 128-token tile: the three-stage form
+        if fp8:
+            return "grouped_gemm_kernel<FP8_SWIGLU, %d, LIGHT>" % (2 if ring else 4)
+        if ring:
+            return "grouped_gemm_kernel<BF16_SWIGLU, 2, LIGHT>"
     def cost(tt):
         bm = 64 * tt
         tiles = E * (-(-(2 * T // E) // bm)) * (H // 128) + (-(-T // bm)) * (Hs // 128)
