@@ -34,25 +34,11 @@ PEAK_HBM_GBPS = 8000.0      # MI355X HBM3E
 
 
 
-def gate_up_kernel_name(T, H, Hs, E, cus=256, fp8=True):
-    """Which kernel the library's launcher runs for the gate/up contraction of a layer (the rule of
-    hdmoe_launch_ffn_gemm in comfyui_amd/csrc/gemm.hip, with HDMOE_SWIGLU4W unset): 320-token tiles in the 8-wave
-    kernel when they do not add a round of tiles to the persistent blocks, else 256-token tiles (fp8: in the 4-wave
-    kernel; with one tile per segment and the experts' half empty on average, in the form of the 8-wave kernel that
-    skips the token blocks without rows)."""
-    if 2 * T <= 128 * E and T <= 256:
-        ring = T <= 128 and 2 * T <= 64 * E      # every segment inside one 128-token tile: the three-stage form
-        if fp8:
-            return "grouped_gemm_kernel<FP8_SWIGLU, %d, LIGHT>" % (2 if ring else 4)
-        if ring:
-            return "grouped_gemm_kernel<BF16_SWIGLU, 2, LIGHT>"
-    def cost(tt):
-        bm = 64 * tt
-        tiles = E * (-(-(2 * T // E) // bm)) * (H // 128) + (-(-T // bm)) * (Hs // 128)
-        return -(-tiles // cus) * (tt + 1)
-    if not fp8:
-        return "grouped_gemm_kernel<BF16_SWIGLU, %d>" % (5 if cost(5) < cost(4) else 4)
-    return "grouped_gemm_kernel<FP8_SWIGLU, 5>" if cost(5) < cost(4) else "swiglu4w_kernel"
+def gate_up_kernel_name(T, D, H, Hs, E, fp8=True):
+    """Which kernel the library's launcher runs for the gate/up contraction of a layer: asked of the library itself
+    (hdmoe_gate_up_kernel_name evaluates the launcher's rule under the current form switches)."""
+    from comfyui_amd import _lib
+    return _lib.lib.hdmoe_gate_up_kernel_name(_lib.W_E4M3FN if fp8 else _lib.W_BF16, T, E, D, H, Hs, 1).decode()
 
 
 def measured_traffic(workload):
@@ -394,7 +380,7 @@ def main():
         "stage_ms": stage_ms,
         "gemm_down_tflops": gemm2_tflops,
         "roofline": {
-            "kernel": gate_up_kernel_name(T, H, Hs, E, fp8=fp8),
+            "kernel": gate_up_kernel_name(T, D, H, Hs, E, fp8=fp8),
             "bound": "mfma",
             "achieved": gemm1_tflops,
             "peak": peak,

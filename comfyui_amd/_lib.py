@@ -24,6 +24,8 @@ MAX_EXPERTS = 16
 E_NULL, E_SHAPE, E_WORKSPACE, E_LAUNCH = -1, -2, -3, -4
 TOPK = 2
 NUM_STAGES = 6
+FORM_SWIGLU4W, FORM_LIGHT = 0, 1
+FORM_AUTO, FORM_NEVER, FORM_ALWAYS = -1, 0, 1
 STAGE_NAMES = ("gate", "dispatch", "quant_permute", "gemm_gate_up", "gemm_down", "combine")
 
 c_void_p = ctypes.c_void_p
@@ -72,6 +74,9 @@ class LayerLayout(ctypes.Structure):
 SIGNATURES = {
     "hdmoe_version": (c_int, []),
     "hdmoe_last_error": (ctypes.c_char_p, []),
+    "hdmoe_set_kernel_form": (c_int, [c_int, c_int]),
+    "hdmoe_get_kernel_form": (c_int, [c_int]),
+    "hdmoe_gate_up_kernel_name": (ctypes.c_char_p, [c_int, c_int, c_int, c_int, c_int, c_int, c_int]),
     "hdmoe_gate_top2": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),
     "hdmoe_gate_top2_f16": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),
     "hdmoe_renorm_top2_bf16": (c_int, [c_void_p, c_int, c_void_p, c_void_p]),
@@ -144,6 +149,11 @@ def check(rc):
     """Raise HdmoeError for a negative return code of an entry point."""
     if rc != 0:
         raise HdmoeError(rc, lib.hdmoe_last_error().decode("utf-8", "replace"))
+
+
+def set_kernel_form(which, value):
+    """hdmoe_set_kernel_form: FORM_SWIGLU4W / FORM_LIGHT to FORM_AUTO / FORM_NEVER / FORM_ALWAYS."""
+    check(lib.hdmoe_set_kernel_form(which, value))
 
 
 def ptr(t):

@@ -48,6 +48,14 @@ static inline size_t hdmoe_align_up(size_t v, size_t a) { return (v + a - 1) / a
 int hdmoe_gate_tokens_per_block(int T);
 size_t hdmoe_gate_hist_bytes(int T, int E);
 
+// Few rows per segment: one m-tile per group and the experts' 256-token tiles half empty on average (up to 256 tokens
+// in a top-2 layer of 4 experts). Such launches run in the forms of the GEMM kernels that skip padding, and their down
+// projection is cut along K for 128-token tiles. One rule for the launcher and for the K cut (which depends on the
+// sizes only, never on the form switches, so that every form of a kernel adds up the same parts in the same order).
+static inline bool hdmoe_few_rows(int rows_dyn, int n_dyn, int rows_static) {
+  return (n_dyn <= 0 || rows_dyn <= 128 * n_dyn) && rows_static <= 256;
+}
+
 constexpr int HDMOE_NUM_CU = 256;   // MI355X
 constexpr int HDMOE_NUM_XCD = 8;
 

@@ -31,8 +31,10 @@
 // from its index and exits if its index is past the real tile count. Block ids are
 // remapped so that each XCD (ids congruent mod 8) walks a contiguous range of tiles,
 // 4 m-tiles deep, and its L2 sees each operand tile reused by neighbouring blocks.
+#include <atomic>
 #include <cmath>
 #include <cstdlib>
+#include <mutex>
 #include <type_traits>
 
 #include "common.h"
@@ -1059,6 +1061,98 @@ int check_dtype(int weight_dtype, const char* what) {
 
 }  // namespace
 
+// ---- which kernel runs a feed-forward contraction ---------------------------------------------------------------
+// Two process-wide switches choose between kernels with the same results bit for bit (hdmoe_set_kernel_form). Their
+// initial values come from the environment variables HDMOE_SWIGLU4W / HDMOE_LIGHT, read once ("0" = never, anything
+// else = always, unset = the launcher's own rule).
+namespace {
+std::atomic<int> g_form[HDMOE_NUM_FORMS] = {{HDMOE_FORM_AUTO}, {HDMOE_FORM_AUTO}};
+std::once_flag g_form_once;
+void form_init() {
+  static const char* const names[HDMOE_NUM_FORMS] = {"HDMOE_SWIGLU4W", "HDMOE_LIGHT"};
+  for (int i = 0; i < HDMOE_NUM_FORMS; ++i) {
+    const char* v = getenv(names[i]);
+    if (v != nullptr) g_form[i].store(v[0] == '0' ? HDMOE_FORM_NEVER : HDMOE_FORM_ALWAYS, std::memory_order_relaxed);
+  }
+}
+int form_of(int which) {
+  std::call_once(g_form_once, form_init);
+  return g_form[which].load(std::memory_order_relaxed);
+}
+
+// The kernels a contraction of the feed-forward can run on.
+enum GemmForm {
+  FORM_SPLIT_K,    // plain modes cut along K (few tiles); its own choice of tile inside
+  FORM_RING3,      // 128-token tiles, three LDS stages, token blocks without rows skipped
+  FORM_LIGHT4,     // 256-token tiles, token blocks without rows skipped
+  FORM_W4,         // fp8 gate/up: the 4-wave kernel (256-token tiles)
+  FORM_TALL5,      // 320-token tiles
+  FORM_BASE4       // 256-token tiles
+};
+
+struct GemmShape {
+  bool swiglu, fp8, split;
+  int rows_dyn, n_dyn, rows_static;  // rows_static = 0: no static group
+  int N_dyn, N_static;
+  bool w4_fits;                      // the 4-wave kernel takes these operands (swiglu4w_fits)
+};
+
+// Expected tiles with evenly loaded experts, static round-robin over the CUs, and a fixed cost per tile of about one
+// 32-token block: rounds x (TT + 1). The taller tile wins when it does not add a round.
+long expected_tile_cost(const GemmShape& sh, int tt) {
+  const int bm = 64 * tt, fpt = sh.swiglu ? BN / 2 : BN;
+  long tiles = 0;
+  if (sh.n_dyn > 0) tiles += (long)sh.n_dyn * ((sh.rows_dyn / sh.n_dyn + bm - 1) / bm) * (sh.N_dyn / fpt);
+  if (sh.rows_static > 0) tiles += (long)((sh.rows_static + bm - 1) / bm) * (sh.N_static / fpt);
+  return ((tiles + HDMOE_NUM_CU - 1) / HDMOE_NUM_CU) * (tt + 1);
+}
+
+// light: the token blocks of a tile that hold no rows are skipped (fp8: the compiler-scheduled K loop instead of the
+// assembly loop, which multiplies padding like rows; 16-bit weights always skip them and take from this only the
+// three-stage ring).
+struct FormChoice { GemmForm form; bool light, ring16, tall; };
+FormChoice pick_form(const GemmShape& sh) {
+  const int f_light = form_of(HDMOE_FORM_LIGHT), f_4w = form_of(HDMOE_FORM_SWIGLU4W);
+  const bool few_rows = hdmoe_few_rows(sh.rows_dyn, sh.n_dyn, sh.rows_static);
+  FormChoice c;
+  // forcing the 4-wave kernel also keeps the light form's default off
+  c.light = sh.fp8 && (f_light != HDMOE_FORM_AUTO ? f_light == HDMOE_FORM_ALWAYS
+                                                   : few_rows && !(sh.swiglu && f_4w == HDMOE_FORM_ALWAYS));
+  c.ring16 = !sh.fp8 && few_rows && f_light != HDMOE_FORM_NEVER;
+  // (bf16: the gate/up kernel only; the down projection measured slower on the taller tile)
+  c.tall = (sh.fp8 || sh.swiglu) && !sh.split && !c.light && expected_tile_cost(sh, 5) < expected_tile_cost(sh, 4);
+  if (sh.split) { c.form = FORM_SPLIT_K; return c; }
+  // Light form, gate/up: with every segment inside one 128-token tile (up to 128 tokens in a top-2 layer of 4 experts)
+  // the three-stage ring of the down projection pays here too (whole layer 78 -> 73 us at 16 tokens, 80 -> 75 at 128;
+  // at 256 tokens the shared expert's second m-tile costs more than the ring gains: 93 -> 105 us).
+  if ((c.light || c.ring16) && sh.swiglu && sh.rows_static <= TileCfg<2>::BM &&
+      (sh.n_dyn <= 0 || sh.rows_dyn <= TileCfg<2>::BM / 2 * sh.n_dyn)) {
+    c.form = FORM_RING3;
+    return c;
+  }
+  if (c.light) { c.form = FORM_LIGHT4; return c; }
+  // The 4-wave form of the gate/up kernel (swiglu4w.h) has the 256-token tile; it takes the launch whenever the
+  // 8-wave kernel would not use its 320-token tile (2-3 % faster there: part of its epilogue hides in the K loop).
+  const bool want4w = f_4w != HDMOE_FORM_AUTO ? f_4w == HDMOE_FORM_ALWAYS : !c.tall;
+  if (sh.fp8 && sh.swiglu && want4w && sh.w4_fits) { c.form = FORM_W4; return c; }
+  c.form = c.tall ? FORM_TALL5 : FORM_BASE4;
+  return c;
+}
+}  // namespace
+
+extern "C" int hdmoe_set_kernel_form(int which, int value) {
+  if (which < 0 || which >= HDMOE_NUM_FORMS || value < HDMOE_FORM_AUTO || value > HDMOE_FORM_ALWAYS)
+    return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_set_kernel_form: which=%d value=%d", which, value);
+  std::call_once(g_form_once, form_init);
+  g_form[which].store(value, std::memory_order_relaxed);
+  return HDMOE_OK;
+}
+
+extern "C" int hdmoe_get_kernel_form(int which) {
+  if (which < 0 || which >= HDMOE_NUM_FORMS) return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_get_kernel_form: which=%d", which);
+  return form_of(which);
+}
+
 // Shared by hdmoe_grouped_swiglu / hdmoe_grouped_down / hdmoe_linear / hdmoe_moe_ffn.
 // groups: n_dyn experts with device-side segments, optionally one static group (the shared expert).
 // gather_dyn (optional): the routed rows are not materialised in segment order; row r of the segments is row
@@ -1073,32 +1167,16 @@ int hdmoe_launch_ffn_gemm(bool swiglu, int weight_dtype, const uint8_t* a_dyn, c
   const int eb = elem_bytes(weight_dtype);
   const bool fp8 = weight_dtype == HDMOE_W_E4M3FN;
   const int feat_per_tile = swiglu ? BN / 2 : BN;
-  // Tile height. Expected tiles with evenly loaded experts, static round-robin over the CUs, and a fixed cost per tile
-  // of about one 32-token block: rounds x (TT + 1). The taller tile wins when it does not add a round.
-  auto expected_cost = [&](int tt) {
-    const int bm = 64 * tt;
-    long tiles = 0;
-    if (n_dyn > 0) tiles += (long)n_dyn * ((rows_dyn / n_dyn + bm - 1) / bm) * (N_dyn / feat_per_tile);
-    if (shared != nullptr && rows_static > 0) tiles += (long)((rows_static + bm - 1) / bm) * (N_static / feat_per_tile);
-    return ((tiles + HDMOE_NUM_CU - 1) / HDMOE_NUM_CU) * (tt + 1);
-  };
   // Split K (runs on the 256-token tile, or the 128-token one of the light form): nparts = the most parts any entry of
   // the plan cuts a tile into (the partial-sum buffer holds that many); no plan = every tile in nparts parts
   const bool split = !swiglu && partial != nullptr && nparts > 1;
-  // Few rows per segment (one m-tile per group, the experts' half empty on average: up to 256 tokens in a top-2
-  // layer of 4 experts): most of every 256-token tile is padding, and the launch runs in the form of the kernel that
-  // skips it (whole layer 12 % faster at 16 tokens, 3 % at 256, 2-15 % slower from 320 tokens on). HDMOE_LIGHT in the
-  // environment overrides: "0" = never, anything else = always (fp8).
-  const char* const env_light = getenv("HDMOE_LIGHT");
-  const bool few_rows = (n_dyn <= 0 || rows_dyn <= 128 * n_dyn) && (shared == nullptr || rows_static <= 256);
-  const char* const env4w = getenv("HDMOE_SWIGLU4W");  // forcing the 4-wave kernel also keeps the default off
-  const bool light = fp8 && (env_light != nullptr ? env_light[0] != '0'
-                                                  : few_rows && !(swiglu && env4w != nullptr && env4w[0] != '0'));
-  // 16-bit weights: their K loop skips empty token blocks anyway; what the small sizes take from the light form is the
-  // three-stage ring on 128-token tiles (HDMOE_LIGHT=0 keeps it off here too)
-  const bool ring16 = !fp8 && few_rows && !(env_light != nullptr && env_light[0] == '0');
-  // (bf16: the gate/up kernel only; the down projection measured slower on the taller tile)
-  const bool tall = (fp8 || swiglu) && !split && !light && expected_cost(5) < expected_cost(4);
+  GemmShape shape;
+  shape.swiglu = swiglu; shape.fp8 = fp8; shape.split = split;
+  shape.rows_dyn = rows_dyn; shape.n_dyn = n_dyn; shape.rows_static = shared != nullptr ? rows_static : 0;
+  shape.N_dyn = N_dyn; shape.N_static = N_static;
+  shape.w4_fits = true;  // settled below, once the groups are filled in
+  FormChoice choice = pick_form(shape);
+  const bool light = choice.light, ring16 = choice.ring16, tall = choice.tall;
   const int BM = tall ? TileCfg<5>::BM : TileCfg<4>::BM;  // tokens per block tile of the kernel that will run
   if (gather_dyn != nullptr && (unsigned long long)gather_rows * K_dyn * eb >= (1ull << 31))
     return hdmoe_fail(HDMOE_E_SHAPE, "%s: %d gathered rows of %d bytes exceed the 2 GiB offset range", what, gather_rows,
@@ -1234,41 +1312,63 @@ int hdmoe_launch_ffn_gemm(bool swiglu, int weight_dtype, const uint8_t* a_dyn, c
     hipLaunchKernelGGL(splitk_reduce_kernel, dim3(blocks), dim3(256), 0, s, ra);
     return hdmoe_check_launch(what);
   }
-  // The 4-wave form of the gate/up kernel (swiglu4w.h) has the 256-token tile; it takes the launch whenever the
-  // 8-wave kernel would not use its 320-token tile (2-3 % faster there: part of its epilogue hides in the K loop).
-  // HDMOE_SWIGLU4W in the environment overrides: "0" = never, anything else = whenever the shapes allow.
-  // Light form, gate/up: with every segment inside one 128-token tile (up to 128 tokens in a top-2 layer of 4 experts)
-  // the three-stage ring of the down projection pays here too (whole layer 78 -> 73 us at 16 tokens, 80 -> 75 at 128;
-  // at 256 tokens the shared expert's second m-tile costs more than the ring gains: 93 -> 105 us).
-  if ((light || ring16) && swiglu && rows_static <= TileCfg<2>::BM &&
-      (n_dyn <= 0 || rows_dyn <= TileCfg<2>::BM / 2 * n_dyn)) {
-    constexpr int BM2 = TileCfg<2>::BM;
-    int tb = 0;
-    if (n_dyn > 0) tb += (rows_dyn / BM2 + n_dyn) * (N_dyn / feat_per_tile);
-    if (shared != nullptr && rows_static > 0) tb += ((rows_static + BM2 - 1) / BM2) * (N_static / feat_per_tile);
-    return fp8 ? launch_grouped<FP8_SWIGLU, 2, true>(args, tb, s, what)
-               : launch_grouped<BF16_SWIGLU, 2, true>(args, tb, s, what);
-  }
-  if (light) return swiglu ? launch_grouped<FP8_SWIGLU, 4, true>(args, tile_bound, s, what)
-                           : launch_grouped<FP8_PLAIN, 4, true>(args, tile_bound, s, what);
-  const bool want4w = env4w != nullptr ? env4w[0] != '0' : !tall;
-  if (fp8 && swiglu && want4w) {
+  if (fp8 && swiglu) {
     long long op_bytes = (long long)(gather_dyn != nullptr ? gather_rows : rows_dyn) * K_dyn;
     if ((long long)rows_static * K_static > op_bytes) op_bytes = (long long)rows_static * K_static;
-    if (swiglu4w_fits(args, op_bytes)) {
+    shape.w4_fits = swiglu4w_fits(args, op_bytes);
+    choice = pick_form(shape);
+  }
+  switch (choice.form) {
+    case FORM_RING3: {
+      constexpr int BM2 = TileCfg<2>::BM;
+      int tb = 0;
+      if (n_dyn > 0) tb += (rows_dyn / BM2 + n_dyn) * (N_dyn / feat_per_tile);
+      if (shared != nullptr && rows_static > 0) tb += ((rows_static + BM2 - 1) / BM2) * (N_static / feat_per_tile);
+      return fp8 ? launch_grouped<FP8_SWIGLU, 2, true>(args, tb, s, what)
+                 : launch_grouped<BF16_SWIGLU, 2, true>(args, tb, s, what);
+    }
+    case FORM_LIGHT4:
+      return swiglu ? launch_grouped<FP8_SWIGLU, 4, true>(args, tile_bound, s, what)
+                    : launch_grouped<FP8_PLAIN, 4, true>(args, tile_bound, s, what);
+    case FORM_W4: {
       int tb = 0;
       if (n_dyn > 0) tb += (rows_dyn / W4_BM + n_dyn) * (N_dyn / W4_FEAT);
       if (shared != nullptr && rows_static > 0) tb += ((rows_static + W4_BM - 1) / W4_BM) * (N_static / W4_FEAT);
       return launch_swiglu4w(args, tb, s, what);
     }
+    case FORM_TALL5:
+      if (fp8) return swiglu ? launch_grouped<FP8_SWIGLU, 5>(args, tile_bound, s, what)
+                             : launch_grouped<FP8_PLAIN, 5>(args, tile_bound, s, what);
+      return launch_grouped<BF16_SWIGLU, 5>(args, tile_bound, s, what);
+    default:
+      break;
   }
-  if (fp8 && tall) return swiglu ? launch_grouped<FP8_SWIGLU, 5>(args, tile_bound, s, what)
-                                 : launch_grouped<FP8_PLAIN, 5>(args, tile_bound, s, what);
   if (fp8) return swiglu ? launch_grouped<FP8_SWIGLU>(args, tile_bound, s, what)
                          : launch_grouped<FP8_PLAIN>(args, tile_bound, s, what);
-  if (tall) return launch_grouped<BF16_SWIGLU, 5>(args, tile_bound, s, what);
   return swiglu ? launch_grouped<BF16_SWIGLU>(args, tile_bound, s, what)
                 : launch_grouped<BF16_PLAIN>(args, tile_bound, s, what);
+}
+
+// Name of the kernel the gate/up contraction of a layer runs on (T tokens, E routed experts top-2 plus a shared expert
+// if Hs > 0), by the launcher's own rule and the current form switches: for reports that name the dominant kernel.
+extern "C" const char* hdmoe_gate_up_kernel_name(int weight_dtype, int T, int E, int D, int H, int Hs,
+                                                 int has_scale_in2) {
+  if (check_dtype(weight_dtype, "hdmoe_gate_up_kernel_name") != HDMOE_OK || T <= 0 || E < 0 || D <= 0 || H <= 0)
+    return "";
+  GemmShape sh;
+  sh.swiglu = true; sh.fp8 = weight_dtype == HDMOE_W_E4M3FN; sh.split = false;
+  sh.rows_dyn = E > 0 ? T * HDMOE_TOPK : 0; sh.n_dyn = E; sh.rows_static = Hs > 0 ? T : 0;
+  sh.N_dyn = H; sh.N_static = Hs;
+  const int kb = D * elem_bytes(weight_dtype);
+  sh.w4_fits = sh.fp8 && has_scale_in2 != 0 && kb % (2 * BK) == 0 && kb >= 16 * BK && H % W4_FEAT == 0 &&
+               (Hs <= 0 || Hs % W4_FEAT == 0) && (long long)T * kb < (1ll << 31);
+  switch (pick_form(sh).form) {
+    case FORM_RING3: return sh.fp8 ? "grouped_gemm_kernel<FP8_SWIGLU, 2, LIGHT>" : "grouped_gemm_kernel<BF16_SWIGLU, 2, LIGHT>";
+    case FORM_LIGHT4: return "grouped_gemm_kernel<FP8_SWIGLU, 4, LIGHT>";
+    case FORM_W4: return "swiglu4w_kernel";
+    case FORM_TALL5: return sh.fp8 ? "grouped_gemm_kernel<FP8_SWIGLU, 5>" : "grouped_gemm_kernel<BF16_SWIGLU, 5>";
+    default: return sh.fp8 ? "grouped_gemm_kernel<FP8_SWIGLU, 4>" : "grouped_gemm_kernel<BF16_SWIGLU, 4>";
+  }
 }
 
 // How the down projection of a layer is cut along K: a pure function of the sizes, so that the workspace layout and
@@ -1303,7 +1403,7 @@ int hdmoe_down_parts(int rows_dyn, int n_dyn, int rows_static, int N, int K_dyn,
   // so segments are counted 1.5 times the mean: an expert that needs a second m-tile must not push the launch into a
   // second round of blocks. (Whole layer, uniform / skewed routing, 256 tokens: 2 parts 99 / 102 us, 3 parts 95 / 110
   // us; 128 tokens: 2 parts 88, 3 parts 81, 5 parts 96 us.)
-  if ((n_dyn <= 0 || rows_dyn <= 128 * n_dyn) && rows_static <= 256) {
+  if (hdmoe_few_rows(rows_dyn, n_dyn, rows_static)) {
     const int bm2 = TileCfg<2>::BM;
     pl.bm = bm2;
     long t2 = 0;

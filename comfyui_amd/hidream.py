@@ -115,6 +115,11 @@ def _pack_key(ffns, dev):
                 return None
             if (sw is not None and sw.device != dev) or (si is not None and si.device != dev):
                 return None
+            # the cached structures hold raw addresses of the module's own tensors: a weight that has to be made
+            # contiguous, or a scale that is not an fp32 scalar in place, is packed from a temporary every call
+            if not w.is_contiguous() or any(t is not None and (t.dtype != torch.float32 or not t.is_contiguous())
+                                            for t in (sw, si)):
+                return None
             key.append((type(l), l.training, w.data_ptr(), w.dtype, b is None, getattr(l, "hdmoe_fp8_matrix_mult", None),
                         None if sw is None else (sw.data_ptr(), sw._version),
                         None if si is None else (si.data_ptr(), si._version)))

@@ -18,18 +18,8 @@
  *   - the only state the library keeps between calls: the thread-local error message, and per device one flag per
  *     GEMM kernel variant recording that hipFuncSetAttribute (the opt-in for more than 64 KiB of dynamic LDS) has
  *     been called for it on that device, plus the device address of the built-in buffer of hdmoe_dispatch_static;
- *   - two environment variables are read, at every call that runs an fp8 feed-forward contraction. Both choose
- *     between kernels with the same results bit for bit.
- *     HDMOE_SWIGLU4W: the gate/up contraction has an 8-wave kernel (256- or 320-token tiles) and a 4-wave one (one
- *     wave per SIMD, 256-token tiles, a tile's SiLU*mul epilogue issued between the MFMAs of the next tile; needs K a
- *     multiple of 256 and at least 2048, and scale_in2). Unset: the 4-wave kernel runs where the 320-token tile would
- *     not be used (up to about 5000 tokens for HiDream's sizes; it is 2-3 % faster there and 1-2 % slower above).
- *     "0": never. Anything else: whenever the shapes allow.
- *     HDMOE_LIGHT: the 8-wave kernels (gate/up and down) have a form whose K loop skips the 32-token blocks of a tile
- *     that hold no rows. Unset: it runs when every segment is one tile and the experts' tiles are half empty on
- *     average (rows per expert <= 128 and shared rows <= 256: up to 256 tokens for HiDream's sizes; 3-12 % faster
- *     there, slower above). "0": never (also keeps 16-bit weights off the three-stage kernels those sizes take).
- *     Anything else: always (fp8);
+ *   - two process-wide switches choose between kernels with the same results bit for bit (hdmoe_set_kernel_form
+ *     below); they start from the environment variables HDMOE_SWIGLU4W / HDMOE_LIGHT, read once at first use;
  *   - return value 0 = enqueued; negative = HDMOE_E_* and nothing was enqueued;
  *     hdmoe_last_error() gives a thread-local message for the last failure;
  *   - scale pointers (float*, device) address the fp32 scalar Parameters
@@ -48,7 +38,7 @@
 extern "C" {
 #endif
 
-#define HDMOE_VERSION 113
+#define HDMOE_VERSION 114
 
 #define HDMOE_OK 0
 #define HDMOE_E_NULL (-1)      /* required pointer is NULL */
@@ -69,6 +59,35 @@ typedef void* hdmoe_stream_t;
 
 int hdmoe_version(void);
 const char* hdmoe_last_error(void);
+
+/* Kernel-form switches. No counterpart in the reference: both choose between kernels of this library whose results are
+ * the same bit for bit, for tests that compare the forms and for measurements. Process-wide; a call in flight on
+ * another thread sees the old or the new value. A HIP graph keeps the kernels that were captured.
+ *   HDMOE_FORM_SWIGLU4W: the fp8 gate/up contraction has an 8-wave kernel (256- or 320-token tiles) and a 4-wave one
+ *     (one wave per SIMD, 256-token tiles, a tile's SiLU*mul epilogue issued between the MFMAs of the next tile; needs
+ *     K a multiple of 256 and at least 2048, and scale_in2). AUTO: the 4-wave kernel runs where the 320-token tile
+ *     would not be used (up to about 5000 tokens for HiDream's sizes; it is 2-3 % faster there and 1-2 % slower
+ *     above). NEVER / ALWAYS (whenever the shapes allow).
+ *   HDMOE_FORM_LIGHT: the 8-wave kernels (gate/up and down) have a form whose K loop skips the 32-token blocks of a
+ *     tile that hold no rows. AUTO: it runs when every segment is one tile and the experts' tiles are half empty on
+ *     average (rows per expert <= 128 and shared rows <= 256: up to 256 tokens for HiDream's sizes; 3-12 % faster
+ *     there, slower above). NEVER (also keeps 16-bit weights off the three-stage kernels those sizes take) / ALWAYS
+ *     (fp8).
+ * Initial values: the environment variables HDMOE_SWIGLU4W / HDMOE_LIGHT, read once ("0" = NEVER, anything else =
+ * ALWAYS, unset = AUTO). hdmoe_get_kernel_form returns the current value. */
+#define HDMOE_FORM_SWIGLU4W 0
+#define HDMOE_FORM_LIGHT 1
+#define HDMOE_NUM_FORMS 2
+#define HDMOE_FORM_AUTO (-1)
+#define HDMOE_FORM_NEVER 0
+#define HDMOE_FORM_ALWAYS 1
+int hdmoe_set_kernel_form(int which, int value);
+int hdmoe_get_kernel_form(int which);
+
+/* Name of the kernel that the gate/up contraction of a whole layer (T tokens, E routed experts top-2, shared expert
+ * if Hs > 0; has_scale_in2: the w2 Linears carry a scale_input) runs on under the current switches, for reports that
+ * name the dominant kernel; "" for sizes the layer does not take. No counterpart in the reference. */
+const char* hdmoe_gate_up_kernel_name(int weight_dtype, int T, int E, int D, int H, int Hs, int has_scale_in2);
 
 /* ---- stage entry points ------------------------------------------------------ */
 

@@ -1,14 +1,12 @@
 """The fp8 contractions of launches with few rows per segment run in the form of the tile kernel whose K loop skips
-the 32-token blocks without rows (csrc/gemm.hip, LIGHT; HDMOE_LIGHT in the environment forces it on or off). Same MFMA,
+the 32-token blocks without rows (csrc/gemm.hip, LIGHT; hdmoe_set_kernel_form forces it on or off). Same MFMA,
 same operand layout, same order over K and same epilogue as the assembly loop, so the same bytes out."""
-import os
-
 import pytest
 import torch
 
 from comfyui_amd import synth
 from oracle import hidream_moe_oracle as O
-from tests.helpers import oracle_params, small_layer
+from tests.helpers import oracle_params, saved_forms, set_form, small_layer
 
 pytestmark = pytest.mark.gpu
 BF16 = torch.bfloat16
@@ -16,13 +14,7 @@ BF16 = torch.bfloat16
 
 @pytest.fixture
 def light_env():
-    old = {k: os.environ.get(k) for k in ("HDMOE_LIGHT", "HDMOE_SWIGLU4W")}
-    yield
-    for k, v in old.items():
-        if v is None:
-            os.environ.pop(k, None)
-        else:
-            os.environ[k] = v
+    yield from saved_forms()
 
 
 def grouped_swiglu(T, D, H, E, seed, dev, s_next):
@@ -52,9 +44,9 @@ def grouped_swiglu(T, D, H, E, seed, dev, s_next):
         return f
     arr = (_lib.FfnWeights * E)(*[weights(w) for w in ws])
     out = []
-    os.environ["HDMOE_SWIGLU4W"] = "0"
+    set_form("HDMOE_SWIGLU4W", "0")
     for form in ("0", "1"):
-        os.environ["HDMOE_LIGHT"] = form
+        set_form("HDMOE_LIGHT", form)
         h = torch.full((2 * T, H), 0x55, dtype=torch.uint8, device=dev)
         _lib.check(_lib.lib.hdmoe_grouped_swiglu(_lib.W_E4M3FN, xs.data_ptr(), offsets.data_ptr(), 2 * T, E, D, H, arr,
                                                  h.data_ptr(), None))
@@ -88,10 +80,10 @@ def test_layer_through_the_light_form(dev, light_env, tokens, scale_in):
     dim = 2048
     sd, x = small_layer(seed=300 + tokens, dim=dim, tokens=tokens, weights="fp8", scale_in=scale_in)
     m = synth.build_module({k: v.to(dev) for k, v in sd.items()}, "fp8", dev, dim=dim)
-    os.environ["HDMOE_SWIGLU4W"] = "0"
-    os.environ["HDMOE_LIGHT"] = "0"
+    set_form("HDMOE_SWIGLU4W", "0")
+    set_form("HDMOE_LIGHT", "0")
     base = m(x.to(dev)).cpu()
-    os.environ["HDMOE_LIGHT"] = "1"
+    set_form("HDMOE_LIGHT", "1")
     light = m(x.to(dev)).cpu()
     assert torch.equal(base.view(torch.int16), light.view(torch.int16))
     idx, w, _, _ = O.gate_fixed_order(x.reshape(-1, dim), sd["gate.weight"])
@@ -116,9 +108,9 @@ def test_dense_feed_forward_through_both_kernels(dev, light_env):
             lin.scale_input.fill_(0.5)
     for shape in ((1, 77, dim), (2, 450, dim)):
         x = torch.randn(shape, generator=g).to(BF16).to(dev)
-        os.environ["HDMOE_LIGHT"] = "0"
+        set_form("HDMOE_LIGHT", "0")
         base = ff(x).cpu()
-        os.environ["HDMOE_LIGHT"] = "1"
+        set_form("HDMOE_LIGHT", "1")
         light = ff(x).cpu()
         assert bool(torch.isfinite(base.float()).all()) and float(base.float().abs().max()) > 0
         assert torch.equal(base.view(torch.int16), light.view(torch.int16))
@@ -127,7 +119,7 @@ def test_dense_feed_forward_through_both_kernels(dev, light_env):
 def test_layer_with_the_light_form_in_a_graph(dev, light_env):
     """Capture and replay of a layer whose contractions take the light form (nothing allocated, the kernel attribute
     set before the capture)."""
-    os.environ["HDMOE_LIGHT"] = "1"
+    set_form("HDMOE_LIGHT", "1")
     dim = 2048
     sd, x = small_layer(seed=17, dim=dim, tokens=200, weights="fp8")
     m = synth.build_module({k: v.to(dev) for k, v in sd.items()}, "fp8", dev, dim=dim)
@@ -174,9 +166,9 @@ def test_bf16_layer_on_the_three_stage_ring(dev, light_env, tokens):
     dim = 2048
     sd, x = small_layer(seed=500 + tokens, dim=dim, tokens=tokens, weights="bf16")
     m = synth.build_module({k: v.to(dev) for k, v in sd.items()}, "bf16", dev, dim=dim)
-    os.environ["HDMOE_LIGHT"] = "0"
+    set_form("HDMOE_LIGHT", "0")
     base = m(x.to(dev)).cpu()
-    os.environ.pop("HDMOE_LIGHT")
+    set_form("HDMOE_LIGHT", None)
     ring = m(x.to(dev)).cpu()
     assert torch.equal(base.view(torch.int16), ring.view(torch.int16))
     idx, w, _, _ = O.gate_fixed_order(x.reshape(-1, dim), sd["gate.weight"])

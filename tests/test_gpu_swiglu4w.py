@@ -1,13 +1,11 @@
-"""The two kernels of the fp8 gate/up contraction (8 waves: csrc/gemm.hip; 4 waves: csrc/swiglu4w.h; HDMOE_SWIGLU4W in
-the environment forces one or the other): same contraction and rounding points, so the same bytes out."""
-import os
-
+"""The two kernels of the fp8 gate/up contraction (8 waves: csrc/gemm.hip; 4 waves: csrc/swiglu4w.h; hdmoe_set_kernel_form
+forces one or the other): same contraction and rounding points, so the same bytes out."""
 import pytest
 import torch
 
 from comfyui_amd import synth
 from oracle import hidream_moe_oracle as O
-from tests.helpers import oracle_params, small_layer
+from tests.helpers import oracle_params, saved_forms, set_form, small_layer
 
 pytestmark = pytest.mark.gpu
 BF16 = torch.bfloat16
@@ -15,12 +13,7 @@ BF16 = torch.bfloat16
 
 @pytest.fixture
 def four_wave():
-    old = os.environ.get("HDMOE_SWIGLU4W")
-    yield
-    if old is None:
-        os.environ.pop("HDMOE_SWIGLU4W", None)
-    else:
-        os.environ["HDMOE_SWIGLU4W"] = old
+    yield from saved_forms()
 
 
 def grouped_swiglu(T, D, H, E, seed, dev, s_next):
@@ -51,7 +44,7 @@ def grouped_swiglu(T, D, H, E, seed, dev, s_next):
     arr = (_lib.FfnWeights * E)(*[weights(w) for w in ws])
     out = []
     for form in ("0", "1"):
-        os.environ["HDMOE_SWIGLU4W"] = form
+        set_form("HDMOE_SWIGLU4W", form)
         h = torch.full((2 * T, H), 0x55, dtype=torch.uint8, device=dev)
         _lib.check(_lib.lib.hdmoe_grouped_swiglu(_lib.W_E4M3FN, xs.data_ptr(), offsets.data_ptr(), 2 * T, E, D, H, arr,
                                                  h.data_ptr(), None))
@@ -81,9 +74,9 @@ def test_layer_through_the_four_wave_kernel(dev, four_wave):
     dim = 2048
     sd, x = small_layer(seed=91, dim=dim, tokens=700, weights="fp8", scale_in=0.5)
     m = synth.build_module({k: v.to(dev) for k, v in sd.items()}, "fp8", dev, dim=dim)
-    os.environ["HDMOE_SWIGLU4W"] = "0"
+    set_form("HDMOE_SWIGLU4W", "0")
     base = m(x.to(dev)).cpu()
-    os.environ["HDMOE_SWIGLU4W"] = "1"
+    set_form("HDMOE_SWIGLU4W", "1")
     four = m(x.to(dev)).cpu()
     assert torch.equal(base.view(torch.int16), four.view(torch.int16))
     idx, w, _, _ = O.gate_fixed_order(x.reshape(-1, dim), sd["gate.weight"])
@@ -107,9 +100,9 @@ def test_dense_feed_forward_through_both_kernels(dev, four_wave):
             lin.scale_weight.copy_(sw)
             lin.scale_input.fill_(0.5)
     x = torch.randn((2, 450, dim), generator=g).to(BF16).to(dev)
-    os.environ["HDMOE_SWIGLU4W"] = "0"
+    set_form("HDMOE_SWIGLU4W", "0")
     base = ff(x).cpu()
-    os.environ["HDMOE_SWIGLU4W"] = "1"
+    set_form("HDMOE_SWIGLU4W", "1")
     four = ff(x).cpu()
     assert bool(torch.isfinite(base.float()).all()) and float(base.float().abs().max()) > 0
     assert torch.equal(base.view(torch.int16), four.view(torch.int16))
@@ -118,7 +111,7 @@ def test_dense_feed_forward_through_both_kernels(dev, four_wave):
 def test_layer_with_the_four_wave_kernel_in_a_graph(dev, four_wave):
     """Capture and replay of a layer whose gate/up contraction takes the 4-wave kernel (no memset nodes, nothing
     allocated, the kernel attribute set before the capture)."""
-    os.environ["HDMOE_SWIGLU4W"] = "1"
+    set_form("HDMOE_SWIGLU4W", "1")
     dim = 2048
     sd, x = small_layer(seed=17, dim=dim, tokens=600, weights="fp8")
     m = synth.build_module({k: v.to(dev) for k, v in sd.items()}, "fp8", dev, dim=dim)

@@ -185,6 +185,25 @@ def test_scale_cache_is_dropped_on_load_and_on_request():
     assert ops.scale_value(p) == 8.0                             # host tensors are read directly by default
 
 
+def test_pointer_cache_refuses_tensors_that_would_be_packed_from_a_temporary():
+    """The cached pointer structures hold raw addresses of the module's own tensors. A weight that is not contiguous
+    is packed from a `contiguous()` temporary, and a scale that is not an fp32 scalar from a cast copy: neither may be
+    cached, or the next call would read memory the allocator has taken back."""
+    dev = torch.device("cpu")
+    ffn = hidream.FeedForwardSwiGLU(64, 96, multiple_of=64, dtype=BF16, operations=ops.disable_weight_init)
+    assert hidream._pack_key([ffn], dev) is not None
+    w = ffn.w1.weight
+    ffn.w1.weight = torch.nn.Parameter(torch.empty((w.shape[1], w.shape[0]), dtype=BF16).t(), requires_grad=False)
+    assert ffn.w1.weight.shape == w.shape and not ffn.w1.weight.is_contiguous()
+    assert hidream._pack_key([ffn], dev) is None
+    ffn.w1.weight = w
+    assert hidream._pack_key([ffn], dev) is not None
+    ffn.w2.scale_input = torch.nn.Parameter(torch.ones((), dtype=torch.float64), requires_grad=False)
+    assert hidream._pack_key([ffn], dev) is None
+    ffn.w2.scale_input = torch.nn.Parameter(torch.ones(2, dtype=torch.float32)[::2].reshape(()), requires_grad=False)
+    assert hidream._pack_key([ffn], dev) is not None      # a 0-dim view is contiguous: its address is its value's
+
+
 def test_fp8_ops_linear_falls_back_when_the_fp8_path_raises(monkeypatch, caplog):
     """comfy/ops.py:367-377: an exception inside fp8_linear is logged and the Linear is computed the plain way."""
     import logging
