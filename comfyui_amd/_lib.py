@@ -60,6 +60,7 @@ class LayerArgs(ctypes.Structure):
         ("stage_events", ctypes.POINTER(c_void_p)),
         ("mod_scale", c_void_p), ("mod_shift", c_void_p), ("mod_gate", c_void_p),
         ("tokens_per_batch", c_int), ("ln_eps", ctypes.c_float), ("uniform_scale_in", c_int),
+        ("scale_check", c_void_p),
     ]
 
 
@@ -67,7 +68,7 @@ class LayerLayout(ctypes.Structure):
     """hdmoe_layer_layout"""
     _fields_ = [(n, c_size_t) for n in
                 ("topk_idx", "topk_weight", "counts", "offsets", "perm", "inv_perm", "dispatch_ws",
-                 "a", "h", "y", "normed", "partials", "total")]
+                 "a", "h", "y", "normed", "partials", "flags", "total")]
 
 
 # name -> (restype, argtypes); every symbol include/hdmoe.h declares

@@ -56,6 +56,25 @@ static inline bool hdmoe_few_rows(int rows_dyn, int n_dyn, int rows_static) {
   return (n_dyn <= 0 || rows_dyn <= 128 * n_dyn) && rows_static <= 256;
 }
 
+// What the gate + cast kernel of the one-call layer decides and verifies from the values behind the scale pointers
+// (see GateQuant in gate.hip).
+struct HdmoeGateScaleChecks {
+  bool decide;               // the kernel picks one row per token or a row per slot and reports it in *layout_flag
+  bool with_shared;          // row-per-slot layout: also write the shared expert's token-order copy
+  int32_t* layout_flag;      // device word: 1 = one row per token
+  int32_t* scale_check;      // optional word (device, or host memory the device can write): set to 1 on a mismatch
+  const float* scale_in3[HDMOE_MAX_EXPERTS];  // scale_input of every expert's w3
+  const float* shared_scale3;                 // of the w3 the shared_scale passed beside this belongs to
+};
+
+// A second description of the gathered token operand of a grouped GEMM, taken when *flag reads 0 on the device.
+struct HdmoeAltOperand {
+  const int32_t* flag;
+  const uint8_t* a;
+  int rows;      // rows of a
+  int shift;     // row = gather[r] >> shift
+};
+
 constexpr int HDMOE_NUM_CU = 256;   // MI355X
 constexpr int HDMOE_NUM_XCD = 8;
 

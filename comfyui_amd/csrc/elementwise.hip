@@ -21,12 +21,16 @@ __device__ __forceinline__ float round_bf16(float f) { return hdmoe_dev_round_bf
 __device__ __forceinline__ uint2 quant8(const uint4& v, float inv) { return hdmoe_q_8(v, inv); }
 __device__ __forceinline__ float inv_scale(const float* s) { return hdmoe_q_uniform(hdmoe_q_inv_scale(s)); }
 
+// scale_in_also: scale_input of a second Linear that reads this cast (w3 beside w1). Where its cast factor differs the
+// one cast cannot serve both: the rows are written as NaN (products with a NaN factor).
 __global__ __launch_bounds__(THREADS) void quant_rows_kernel(const uint4* __restrict__ x, long rows, int row16,
-                                                             const float* scale_in, uint2* __restrict__ out) {
+                                                             const float* scale_in, const float* scale_in_also,
+                                                             uint2* __restrict__ out) {
   const int lane = threadIdx.x & 63;
   const long wave = (long)blockIdx.x * WAVES + (threadIdx.x >> 6);
   const long nwaves = (long)gridDim.x * WAVES;
-  const float inv = inv_scale(scale_in);
+  float inv = inv_scale(scale_in);
+  if (scale_in_also != scale_in && inv_scale(scale_in_also) != inv) inv = __builtin_nanf("");
   for (long r = wave; r < rows; r += nwaves)
     for (int u = lane; u < row16; u += 64) out[r * row16 + u] = quant8(x[r * row16 + u], inv);
 }
@@ -379,6 +383,13 @@ int hdmoe_launch_quant_dispatch(const void* x_bf16, const int32_t* perm, const i
   return hdmoe_check_launch(what);
 }
 
+int hdmoe_launch_quant_rows(const void* x_bf16, int64_t rows, int D, const float* scale_input_dev,
+                            const float* scale_input_also_dev, void* out_fp8, hipStream_t s, const char* what) {
+  hipLaunchKernelGGL(quant_rows_kernel, dim3(row_blocks(rows)), dim3(THREADS), 0, s, static_cast<const uint4*>(x_bf16),
+                     (long)rows, D / 8, scale_input_dev, scale_input_also_dev, static_cast<uint2*>(out_fp8));
+  return hdmoe_check_launch(what);
+}
+
 extern "C" int hdmoe_quant_fp8(const void* x_bf16, int64_t rows, int D, const float* scale_input_dev, void* out_fp8,
                                hdmoe_stream_t stream) {
   HDMOE_REQUIRE_PTR(x_bf16);
@@ -387,10 +398,8 @@ extern "C" int hdmoe_quant_fp8(const void* x_bf16, int64_t rows, int D, const fl
     return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_quant_fp8: rows=%lld D=%d (D must be a positive multiple of 8)",
                       (long long)rows, D);
   if (rows == 0) return HDMOE_OK;
-  hipLaunchKernelGGL(quant_rows_kernel, dim3(row_blocks(rows)), dim3(THREADS), 0, static_cast<hipStream_t>(stream),
-                     static_cast<const uint4*>(x_bf16), (long)rows, D / 8, scale_input_dev,
-                     static_cast<uint2*>(out_fp8));
-  return hdmoe_check_launch("hdmoe_quant_fp8");
+  return hdmoe_launch_quant_rows(x_bf16, rows, D, scale_input_dev, scale_input_dev, out_fp8,
+                                 static_cast<hipStream_t>(stream), "hdmoe_quant_fp8");
 }
 
 extern "C" int hdmoe_quant_permute_fp8(const void* x_bf16, const int32_t* perm, const int32_t* offsets, int T, int D,

@@ -200,6 +200,21 @@ struct GateQuant {
   const float* shared_scale;
   uint2* xq_routed;           // [2T, D] e4m3fn
   uint2* xq_shared;           // [T, D] e4m3fn or NULL
+  // Decisions and checks that depend on the VALUES behind the scale pointers are made here, on the device, from
+  // those values: the host would have to read them back to know them, and a copy it keeps goes stale when a scale
+  // tensor is written in place.
+  //   decide != 0: both outputs are given and the kernel chooses. If every expert (and the shared expert) casts the
+  //     tokens with the same factor, it writes one row per token to xq_shared and 1 to *layout_flag; else the rows
+  //     2t, 2t+1 of xq_routed (and the shared expert's copy if with_shared) and 0 to *layout_flag. The GEMM that
+  //     follows reads the flag and the matching operand.
+  //   scale_in3 / shared_scale3: scale_input of the w3 Linears. w1 and w3 read one cast of the tokens, made with
+  //     w1's factor; where w3's factor differs the cast cannot serve both, the rows are written as NaN (so is then
+  //     the layer's output) and *scale_check, if given, is set to 1.
+  int decide, with_shared;
+  int32_t* layout_flag;
+  int32_t* scale_check;
+  HdmoeScalePtrs scale_in3;
+  const float* shared_scale3;
   // LN variant of the register kernel: the row is LayerNorm(x) * (1 + scale[b]) + shift[b] (as ln_modulate_kernel
   // computes it, bit for bit), b = token / tokens_per_batch; the normalised tokens are never written as bf16
   const uint4* mod_scale;     // [batch, D] bf16
@@ -269,10 +284,30 @@ __global__ __launch_bounds__(WAVES_PER_BLOCK * 64, 3) void gate_top2_reg_kernel(
   // the 1/scale_input of every expert, read once: a load that depends on the routing inside the token loop
   // would make every token wait for its predecessor's stores (loads and stores retire in order)
   float inv_e[E], invs = -1.0f;
+  bool one_row = false, with_shared = false;
   if constexpr (QUANT) {
+    bool ok13 = true, same = true;
 #pragma unroll
-    for (int e = 0; e < E; ++e) inv_e[e] = hdmoe_q_inv_scale(q.scale_in.p[e]);
+    for (int e = 0; e < E; ++e) {
+      inv_e[e] = hdmoe_q_inv_scale(q.scale_in.p[e]);
+      if (q.scale_in3.p[e] != q.scale_in.p[e]) ok13 = ok13 && hdmoe_q_inv_scale(q.scale_in3.p[e]) == inv_e[e];
+    }
     invs = hdmoe_q_uniform(hdmoe_q_inv_scale(q.shared_scale));
+    if (q.shared_scale3 != q.shared_scale) ok13 = ok13 && hdmoe_q_inv_scale(q.shared_scale3) == invs;
+#pragma unroll
+    for (int e = 0; e < E; ++e) same = same && inv_e[e] == invs;
+    one_row = q.decide ? same : q.xq_routed == nullptr;
+    with_shared = q.decide ? q.with_shared != 0 : q.xq_shared != nullptr;
+    if (!ok13) {
+      // the factors are NaN from here on: every product and so every byte written below is NaN
+      invs = __builtin_nanf("");
+#pragma unroll
+      for (int e = 0; e < E; ++e) inv_e[e] = invs;
+    }
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+      if (q.decide) *q.layout_flag = same ? 1 : 0;
+      if (!ok13 && q.scale_check != nullptr) *q.scale_check = 1;
+    }
   }
   for (; t < t_end; t += walk.step) {
     const int tn = t + walk.step;
@@ -315,7 +350,7 @@ __global__ __launch_bounds__(WAVES_PER_BLOCK * 64, 3) void gate_top2_reg_kernel(
       }
       inv0 = hdmoe_q_uniform(inv0);
       inv1 = hdmoe_q_uniform(inv1);
-      if (q.xq_routed == nullptr) {
+      if (one_row) {
         // one scale_input for all: one row per token
 #pragma unroll
         for (int c = 0; c < NCHUNK; ++c) q.xq_shared[(size_t)t * ROW16 + c * 64 + lane] = hdmoe_q_8(cur[c], invs);
@@ -327,7 +362,7 @@ __global__ __launch_bounds__(WAVES_PER_BLOCK * 64, 3) void gate_top2_reg_kernel(
           const uint2 v0 = hdmoe_q_8(cur[c], inv0);
           r0[c * 64 + lane] = v0;
           r0[ROW16 + c * 64 + lane] = same01 ? v0 : hdmoe_q_8(cur[c], inv1);
-          if (q.xq_shared != nullptr)
+          if (with_shared)
             q.xq_shared[(size_t)t * ROW16 + c * 64 + lane] = same0s ? v0 : hdmoe_q_8(cur[c], invs);
         }
       }
@@ -350,6 +385,24 @@ __global__ __launch_bounds__(WAVES_PER_BLOCK * 64) void gate_top2_generic_kernel
   int cnt[E];
 #pragma unroll
   for (int e = 0; e < E; ++e) cnt[e] = 0;
+  // the decisions and checks on the scale values (see GateQuant), once per wave
+  bool one_row = false, with_shared = false, ok13 = true;
+  if constexpr (QUANT) {
+    bool same = true;
+    const float invs = hdmoe_q_inv_scale(q.shared_scale);
+    if (q.shared_scale3 != q.shared_scale) ok13 = hdmoe_q_inv_scale(q.shared_scale3) == invs;
+    for (int e = 0; e < E; ++e) {
+      const float inv = hdmoe_q_inv_scale(q.scale_in.p[e]);
+      same = same && inv == invs;
+      if (q.scale_in3.p[e] != q.scale_in.p[e]) ok13 = ok13 && hdmoe_q_inv_scale(q.scale_in3.p[e]) == inv;
+    }
+    one_row = q.decide ? same : q.xq_routed == nullptr;
+    with_shared = q.decide ? q.with_shared != 0 : q.xq_shared != nullptr;
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+      if (q.decide) *q.layout_flag = same ? 1 : 0;
+      if (!ok13 && q.scale_check != nullptr) *q.scale_check = 1;
+    }
+  }
   for (int t = walk.first; t < t_end; t += walk.step) {
     float logit[E];
 #pragma unroll
@@ -364,16 +417,17 @@ __global__ __launch_bounds__(WAVES_PER_BLOCK * 64) void gate_top2_generic_kernel
 #pragma unroll
     for (int e = 0; e < E; ++e) cnt[e] += (i0 == e) + (i1 == e);
     if constexpr (QUANT) {
-      const float inv0 = hdmoe_q_uniform(hdmoe_q_inv_scale(q.scale_in.p[i0]));
-      const float inv1 = hdmoe_q_uniform(hdmoe_q_inv_scale(q.scale_in.p[i1]));
-      const float invs = hdmoe_q_uniform(hdmoe_q_inv_scale(q.shared_scale));
+      const float bad = __builtin_nanf("");   // a cast that cannot serve w1 and w3 alike: NaN rows
+      const float inv0 = hdmoe_q_uniform(ok13 ? hdmoe_q_inv_scale(q.scale_in.p[i0]) : bad);
+      const float inv1 = hdmoe_q_uniform(ok13 ? hdmoe_q_inv_scale(q.scale_in.p[i1]) : bad);
+      const float invs = hdmoe_q_uniform(ok13 ? hdmoe_q_inv_scale(q.shared_scale) : bad);
       for (int u = lane; u < row16; u += 64) {
         const uint4 xv = x[(size_t)t * row16 + u];
-        if (q.xq_routed != nullptr) {
+        if (!one_row) {
           q.xq_routed[(size_t)(2 * t) * row16 + u] = hdmoe_q_8(xv, inv0);
           q.xq_routed[(size_t)(2 * t + 1) * row16 + u] = hdmoe_q_8(xv, inv1);
         }
-        if (q.xq_shared != nullptr) q.xq_shared[(size_t)t * row16 + u] = hdmoe_q_8(xv, invs);
+        if (one_row || with_shared) q.xq_shared[(size_t)t * row16 + u] = hdmoe_q_8(xv, invs);
       }
     }
   }
@@ -544,9 +598,19 @@ int hdmoe_launch_gate_quant(const void* x_bf16, const void* gate_w_bf16, int T, 
                             void* topk_weight_bf16, const float* const* scale_input, const float* shared_scale,
                             void* xq_routed, void* xq_shared, hipStream_t s, const char* what,
                             const void* mod_scale = nullptr, const void* mod_shift = nullptr, int tokens_per_batch = 0,
-                            float ln_eps = 0.0f, int32_t* block_hist = nullptr) {
+                            float ln_eps = 0.0f, int32_t* block_hist = nullptr, const HdmoeGateScaleChecks* checks = nullptr) {
   GateQuant q;
   memset(&q, 0, sizeof(q));
+  for (int e = 0; e < E && e < HDMOE_MAX_EXPERTS; ++e) q.scale_in3.p[e] = scale_input[e];  // nothing to compare
+  q.shared_scale3 = shared_scale;
+  if (checks != nullptr) {
+    q.decide = checks->decide ? 1 : 0;
+    q.with_shared = checks->with_shared ? 1 : 0;
+    q.layout_flag = checks->layout_flag;
+    q.scale_check = checks->scale_check;
+    for (int e = 0; e < E && e < HDMOE_MAX_EXPERTS; ++e) q.scale_in3.p[e] = checks->scale_in3[e];
+    q.shared_scale3 = checks->shared_scale3;
+  }
   if (mod_scale != nullptr) {
     q.mod_scale = static_cast<const uint4*>(mod_scale);
     q.mod_shift = static_cast<const uint4*>(mod_shift);

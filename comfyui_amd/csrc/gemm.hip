@@ -81,6 +81,8 @@ struct GemmGroup {
   const float* sb0;     // scale_weight of b0 (fp8)
   const float* sb1;     // scale_weight of b1 (fp8, swiglu)
   const float* s_in;    // scale_input of this Linear (fp8), NULL = 1
+  const float* s_in_b;  // swiglu: scale_input of the w3 Linear (its value may differ from w1's where both round to the
+                        // same cast factor); NULL = s_in
   const float* s_next;  // scale_input of the Linear that consumes the output (fp8 swiglu), NULL = clamp rule
   uint8_t* out;         // [rows, n_out] in the element type of the mode
   int row_begin;        // >= 0: static segment [row_begin, row_end); < 0: offsets[dyn], offsets[dyn+1]
@@ -106,6 +108,10 @@ struct GemmArgs {
   int nparts;
   long long part_stride;  // floats between two parts
   HdmoeSplitPlan plan;    // split K only
+  // Gathered groups only: where *alt.flag reads 0 on the device, their token operand is alt.a (alt.rows rows, row
+  // gather[r] >> alt.shift) instead of what the groups say (the gate kernel of the layer picks the layout of the fp8
+  // tokens from the scale values and leaves the flag). flag NULL = off.
+  HdmoeAltOperand alt;
 };
 
 __device__ __forceinline__ int swz(int row) { return ((row >> 1) & 7) ^ ((row & 1) << 2); }
@@ -259,6 +265,11 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
     if (gg.row_begin >= 0) { rb = gg.row_begin; re = gg.row_end; }
     else { rb = __builtin_amdgcn_readlane(off_lane, gg.dyn); re = __builtin_amdgcn_readlane(off_lane, gg.dyn + 1); }
   };
+  // the gathered token operand: as the groups describe it, or the alternative the flag selects
+  const bool use_alt = args.alt.flag != nullptr && __builtin_amdgcn_readfirstlane(*args.alt.flag) == 0;
+  auto gathered_a = [&](const GemmGroup& gg) { return use_alt ? args.alt.a : gg.a; };
+  auto gathered_rows = [&](const GemmGroup& gg) { return use_alt ? args.alt.rows : gg.a_rows; };
+  auto gathered_shift = [&](const GemmGroup& gg) { return use_alt ? args.alt.shift : gg.gather_shift; };
   // split K: which cut of the plan runs (a function of the segment sizes; the kernel that adds the parts up makes the
   // same choice)
   int plan_idx = 0;
@@ -367,7 +378,7 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
 #pragma unroll
     for (int j = 0; j < A_SLABS; ++j) {
       const int r = j * 64 + ld_row;
-      gi[j] = (gg.gather != nullptr && r < d.rows_here) ? (gg.gather[d.row0 + r] >> gg.gather_shift) : -1;
+      gi[j] = (gg.gather != nullptr && r < d.rows_here) ? (gg.gather[d.row0 + r] >> gathered_shift(gg)) : -1;
     }
   };
   // the same three resources as plain descriptor words, for the loads issued from the assembly blocks
@@ -383,7 +394,7 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
     const GemmGroup& gg = args.g[d.g];
     k_base = d.kt0 * BK;
     if constexpr (FP8) {
-      if (gg.gather != nullptr) ra4 = raw_rsrc(gg.a, (uint32_t)gg.a_rows * (uint32_t)d.kbytes);
+      if (gg.gather != nullptr) ra4 = raw_rsrc(gathered_a(gg), (uint32_t)gathered_rows(gg) * (uint32_t)d.kbytes);
       else ra4 = raw_rsrc(gg.a + (size_t)d.row0 * d.kbytes, (uint32_t)d.rows_here * (uint32_t)d.kbytes);
       const uint32_t wrows = SWIGLU ? BN / 2 : BN - 32;
       rb04 = raw_rsrc(gg.b0 + (size_t)d.n0 * d.kbytes, wrows * (uint32_t)d.kbytes);
@@ -392,7 +403,7 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
     }
     if (gg.gather != nullptr) {
       // rows past the segment end get an offset beyond the buffer and read as zero
-      src_a = make_rsrc(gg.a, (uint32_t)gg.a_rows * (uint32_t)d.kbytes);
+      src_a = make_rsrc(gathered_a(gg), (uint32_t)gathered_rows(gg) * (uint32_t)d.kbytes);
 #pragma unroll
       for (int j = 0; j < A_SLABS; ++j) src_voff[j] = gi[j] >= 0 ? gi[j] * d.kbytes + ld_chunk * 16 : (int)0x80000000u;
     } else {
@@ -639,7 +650,7 @@ __global__ __launch_bounds__(NTHREADS) void grouped_gemm_kernel(const GemmArgs a
       const float s_in = gg.s_in ? *gg.s_in : 1.0f;
       ep_a = s_in * *gg.sb0;
       if constexpr (SWIGLU) {
-        ep_b = s_in * *gg.sb1;
+        ep_b = (gg.s_in_b ? *gg.s_in_b : s_in) * *gg.sb1;
         ep_next = gg.s_next ? hdmoe_dev_round_bf16(__fdiv_rn(1.0f, *gg.s_next)) : -1.0f;
       }
     }
@@ -1163,7 +1174,7 @@ int hdmoe_launch_ffn_gemm(bool swiglu, int weight_dtype, const uint8_t* a_dyn, c
                           int K_static, int N_static, hipStream_t s, const char* what,
                           const int32_t* gather_dyn = nullptr, int gather_rows = 0, float* partial = nullptr,
                           int nparts = 1, int gather_shift = 0, bool reduce = true,
-                          const HdmoeSplitPlan* plan = nullptr) {
+                          const HdmoeSplitPlan* plan = nullptr, const HdmoeAltOperand* alt = nullptr) {
   const int eb = elem_bytes(weight_dtype);
   const bool fp8 = weight_dtype == HDMOE_W_E4M3FN;
   const int feat_per_tile = swiglu ? BN / 2 : BN;
@@ -1178,11 +1189,13 @@ int hdmoe_launch_ffn_gemm(bool swiglu, int weight_dtype, const uint8_t* a_dyn, c
   FormChoice choice = pick_form(shape);
   const bool light = choice.light, ring16 = choice.ring16, tall = choice.tall;
   const int BM = tall ? TileCfg<5>::BM : TileCfg<4>::BM;  // tokens per block tile of the kernel that will run
-  if (gather_dyn != nullptr && (unsigned long long)gather_rows * K_dyn * eb >= (1ull << 31))
-    return hdmoe_fail(HDMOE_E_SHAPE, "%s: %d gathered rows of %d bytes exceed the 2 GiB offset range", what, gather_rows,
-                      K_dyn * eb);
+  const int gather_rows_max = (alt != nullptr && alt->rows > gather_rows) ? alt->rows : gather_rows;
+  if (gather_dyn != nullptr && (unsigned long long)gather_rows_max * K_dyn * eb >= (1ull << 31))
+    return hdmoe_fail(HDMOE_E_SHAPE, "%s: %d gathered rows of %d bytes exceed the 2 GiB offset range", what,
+                      gather_rows_max, K_dyn * eb);
   GemmArgs args;
   memset(&args, 0, sizeof(args));
+  if (alt != nullptr && gather_dyn != nullptr) args.alt = *alt;
   args.nparts = 1;
   args.offsets = offsets;
   args.n_offsets = n_dyn;
@@ -1201,7 +1214,7 @@ int hdmoe_launch_ffn_gemm(bool swiglu, int weight_dtype, const uint8_t* a_dyn, c
     gg.kbytes = K_dyn * eb;
     if (swiglu) {
       gg.b0 = static_cast<const uint8_t*>(w.w1); gg.b1 = static_cast<const uint8_t*>(w.w3);
-      gg.sb0 = w.scale_w1; gg.sb1 = w.scale_w3; gg.s_in = w.scale_in1; gg.s_next = w.scale_in2;
+      gg.sb0 = w.scale_w1; gg.sb1 = w.scale_w3; gg.s_in = w.scale_in1; gg.s_in_b = w.scale_in3; gg.s_next = w.scale_in2;
     } else {
       gg.b0 = static_cast<const uint8_t*>(w.w2); gg.sb0 = w.scale_w2; gg.s_in = w.scale_in2;
     }
@@ -1223,7 +1236,7 @@ int hdmoe_launch_ffn_gemm(bool swiglu, int weight_dtype, const uint8_t* a_dyn, c
     gg.kbytes = K_static * eb;
     if (swiglu) {
       gg.b0 = static_cast<const uint8_t*>(w.w1); gg.b1 = static_cast<const uint8_t*>(w.w3);
-      gg.sb0 = w.scale_w1; gg.sb1 = w.scale_w3; gg.s_in = w.scale_in1; gg.s_next = w.scale_in2;
+      gg.sb0 = w.scale_w1; gg.sb1 = w.scale_w3; gg.s_in = w.scale_in1; gg.s_in_b = w.scale_in3; gg.s_next = w.scale_in2;
     } else {
       gg.b0 = static_cast<const uint8_t*>(w.w2); gg.sb0 = w.scale_w2; gg.s_in = w.scale_in2;
     }
@@ -1313,7 +1326,7 @@ int hdmoe_launch_ffn_gemm(bool swiglu, int weight_dtype, const uint8_t* a_dyn, c
     return hdmoe_check_launch(what);
   }
   if (fp8 && swiglu) {
-    long long op_bytes = (long long)(gather_dyn != nullptr ? gather_rows : rows_dyn) * K_dyn;
+    long long op_bytes = (long long)(gather_dyn != nullptr ? gather_rows_max : rows_dyn) * K_dyn;
     if ((long long)rows_static * K_static > op_bytes) op_bytes = (long long)rows_static * K_static;
     shape.w4_fits = swiglu4w_fits(args, op_bytes);
     choice = pick_form(shape);

@@ -10,7 +10,7 @@ int hdmoe_launch_ffn_gemm(bool swiglu, int weight_dtype, const uint8_t* a_dyn, c
                           int K_static, int N_static, hipStream_t s, const char* what,
                           const int32_t* gather_dyn = nullptr, int gather_rows = 0, float* partial = nullptr,
                           int nparts = 1, int gather_shift = 0, bool reduce = true,
-                          const HdmoeSplitPlan* plan = nullptr);
+                          const HdmoeSplitPlan* plan = nullptr, const HdmoeAltOperand* alt = nullptr);
 int hdmoe_launch_combine_partials(const float* partial, long long part_stride, const HdmoeSplitPlan& plan,
                                   int rows_dyn, int n_dyn,
                                   const int32_t* offsets, bool fp8, const hdmoe_ffn_weights* experts,
@@ -27,13 +27,16 @@ int hdmoe_launch_gate_quant(const void* x_bf16, const void* gate_w_bf16, int T, 
                             void* topk_weight_bf16, const float* const* scale_input, const float* shared_scale,
                             void* xq_routed, void* xq_shared, hipStream_t s, const char* what,
                             const void* mod_scale = nullptr, const void* mod_shift = nullptr, int tokens_per_batch = 0,
-                            float ln_eps = 0.0f, int32_t* block_hist = nullptr);
+                            float ln_eps = 0.0f, int32_t* block_hist = nullptr,
+                            const HdmoeGateScaleChecks* checks = nullptr);
 int hdmoe_launch_gate(const void* x_bf16, const void* gate_w_bf16, int T, int D, int E, int32_t* topk_idx,
                       void* topk_weight_bf16, int32_t* block_hist, hipStream_t s, const char* what);
 int hdmoe_launch_dispatch_scatter(const int32_t* topk_idx, int T, int E, int32_t* counts, int32_t* offsets,
                                   int32_t* perm, int32_t* inv_perm, const int32_t* block_hist, int tokens_per_hist,
                                   hipStream_t s, const char* what);
 bool hdmoe_gate_quant_takes_ln(int D, int E);
+int hdmoe_launch_quant_rows(const void* x_bf16, int64_t rows, int D, const float* scale_input_dev,
+                            const float* scale_input_also_dev, void* out_fp8, hipStream_t s, const char* what);
 int hdmoe_launch_combine(const void* y_sorted_bf16, const int32_t* inv_perm, const void* topk_weight_bf16,
                          const void* shared_bf16, const void* gate_bf16, const void* residual_bf16, int tokens_per_batch,
                          int T, int D, void* out_bf16, hipStream_t s, const char* what, bool f16 = false);
@@ -81,6 +84,8 @@ extern "C" int hdmoe_layer_layout_get(int T, int D, int H, int Hs, int E, int we
   // fp32 partial sums of a down projection cut along K (small token counts), [parts][2T + T][D]
   const int parts = hdmoe_down_parts((int)n, E, Hs > 0 ? T : 0, D, H, Hs, weight_dtype);
   out->partials = take(parts > 1 ? (size_t)parts * (n + (Hs > 0 ? (size_t)T : 0)) * D * 4 : 0);
+  // one word the gate + cast kernel leaves for the gate/up GEMM: which layout of the fp8 tokens it wrote
+  out->flags = take(256);
   out->total = off;
   return HDMOE_OK;
 }
@@ -177,29 +182,50 @@ extern "C" int hdmoe_moe_ffn(const hdmoe_layer_args* p, hdmoe_stream_t stream) {
   // serves them all and the gate/up GEMM reads row perm[r] / 2 of it. Otherwise the token is cast for its two experts
   // (rows 2t, 2t+1 of a_routed, i.e. in flat slot order) and for the shared expert, and the GEMM reads the routed rows
   // through the permutation instead of from a permuted copy.
-  bool one_copy = false;
+  // Which of the two it is depends on the VALUES of the scale_inputs. The host sees pointers: all the same pointer
+  // (all NULL included) is one copy, a mix of NULL (clamp rule) and non-NULL is never one copy; for different non-NULL
+  // pointers the gate kernel compares the values on the device, writes the layout that fits and leaves a flag the
+  // gate/up GEMM reads (uniform_scale_in of the arguments is not needed for that and is not looked at). The same
+  // kernel checks that w1 and w3 of every group cast the tokens alike (they read one cast).
+  bool one_copy = false, decide = false;
   if (fp8) {
-    one_copy = true;
     const float* first = p->experts[0].scale_in1;
-    for (int e = 1; e < E; ++e) one_copy = one_copy && p->experts[e].scale_in1 == first;
-    if (Hs > 0) one_copy = one_copy && p->shared->scale_in1 == first;
-    one_copy = one_copy || p->uniform_scale_in != 0;
-    // a mix of NULL (clamp rule) and non-NULL scale_inputs is never uniform, whatever the caller says
-    for (int e = 0; e < E; ++e) one_copy = one_copy && ((p->experts[e].scale_in1 == nullptr) == (first == nullptr));
-    if (Hs > 0) one_copy = one_copy && ((p->shared->scale_in1 == nullptr) == (first == nullptr));
+    bool same_ptr = true, mixed = false;
+    for (int e = 0; e < E; ++e) {
+      same_ptr = same_ptr && p->experts[e].scale_in1 == first;
+      mixed = mixed || ((p->experts[e].scale_in1 == nullptr) != (first == nullptr));
+    }
+    if (Hs > 0) {
+      same_ptr = same_ptr && p->shared->scale_in1 == first;
+      mixed = mixed || ((p->shared->scale_in1 == nullptr) != (first == nullptr));
+    }
+    one_copy = same_ptr;
+    decide = !same_ptr && !mixed;
   }
+  int32_t* const layout_flag = reinterpret_cast<int32_t*>(ws + l.flags);
   if (fp8) {
     const float* sin[HDMOE_MAX_EXPERTS];
-    for (int e = 0; e < E; ++e) sin[e] = p->experts[e].scale_in1;
-    const float* token_scale = (Hs > 0 && !one_copy) ? p->shared->scale_in1 : p->experts[0].scale_in1;
+    HdmoeGateScaleChecks checks = {};
+    for (int e = 0; e < E; ++e) {
+      sin[e] = p->experts[e].scale_in1;
+      checks.scale_in3[e] = p->experts[e].scale_in3;
+    }
+    // the scale of the token-order copy: the shared expert's, or (one copy for all, no shared expert) the experts'
+    const hdmoe_ffn_weights& token_w = Hs > 0 ? *p->shared : p->experts[0];
+    checks.decide = decide;
+    checks.with_shared = Hs > 0;
+    checks.layout_flag = layout_flag;
+    checks.scale_check = p->scale_check;
     // the one copy sits where the shared expert's copy would (without a shared expert that room does not exist: the
-    // start of the routed rows' room then)
-    if (one_copy && Hs == 0) a_shared = a_routed;
-    if (int rc = hdmoe_launch_gate_quant(xin, p->gate_w, T, D, E, idx, tw, sin, (Hs > 0 || one_copy) ? token_scale : nullptr,
-                                         one_copy ? nullptr : a_routed, (Hs > 0 || one_copy) ? a_shared : nullptr, s,
+    // start of the routed rows' room then; only one of the two layouts is written in a call)
+    if (Hs == 0) a_shared = a_routed;
+    const bool token_copy = Hs > 0 || one_copy || decide;
+    checks.shared_scale3 = token_copy ? token_w.scale_in3 : nullptr;
+    if (int rc = hdmoe_launch_gate_quant(xin, p->gate_w, T, D, E, idx, tw, sin, token_copy ? token_w.scale_in1 : nullptr,
+                                         one_copy ? nullptr : a_routed, token_copy ? a_shared : nullptr, s,
                                          "hdmoe_moe_ffn (gate + quantise)",
                                          ln_in_gate ? p->mod_scale : nullptr, ln_in_gate ? p->mod_shift : nullptr,
-                                         p->tokens_per_batch, p->ln_eps, hist))
+                                         p->tokens_per_batch, p->ln_eps, hist, &checks))
       return rc;
   } else {
     if (D % 8 != 0) return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_moe_ffn: D=%d must be a multiple of 8", D);
@@ -228,12 +254,19 @@ extern "C" int hdmoe_moe_ffn(const hdmoe_layer_args* p, hdmoe_stream_t stream) {
 
   mark();
   // gate/up projections + SiLU*mul, routed experts and shared expert in one launch
-  const bool per_token = one_copy || !fp8;  // the routed operand holds one row per token (else one per flat slot)
-  const uint8_t* const a_dyn = !fp8 ? static_cast<const uint8_t*>(xin) : (one_copy ? a_shared : a_routed);
+  // the routed operand holds one row per token (else one per flat slot); when the gate kernel decided, the
+  // one-row-per-token form is described here and the other one as the alternative its flag selects
+  const bool per_token = one_copy || decide || !fp8;
+  const uint8_t* const a_dyn = !fp8 ? static_cast<const uint8_t*>(xin) : (per_token ? a_shared : a_routed);
+  HdmoeAltOperand alt;
+  alt.flag = layout_flag;
+  alt.a = a_routed;
+  alt.rows = (int)n;
+  alt.shift = 0;
   if (int rc = hdmoe_launch_ffn_gemm(true, wd, a_dyn, offsets, (int)n, E, p->experts, h_routed,
                                      a_static, Hs > 0 ? T : 0, p->shared, h_shared, D, H, D, Hs, s,
                                      "hdmoe_moe_ffn (gate/up)", perm, per_token ? T : (int)n, nullptr, 1,
-                                     per_token ? 1 : 0))
+                                     per_token ? 1 : 0, true, nullptr, decide ? &alt : nullptr))
     return rc;
   mark();
   // down projections, both in one launch
@@ -294,7 +327,10 @@ extern "C" int hdmoe_ffn_swiglu(int weight_dtype, const void* x_bf16, int rows, 
   const uint8_t* a = static_cast<const uint8_t*>(x_bf16);
   uint8_t* h = ws;
   if (fp8) {
-    if (int rc = hdmoe_quant_fp8(x_bf16, rows, D, w->scale_in1, ws, stream)) return rc;
+    if (D % 8 != 0) return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_ffn_swiglu: D=%d must be a multiple of 8", D);
+    // one cast for w1 and w3, made with w1's factor and checked against w3's on the device
+    if (int rc = hdmoe_launch_quant_rows(x_bf16, rows, D, w->scale_in1, w->scale_in3, ws, s, "hdmoe_ffn_swiglu (quantise)"))
+      return rc;
     a = ws;
     h = ws + hdmoe_align_up((size_t)rows * D, 256);
   }

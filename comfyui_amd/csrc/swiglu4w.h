@@ -92,6 +92,11 @@ __global__ __launch_bounds__(W4_THREADS) __attribute__((amdgpu_waves_per_eu(1, 1
     return d;
   };
 
+  // the gathered token operand: as the groups describe it, or the alternative the flag selects (GemmArgs::alt)
+  const bool use_alt = args.alt.flag != nullptr && sgpr(*args.alt.flag) == 0;
+  auto token_base = [&](const GemmGroup& gg) { return (use_alt && gg.gather != nullptr) ? args.alt.a : gg.a; };
+  auto gather_shift = [&](const GemmGroup& gg) { return use_alt ? args.alt.shift : gg.gather_shift; };
+
   Tile4 cur = decode(0);
   if (cur.g < 0) return;   // block-uniform: every wave of the block leaves together
   Tile4 nxt = decode(1);
@@ -143,7 +148,7 @@ __global__ __launch_bounds__(W4_THREADS) __attribute__((amdgpu_waves_per_eu(1, 1
     for (int j = 0; j < 8; ++j) {
       const int r = j * 32 + ld_row;
       int v = -1;
-      if (r < d.rows_here) v = gg.gather != nullptr ? (gg.gather[d.row0 + r] >> gg.gather_shift) : d.row0 + r;
+      if (r < d.rows_here) v = gg.gather != nullptr ? (gg.gather[d.row0 + r] >> gather_shift(gg)) : d.row0 + r;
       gi[j] = v;
     }
   };
@@ -157,7 +162,7 @@ __global__ __launch_bounds__(W4_THREADS) __attribute__((amdgpu_waves_per_eu(1, 1
     }
     const GemmGroup& gg = args.g[d.g];
     kbytes = gg.kbytes;
-    ra = raw_rsrc(gg.a, 0x7fffffffu);   // rows are valid by construction; rows past the tile get an offset of 2^31
+    ra = raw_rsrc(token_base(gg), 0x7fffffffu);   // rows are valid by construction; rows past the tile get an offset of 2^31
     rb0 = raw_rsrc(gg.b0 + (size_t)d.n0 * kbytes, (uint32_t)W4_FEAT * (uint32_t)kbytes);
     rb1 = raw_rsrc(gg.b1 + (size_t)d.n0 * kbytes, (uint32_t)W4_FEAT * (uint32_t)kbytes);
 #pragma unroll
@@ -171,7 +176,7 @@ __global__ __launch_bounds__(W4_THREADS) __attribute__((amdgpu_waves_per_eu(1, 1
 
   // ---- first two K steps of the block's first tile, as a burst ------------------------------------------------
   {
-    const __amdgpu_buffer_rsrc_t pa = make_rsrc(args.g[cur.g].a, 0x7fffffffu);
+    const __amdgpu_buffer_rsrc_t pa = make_rsrc(token_base(args.g[cur.g]), 0x7fffffffu);
     const __amdgpu_buffer_rsrc_t pb0 = make_rsrc(args.g[cur.g].b0 + (size_t)cur.n0 * kbytes, (uint32_t)W4_FEAT * (uint32_t)kbytes);
     const __amdgpu_buffer_rsrc_t pb1 = make_rsrc(args.g[cur.g].b1 + (size_t)cur.n0 * kbytes, (uint32_t)W4_FEAT * (uint32_t)kbytes);
 #pragma unroll
@@ -203,7 +208,7 @@ __global__ __launch_bounds__(W4_THREADS) __attribute__((amdgpu_waves_per_eu(1, 1
     const GemmGroup& gg = args.g[cur.g];
     const float s_in = gg.s_in ? scalar_load(gg.s_in) : 1.0f;
     const int sg_bits = sgpr(__float_as_int(s_in * scalar_load(gg.sb0)));
-    const int su_bits = sgpr(__float_as_int(s_in * scalar_load(gg.sb1)));
+    const int su_bits = sgpr(__float_as_int((gg.s_in_b ? scalar_load(gg.s_in_b) : s_in) * scalar_load(gg.sb1)));
     const int inv_next_bits = sgpr(__float_as_int(hdmoe_dev_round_bf16(__fdiv_rn(1.0f, scalar_load(gg.s_next)))));
     const int pairs = sgpr(gg.kbytes / (2 * BK));
     const int kb32 = sgpr(32 * gg.kbytes);

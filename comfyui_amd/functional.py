@@ -366,12 +366,15 @@ def layer_layout(T, D, H, Hs, E, code):
 
 
 def moe_ffn(x2d, gate_w, experts, shared, H, Hs, weight_dtype, out=None, workspace=None, want_routing=False,
-            stage_events=None, modulation=None, tokens_per_batch=None, ln_eps=1e-6, uniform_scale_in=False):
+            stage_events=None, modulation=None, tokens_per_batch=None, ln_eps=1e-6, uniform_scale_in=False,
+            scale_check=None):
     """The whole layer as one enqueue. experts: list of FfnWeights, shared: FfnWeights or None.
     modulation=(shift, scale, gate), each [B, D] bf16, turns the call into the block's feed-forward branch:
     out = x + gate * layer(LayerNorm(x) * (1 + scale) + shift), with T == B * tokens_per_batch.
-    uniform_scale_in: the caller has checked that scale_input of w1/w3 is the same value for every routed expert
-    and the shared expert (fp8): the tokens are then cast once instead of three times.
+    uniform_scale_in: accepted and not used (the casting kernel compares the scale_input values on the device and
+    casts the tokens once when they agree).
+    scale_check: optional pinned int32 tensor of one element that the casting kernel sets to 1 when w1 and w3 of a
+    feed-forward turn out to cast the tokens differently (the output is then NaN).
     Returns out [T,D] bf16 (and topk_idx int32, topk_weight bf16 when want_routing)."""
     _need_hip(x2d, "moe_ffn x", BF16)
     _need_hip(gate_w, "moe_ffn gate weight", BF16)
@@ -397,6 +400,10 @@ def moe_ffn(x2d, gate_w, experts, shared, H, Hs, weight_dtype, out=None, workspa
         args.shared = ctypes.pointer(sh)
     args.out, args.workspace, args.workspace_bytes = ptr(out), ptr(workspace), workspace.numel()
     args.uniform_scale_in = 1 if uniform_scale_in else 0
+    if scale_check is not None:
+        if scale_check.dtype != torch.int32 or scale_check.numel() < 1 or not (scale_check.is_cuda or scale_check.is_pinned()):
+            raise TypeError("moe_ffn: scale_check must be an int32 tensor on the device or in pinned host memory")
+        args.scale_check = ptr(scale_check)
     if modulation is not None:
         shift, scale, gate = (_per_batch(m, "moe_ffn modulation", D, x2d.device) for m in modulation)
         if not tokens_per_batch or T != shift.shape[0] * tokens_per_batch or not (shift.shape == scale.shape == gate.shape):

@@ -126,6 +126,21 @@ def _pack_key(ffns, dev):
     return tuple(key)
 
 
+def _gate_check(gate):
+    """What the HIP gate kernel computes, checked on any gate module with the reference's attributes (this package's
+    MoEGate or the reference's own, model.py:242-259)."""
+    if getattr(gate, "scoring_func", "softmax") != 'softmax':
+        raise NotImplementedError(f'insupportable scoring function for MoE gating: {gate.scoring_func}')
+    if getattr(gate, "top_k", 2) != 2:
+        raise NotImplementedError("the HIP gate kernel selects the top 2 experts")
+
+
+def _gate_weight(gate, hidden_states):
+    """The gate weight in the activations' dtype on their device (model.py:268 routes it through cast_to because a
+    bare Parameter may have been left on the offload device)."""
+    return amd_ops.cast_to(gate.weight, dtype=hidden_states.dtype, device=hidden_states.device).contiguous()
+
+
 class FeedForwardSwiGLU(nn.Module):
     def __init__(self, dim: int, hidden_dim: int, multiple_of: int = 256,
                  ffn_dim_multiplier: Optional[float] = None, dtype=None, device=None, operations=None):
@@ -186,15 +201,10 @@ class MoEGate(nn.Module):
         pass
 
     def _check(self):
-        if self.scoring_func != 'softmax':
-            raise NotImplementedError(f'insupportable scoring function for MoE gating: {self.scoring_func}')
-        if self.top_k != 2:
-            raise NotImplementedError("the HIP gate kernel selects the top 2 experts")
+        _gate_check(self)
 
     def device_weight(self, hidden_states):
-        """The gate weight in the activations' dtype on their device (model.py:268 routes it through
-        cast_to because a bare Parameter may have been left on the offload device)."""
-        return amd_ops.cast_to(self.weight, dtype=hidden_states.dtype, device=hidden_states.device).contiguous()
+        return _gate_weight(self, hidden_states)
 
     def forward(self, hidden_states):
         self._check()
@@ -224,6 +234,8 @@ class MOEFeedForwardSwiGLU(nn.Module):
         """Device pointers of all 15 Linears for the one-call path, or None when the layer
         needs the per-Linear composition. Returned tensors are kept alive by the caller."""
         ffns = list(self.experts) + [self.shared_experts]
+        if amd_ops.take_scale_check(x.device):   # a kernel found a cached scale value stale: rebuild from the tensors
+            self.__dict__["_packed"] = None
         # resident, unpatched weights: the structures of the previous call hold as long as nothing they were built
         # from has changed
         key = _pack_key(ffns, x.device)
@@ -242,15 +254,9 @@ class MOEFeedForwardSwiGLU(nn.Module):
             if fw is None:
                 return None
             packed.append(fw)
-        # one scale_input value for every Linear that reads the tokens: they are cast to fp8 once
+        # whether one scale_input value serves every Linear that reads the tokens (they are then cast to fp8 once) is
+        # decided on the device from the values themselves; the attribute stays for callers of functional.moe_ffn
         uniform = False
-        if wdt == FP8:
-            sis = [getattr(f.w1, "scale_input", None) for f in ffns]
-            if all(si is None for si in sis):
-                uniform = True
-            elif all(si is not None for si in sis):
-                v0 = amd_ops.scale_value(sis[0])
-                uniform = all(amd_ops.scale_value(si) == v0 for si in sis[1:])
         self.__dict__["_uniform_scale_in"] = uniform
         if key is not None:
             # the structures hold raw pointers of tensors the module owns and the key was read from: no tensor is
@@ -264,18 +270,18 @@ class MOEFeedForwardSwiGLU(nn.Module):
         if x.dtype != BF16 or not x.is_cuda:
             raise RuntimeError(f"MOEFeedForwardSwiGLU: expected a bfloat16 HIP tensor, got {x.dtype} on {x.device}; "
                                "comfyui_amd has no CPU path")
-        self.gate._check()
+        _gate_check(self.gate)      # any gate module with the reference's attributes, not only this package's
         orig_shape = x.shape
         x2 = x.reshape(-1, orig_shape[-1]).contiguous()
-        gate_w = self.gate.device_weight(x2)
+        gate_w = _gate_weight(self.gate, x2)
         # renormalised gate weights are not part of the one-call path: the stages are composed
-        got = None if self.gate.norm_topk_prob else self._collect(x2)
+        got = None if getattr(self.gate, "norm_topk_prob", False) else self._collect(x2)
         if got is not None:
             wdt, experts, shared, keep = got
             H = self.experts[0].w1.weight.shape[0]
             Hs = self.shared_experts.w1.weight.shape[0]
             y = HF.moe_ffn(x2, gate_w, experts, shared, H, Hs, wdt, stage_events=stage_events,
-                           uniform_scale_in=self._uniform_scale_in)
+                           scale_check=amd_ops.scale_check_word(x2.device) if wdt == FP8 else None)
             del keep
             return y.view(*orig_shape)
         return self._forward_composed(x2, gate_w).view(*orig_shape)
@@ -288,18 +294,18 @@ class MOEFeedForwardSwiGLU(nn.Module):
         if x.dtype != BF16 or not x.is_cuda or x.dim() != 3:
             raise RuntimeError(f"MOEFeedForwardSwiGLU.forward_branch: expected a [B,S,dim] bfloat16 HIP tensor, got "
                                f"{tuple(x.shape)} {x.dtype} on {x.device}; comfyui_amd has no CPU path")
-        self.gate._check()
+        _gate_check(self.gate)
         B, S, D = x.shape
         x2 = x.reshape(-1, D).contiguous()
         mods = tuple(m.reshape(B, D).contiguous() for m in (shift, scale, gate))
-        gate_w = self.gate.device_weight(x2)
-        got = None if self.gate.norm_topk_prob else self._collect(x2)
+        gate_w = _gate_weight(self.gate, x2)
+        got = None if getattr(self.gate, "norm_topk_prob", False) else self._collect(x2)
         if got is not None:
             wdt, experts, shared, keep = got
             H = self.experts[0].w1.weight.shape[0]
             Hs = self.shared_experts.w1.weight.shape[0]
             y = HF.moe_ffn(x2, gate_w, experts, shared, H, Hs, wdt, stage_events=stage_events, modulation=mods,
-                           uniform_scale_in=self._uniform_scale_in,
+                           scale_check=amd_ops.scale_check_word(x2.device) if wdt == FP8 else None,
                            tokens_per_batch=S, ln_eps=eps)
             del keep
             return y.view(B, S, D)
@@ -313,7 +319,7 @@ class MOEFeedForwardSwiGLU(nn.Module):
         offloaded or mixed-dtype weights, dequantising scaled-fp8 Linears)."""
         E = len(self.experts)
         idx, w = HF.gate_top2(x2, gate_w)
-        if self.gate.norm_topk_prob:
+        if getattr(self.gate, "norm_topk_prob", False):
             w = HF.renorm_top2(w)
         counts, offsets, perm, inv_perm = HF.dispatch(idx, E)
         xs = HF.permute_bf16(x2, perm)

@@ -115,11 +115,40 @@ _scale_epoch = 0
 
 def invalidate_scale_cache():
     """Forget every cached scale_input value. Called when a Linear of this package loads a state dict or takes a new
-    weight (ops.py); call it after changing a scale_input Parameter in place by other means (`p.data.copy_()` does
-    not bump the version counter the cache looks at)."""
+    weight, and when a kernel reports that a cached value was stale (take_scale_check). The cache only feeds one host
+    decision (do w1 and w3 of a feed-forward share their cast factor, i.e. can the fused kernels run); the kernels
+    read every scale from the device and verify that decision there, so a stale entry (`p.data.copy_()` does not bump
+    the version counter the cache looks at) gives NaN and a dropped cache, never a wrong number."""
     global _scale_epoch
     _scale_epoch += 1
     _scale_cache.clear()
+
+
+_scale_check_words = {}
+
+
+def scale_check_word(device):
+    """One pinned int32 per device that the layer's casting kernel sets to 1 when the scale_input values it finds on
+    the device contradict what the host asserted from its cached copies (w1 and w3 of a feed-forward must cast the
+    tokens alike); that call's output is NaN. Reading it costs no synchronisation: the module looks at it at the
+    start of every forward and drops the cache (take_scale_check)."""
+    t = _scale_check_words.get(device)
+    if t is None:
+        t = torch.zeros(1, dtype=torch.int32).pin_memory()
+        _scale_check_words[device] = t
+    return t
+
+
+def take_scale_check(device):
+    """True once after a kernel has raised the device's check word; the scale cache is dropped with it."""
+    t = _scale_check_words.get(device)
+    if t is None or int(t[0]) == 0:
+        return False
+    t.zero_()
+    invalidate_scale_cache()
+    logging.warning("comfyui_amd: a scale_input changed in place since its value was read; the output of the last "
+                    "forward that used it is NaN. Cached scale values dropped.")
+    return True
 
 
 def scale_value(p, use_cache=None):

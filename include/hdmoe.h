@@ -167,9 +167,12 @@ typedef struct hdmoe_ffn_weights {
   const float* scale_in2; /* scale_input of w2 */
   const float* scale_in3; /* scale_input of w3 */
   /* w1 and w3 read the same input, which the fused kernels quantise once, with scale_in1: the two scale_inputs must
-   * hold the same value. The library cannot compare device scalars without synchronising, so it accepts
-   * scale_in1 == scale_in3 as pointers (both NULL included) and, for two different non-NULL pointers, only a caller
-   * that sets this field to nonzero, asserting that the two values are equal; anything else is HDMOE_E_SHAPE. */
+   * give the same cast factor bf16(1 / scale_input). The host cannot compare device scalars without synchronising, so
+   * the entry points accept scale_in1 == scale_in3 as pointers (both NULL included) and, for two different non-NULL
+   * pointers, only a caller that sets this field to nonzero, asserting that the two values are equal; anything else
+   * is HDMOE_E_SHAPE. The kernel that casts compares the two factors on the device and writes NaN instead of a cast
+   * made with the wrong one (hdmoe_moe_ffn, hdmoe_ffn_swiglu). Each Linear's own scale_input value enters its
+   * output scale. */
   int same_scale_in13;
 } hdmoe_ffn_weights;
 
@@ -323,11 +326,18 @@ typedef struct hdmoe_layer_args {
   const void* mod_gate;
   int tokens_per_batch;
   float ln_eps;
-  /* fp8 only. When w1/w3 of every routed expert and of the shared expert have the same scale_input, the tokens are
-   * cast to e4m3fn once (one row per token instead of three) and every group of the gate/up GEMM reads that copy.
-   * The library sees this by itself when all those scale_in1 pointers are equal (all NULL included); nonzero here is
-   * the caller's assertion that different pointers hold the same value. */
+  /* fp8 only. When w1/w3 of every routed expert and of the shared expert cast the tokens with the same factor, the
+   * tokens are cast to e4m3fn once (one row per token instead of three) and every group of the gate/up GEMM reads
+   * that copy. Whether they do is decided on the device, by the kernel that casts, from the values behind the
+   * scale_in1 pointers at the time it runs (equal pointers and all-NULL are seen on the host). This field is a hint
+   * of earlier versions and is not looked at. */
   int uniform_scale_in;
+  /* Optional (may be NULL): one int32 the device can write (device memory, or pinned host memory through its device
+   * address). w1 and w3 of a feed-forward read one cast of the tokens, so same_scale_in13 of hdmoe_ffn_weights is an
+   * assertion about device values that the host may hold a stale copy of. The casting kernel verifies it: where the
+   * two factors differ it writes NaN rows (the output of the call is then NaN, not a wrong number) and sets this
+   * word to 1. A caller that caches its comparison of the values can poll the word and drop the cache. */
+  int32_t* scale_check;
 } hdmoe_layer_args;
 
 #define HDMOE_NUM_STAGES 6
@@ -350,7 +360,7 @@ int hdmoe_ffn_swiglu(int weight_dtype, const void* x_bf16, int rows, int D, int 
 /* Where the pieces of the workspace live, for tests that inspect intermediates. */
 typedef struct hdmoe_layer_layout {
   size_t topk_idx, topk_weight, counts, offsets, perm, inv_perm, dispatch_ws;
-  size_t a, h, y, normed, partials, total;
+  size_t a, h, y, normed, partials, flags, total;
 } hdmoe_layer_layout;
 int hdmoe_layer_layout_get(int T, int D, int H, int Hs, int E, int weight_dtype,
                            hdmoe_layer_layout* out);

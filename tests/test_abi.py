@@ -39,7 +39,7 @@ def test_header_constants_match_binding():
     assert (int(consts["HDMOE_E_NULL"]), int(consts["HDMOE_E_SHAPE"]), int(consts["HDMOE_E_WORKSPACE"]),
             int(consts["HDMOE_E_LAUNCH"])) == (_lib.E_NULL, _lib.E_SHAPE, _lib.E_WORKSPACE, _lib.E_LAUNCH)
     assert ctypes.sizeof(_lib.FfnWeights) == 10 * 8
-    assert ctypes.sizeof(_lib.LayerLayout) == 13 * 8
+    assert ctypes.sizeof(_lib.LayerLayout) == 14 * 8
 
 
 def test_struct_layouts_match_what_a_c_compiler_sees(tmp_path):

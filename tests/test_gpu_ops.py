@@ -263,40 +263,117 @@ def test_stacked_layers_at_32768_tokens(dev):
     """Stacked sweep (benchmark configuration 4) at its full depth: 48 independent fp8 layers at 2 x 16384 tokens,
     x <- x + FFN(LayerNorm(x)) with the block's affine-free LayerNorm (model.py:393,430) so the residual stream
     stays in range. Weights are drawn on the device (the CPU generator would need minutes for 11.5 GB) and copied
-    back for the oracle, which follows a token subset: tokens are independent through the whole stack. Every layer's
-    whole output must be finite and routing is compared bit for bit on the subset."""
-    from comfyui_amd import functional as HF
-    T, D, L = 32768, synth.DIM, 48
+    back for the oracle. Even layers take torch's LayerNorm and the plain layer; odd layers go through the block's
+    one-enqueue branch with a modulation (LayerNorm + modulation inside the gate kernel, gated residual inside the
+    combine), the form the benchmark of this configuration runs.
+
+    Every layer is called with its own workspace, and what is compared is what the layer itself decided: its routing
+    rows, its segment bounds and its permutation. On every layer a token subset is followed through the oracle
+    (tokens are independent through the whole stack); on layers 0, 23 and 47 ALL 32768 routing rows, the counts, the
+    offsets and both permutations are compared with the oracle bit for bit, and the output subset grows to 500+ tokens
+    that include the rows of the last, partial tile of every expert segment for both tile heights in use at this size,
+    the tile the shared expert ends in, and rows on either side of every tile boundary near a segment start."""
+    from comfyui_amd import _lib, functional as HF
+    T, D, L, E, B = 32768, synth.DIM, 48, 4, 2
+    S = T // B
+    FULL = (0, 23, 47)
     g = torch.Generator().manual_seed(99)
-    x0 = torch.randn((2, T // 2, D), generator=g).to(BF16)
-    sel = torch.randperm(T, generator=g)[:16].sort().values
-    xd = x0.to(dev)
+    x0 = torch.randn((B, S, D), generator=g).to(BF16)
+    base = torch.randperm(T, generator=g)[:32].sort().values
+    xd = x0.to(dev).reshape(T, D)
     ln = lambda t: torch.nn.functional.layer_norm(t.float(), (D,), eps=1e-6).to(BF16)
-    worst = dict(rel_rms=0.0, max_over_max=0.0)
+    worst = dict(rel_rms=0.0, max_over_rms=0.0, max_over_max=0.0)
+    lay = ws = None
     for layer in range(L):
         master, _ = synth.make_weights(layer, device=dev)
         sd_dev = synth.to_state_dict(master, "fp8")
         del master
         m = synth.build_module(sd_dev, "fp8", dev)
         sd = {k: v.cpu() for k, v in sd_dev.items()}
-        # the oracle starts every layer from the device's own residual stream (for the token subset): rounding
-        # differences of one layer would otherwise flip e4m3 neighbours in the next and the two runs drift apart
-        xs = xd.reshape(-1, D)[sel].cpu().unsqueeze(0)
-        hd = ln(xd)
-        idx_d, w_d = HF.gate_top2(hd.reshape(-1, D)[sel.to(dev)].contiguous(), m.gate.weight)
-        xd = xd + m(hd)
+        branch = layer % 2 == 1
+        full = layer in FULL
+        wdt, experts, shared, keep = m._collect(xd)
+        H, Hs = m.experts[0].w1.weight.shape[0], m.shared_experts.w1.weight.shape[0]
+        if lay is None:
+            lay = HF.layer_layout(T, D, H, Hs, E, _lib.W_E4M3FN)
+            ws = torch.empty(lay.total, dtype=torch.uint8, device=dev)
+        ws[:lay.a].fill_(0x5A)    # stale routing and permutation bytes: everything compared below must be rewritten
+        x_in = xd
+        if branch:
+            gm = torch.Generator().manual_seed(1000 + layer)
+            shift, scale = ((torch.randn((B, D), generator=gm) * 0.1).to(BF16) for _ in range(2))
+            gate_mlp = (1.0 + torch.randn((B, D), generator=gm) * 0.1).to(BF16)
+            out, idx_d, w_d = HF.moe_ffn(x_in, m.gate.device_weight(x_in), experts, shared, H, Hs, wdt, workspace=ws,
+                                         want_routing=True, uniform_scale_in=m._uniform_scale_in,
+                                         modulation=(shift.to(dev), scale.to(dev), gate_mlp.to(dev)), tokens_per_batch=S)
+            xd = out
+        else:
+            hd = ln(x_in)
+            out, idx_d, w_d = HF.moe_ffn(hd, m.gate.device_weight(hd), experts, shared, H, Hs, wdt, workspace=ws,
+                                         want_routing=True, uniform_scale_in=m._uniform_scale_in)
+            xd = x_in + out
         assert bool(torch.isfinite(xd.float()).all()), f"layer {layer}: non-finite residual stream"
-        h = ln(xs)
-        idx, w, _, _ = O.gate_fixed_order(h.reshape(-1, D), sd["gate.weight"])
-        assert torch.equal(idx_d.cpu(), idx) and torch.equal(w_d.cpu().view(torch.int16), w.view(torch.int16)), layer
-        ref = xs + O.moe_forward(h, oracle_params(sd, 4), "fp8mm", gate_result=(idx, w))
-        got = xd.reshape(-1, D)[sel].cpu()
-        met = O.error_metrics(got, ref.reshape(-1, D))
+        ints = lambda off, n: ws[off:off + 4 * n].view(torch.int32).cpu()
+        offsets_d, perm_d = ints(lay.offsets, E + 1), ints(lay.perm, 2 * T)
+        idx_d, w_d = idx_d.cpu(), w_d.cpu()
+
+        def normed(rows):
+            """Residual-stream rows and layer-input rows of tokens `rows` (ascending). The oracle starts every layer from
+            the device's own residual stream: rounding differences of one layer would otherwise flip e4m3 neighbours in
+            the next. In the branch form the LayerNorm + modulation are the library's and the oracle restates them."""
+            xs = x_in[rows.to(dev)].cpu()
+            if not branch:
+                return xs, hd[rows.to(dev)].cpu()   # torch's LayerNorm is the harness's, not the library's: taken as is
+            parts = []
+            for b in range(B):
+                r = xs[(rows >= b * S) & (rows < (b + 1) * S)]
+                if r.shape[0]:
+                    parts.append(O.ln_modulate_c(r, shift[b:b + 1], scale[b:b + 1], r.shape[0]))
+            return xs, torch.cat(parts)
+
+        sel = base
+        if full:
+            # routing of every token, and the dispatch it implies, against the oracle
+            _, h_all = normed(torch.arange(T))
+            idx_r, w_r, _, _ = O.gate_fixed_order(h_all, sd["gate.weight"])
+            assert torch.equal(idx_d, idx_r), f"layer {layer}: routing indices differ"
+            assert torch.equal(w_d.view(torch.int16), w_r.view(torch.int16)), f"layer {layer}: routing weights differ"
+            counts_r, offs_r, perm_r, inv_r = O.dispatch(idx_r, E)
+            assert torch.equal(ints(lay.counts, E), counts_r.to(torch.int32))
+            assert torch.equal(offsets_d, offs_r.to(torch.int32))
+            assert torch.equal(perm_d, perm_r.to(torch.int32)), f"layer {layer}: permutation differs"
+            assert torch.equal(ints(lay.inv_perm, 2 * T), inv_r.reshape(-1).to(torch.int32))
+            del h_all
+            offs = offsets_d.tolist()
+            picks = [base, torch.randperm(T, generator=g)[:160], torch.arange(T - 72, T), torch.arange(0, 24),
+                     torch.arange(S - 12, S + 12),
+                     torch.arange((T // 320) * 320 - 8, (T // 320) * 320 + 8), torch.arange(T - 256 - 8, T - 256 + 8)]
+            for e in range(E):
+                lo, hi = offs[e], offs[e + 1]
+                for tile in (256, 320):
+                    tail = lo + ((hi - lo) // tile) * tile          # first row of the segment's partial tile
+                    rows = torch.cat([torch.arange(max(lo, tail - 8), min(hi, tail + 24)), torch.arange(max(lo, hi - 24), hi),
+                                      torch.arange(lo, min(hi, lo + 12)), torch.arange(min(hi, lo + tile - 6), min(hi, lo + tile + 6))])
+                    picks.append(perm_d[rows].long() // 2)
+            sel = torch.unique(torch.cat(picks))
+            assert sel.numel() >= 500
+        xs, h = normed(sel)
+        idx, w, _, _ = O.gate_fixed_order(h, sd["gate.weight"])
+        assert torch.equal(idx_d[sel], idx) and torch.equal(w_d[sel].view(torch.int16), w.view(torch.int16)), layer
+        y = O.moe_forward(h.unsqueeze(0), oracle_params(sd, E), "fp8mm", gate_result=(idx, w)).reshape(-1, D)
+        if branch:
+            b_of = (sel // S).long()
+            ref = gate_mlp[b_of] * y + xs      # model.py:432-433 on bf16 tensors: product rounded, then the sum
+        else:
+            ref = xs + y
+        got = xd[sel.to(dev)].cpu()
+        met = O.error_metrics(got, ref)
         worst = {k: max(worst[k], met[k]) for k in worst}
-        if layer % 8 == 0 or layer == L - 1:
-            print(f"layer {layer}: rms(x)={float(got.float().pow(2).mean().sqrt()):.3f} {met}", flush=True)
-        assert met["rel_rms"] <= 1e-2 and met["max_over_max"] <= 3e-2, (layer, met)
-        del m, sd_dev, sd
+        if layer % 8 == 0 or full:
+            print(f"layer {layer} ({'branch' if branch else 'plain'}, {sel.numel()} tokens): "
+                  f"rms(x)={float(got.float().pow(2).mean().sqrt()):.3f} {met}", flush=True)
+        assert met["rel_rms"] <= 1e-2 and met["max_over_max"] <= 3e-2 and met["max_over_rms"] <= 3e-2, (layer, met)
+        del m, sd_dev, sd, keep
     print("worst over the stack", worst)
 
 

@@ -125,6 +125,24 @@ def test_bf16_rounding_points_match_torch_kernels():
     assert float((lg.softmax(-1).view(torch.int16) != sm.view(torch.int16)).float().mean()) < 2e-3
 
 
+def test_reference_bf16_dataflow_against_its_own_fp32_evaluation():
+    """What "within max-abs / RMS error 3e-2 of the reference computed in fp32" can mean. The reference's own dataflow
+    on a device rounds every intermediate to bf16 and casts two of them to e4m3; evaluated by the oracle on the CPU,
+    that dataflow and the same layer with fp32 intermediates differ by about 2e-2 in rms(err)/rms(ref) and in
+    max|err|/max|ref|, inside the tolerance, and by 0.1 and more in max|err|/rms(ref): the cross ratio of the largest
+    error to the typical output is several times the tolerance for the reference against itself, so it cannot be the
+    gate for an implementation of it. The GPU tests gate the first two and report the third."""
+    sd, x = small_layer(seed=2, dim=512, tokens=400, weights="fp8")
+    params = oracle_params(sd, 4)
+    idx, w, _, _ = O.gate_fixed_order(x.reshape(-1, 512), sd["gate.weight"])
+    as_run = O.moe_forward(x, params, "fp8mm", gate_result=(idx, w))
+    in_fp32 = O.moe_forward(x.float(), params, "fp8mm", gate_result=(idx, w.float()))
+    m = O.error_metrics(as_run, in_fp32)
+    print(m)
+    assert m["rel_rms"] <= 3e-2 and m["max_over_max"] <= 3e-2
+    assert m["max_over_rms"] > 2 * 3e-2
+
+
 def test_synth_configs_shapes():
     assert synth.H_ROUTED == 6912 and synth.H_SHARED == 3584
     master, g = synth.make_weights(0, dim=128, hidden_arg=384)
