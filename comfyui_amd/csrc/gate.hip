@@ -22,6 +22,7 @@
 namespace {
 
 constexpr int WAVES_PER_BLOCK = 4;
+constexpr int GATE_BLOCKS_PER_CU = 2;   // resident blocks per CU the grids are sized for
 
 __device__ __forceinline__ float exp_neg(float x) {
   // exp(x), x <= 0: ln2 split range reduction, degree-5 polynomial, exponent
@@ -238,9 +239,9 @@ __device__ __forceinline__ TokenWalk token_walk(int T, int tpb) {
   return {(int)blockIdx.x * WAVES_PER_BLOCK + wv, T, (int)gridDim.x * WAVES_PER_BLOCK};
 }
 
-template <int E>
+template <int E, int NWAVES = WAVES_PER_BLOCK>
 __device__ __forceinline__ void write_block_hist(const int (&cnt)[E], int32_t* __restrict__ block_hist) {
-  __shared__ int32_t wave_cnt[WAVES_PER_BLOCK][E];
+  __shared__ int32_t wave_cnt[NWAVES][E];
   if (block_hist == nullptr) return;  // kernel argument: the same for every thread
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   if (lane == 0) {
@@ -251,31 +252,170 @@ __device__ __forceinline__ void write_block_hist(const int (&cnt)[E], int32_t* _
   if (threadIdx.x < E) {
     int32_t sum = 0;
 #pragma unroll
-    for (int w = 0; w < WAVES_PER_BLOCK; ++w) sum += wave_cnt[w][threadIdx.x];
+    for (int w = 0; w < NWAVES; ++w) sum += wave_cnt[w][threadIdx.x];
     block_hist[(size_t)blockIdx.x * E + threadIdx.x] = sum;
   }
 }
 
+// ---- the kernel for D = NCHUNK * 512 and up to 4 experts ------------------------------------------------------
+// Two tokens per wave and trip. The gate weight sits in LDS as fp32 (E * D * 4 bytes: 40 KiB for HiDream), written
+// once per block, so that the dot products are fused multiply-adds on LDS operands with nothing to unpack but the
+// tokens, and one read of a weight slice serves both tokens. The 2 * E partial sums per lane are added up across the
+// wave in the butterfly order of wave_sum, but folded: at the step with offset 32 the lower half of the wave keeps
+// the sums of one expert and the upper half those of another (v[l] + v[l ^ 32] is the same number in both lanes, so
+// computing it once loses nothing), at offset 16 the four 16-lane rows end up with the four experts, and the last
+// four steps run on one register instead of four. Row e of that register then holds logit e; softmax is evaluated
+// once on the rows (its exponential and division once per token instead of once per expert), the E scores come
+// back through lane reads, and the top-2 selection and everything after it is wave-uniform.
+// Every floating-point operation has the operands and the order of the one-token form, so the results are the same
+// bit for bit.
+__device__ __forceinline__ float fold32(float a, float b) {
+  auto h = __builtin_amdgcn_permlane32_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+  return __uint_as_float(h[0]) + __uint_as_float(h[1]);   // lanes 0-31: a[l] + a[l + 32]; lanes 32-63: the same for b
+}
+__device__ __forceinline__ float fold16(float a, float b) {
+  auto h = __builtin_amdgcn_permlane16_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+  return __uint_as_float(h[0]) + __uint_as_float(h[1]);   // rows 0, 2: a's rows 0 + 1, 2 + 3; rows 1, 3: b's
+}
+__device__ __forceinline__ float row_sum(float v) {      // offsets 8, 4, 2, 1 inside every 16-lane row
+  int x = __float_as_int(v);
+  v = v + __int_as_float(__builtin_amdgcn_update_dpp(x, x, 0x128, 0xf, 0xf, false));  // row_ror:8
+  x = __float_as_int(v);
+  v = v + __int_as_float(__builtin_amdgcn_update_dpp(x, x, 0x124, 0xf, 0xf, false));  // row_ror:4
+  x = __float_as_int(v);
+  v = v + __int_as_float(__builtin_amdgcn_update_dpp(x, x, 0x4e, 0xf, 0xf, false));   // quad_perm:[2,3,0,1]
+  x = __float_as_int(v);
+  v = v + __int_as_float(__builtin_amdgcn_update_dpp(x, x, 0xb1, 0xf, 0xf, false));   // quad_perm:[1,0,3,2]
+  return v;
+}
+__device__ __forceinline__ float lane_value(float v, int lane) {
+  return __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(v), lane));
+}
+// partial sums of up to 4 experts -> one register whose 16-lane row e holds the wave total of expert e
+template <int E>
+__device__ __forceinline__ float expert_rows(const float (&acc)[E]) {
+  const float a0 = acc[0], a1 = acc[1], a2 = E > 2 ? acc[2] : 0.0f, a3 = E > 3 ? acc[3] : 0.0f;
+  return row_sum(fold16(fold32(a0, a2), fold32(a1, a3)));
+}
+
+// logits in rows -> routing of one token (wave-uniform): indices, the two scores
+template <int E>
+__device__ __forceinline__ void finish_rows(float rows, int& i0, int& i1, float& s0, float& s1) {
+  const float lg = GateBf16::round(rows);          // F.linear output is a bf16 tensor
+  float l[E];
+#pragma unroll
+  for (int e = 0; e < E; ++e) l[e] = lane_value(lg, 16 * e);
+  float mx = l[0];
+#pragma unroll
+  for (int e = 1; e < E; ++e) mx = l[e] > mx ? l[e] : mx;
+  const float ex = exp_neg(lg - mx);               // row e: exp(logit e - max); rows past E hold nothing of use
+  float sum = 0.0f;
+#pragma unroll
+  for (int e = 0; e < E; ++e) sum = sum + lane_value(ex, 16 * e);
+  const float sc = GateBf16::round(__fdiv_rn(ex, sum));   // so is the softmax output
+  float score[E];
+#pragma unroll
+  for (int e = 0; e < E; ++e) score[e] = lane_value(sc, 16 * e);
+  // first two of a stable descending sort: strict '>' keeps the lower index on ties
+  i0 = 0;
+  s0 = score[0];
+#pragma unroll
+  for (int e = 1; e < E; ++e)
+    if (score[e] > s0) { s0 = score[e]; i0 = e; }
+  i1 = -1;
+  s1 = 0.0f;
+#pragma unroll
+  for (int e = 0; e < E; ++e) {
+    if (e == i0) continue;
+    if (i1 < 0 || score[e] > s1) { s1 = score[e]; i1 = e; }
+  }
+}
+
+// Wave totals of a and of b (what wave_sum returns for each), as wave-uniform values: a in the lower half of the
+// wave, b in the upper half from the first step on.
+__device__ __forceinline__ void wave_sum2(float a, float b, float& ta, float& tb) {
+  float v = fold32(a, b);
+  const uint32_t u = __float_as_uint(v);
+  auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  v = row_sum(__uint_as_float(r[0]) + __uint_as_float(r[1]));
+  ta = lane_value(v, 0);
+  tb = lane_value(v, 32);
+}
+
+// LayerNorm statistics of two rows held in registers: ln_stats for each, the wave sums taken together
+template <int NCHUNK>
+__device__ __forceinline__ void ln_stats2(const uint4 (&va)[NCHUNK], const uint4 (&vb)[NCHUNK], float fD, float eps,
+                                          float& mean_a, float& rstd_a, float& mean_b, float& rstd_b) {
+  float sa = 0.0f, sb = 0.0f;
+#pragma unroll
+  for (int c = 0; c < NCHUNK; ++c) {
+    float f[8], g[8];
+    unpack8(va[c], f);
+    unpack8(vb[c], g);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) { sa = sa + f[j]; sb = sb + g[j]; }
+  }
+  float ta, tb;
+  wave_sum2(sa, sb, ta, tb);
+  mean_a = __fdiv_rn(ta, fD);
+  mean_b = __fdiv_rn(tb, fD);
+  float qa = 0.0f, qb = 0.0f;
+#pragma unroll
+  for (int c = 0; c < NCHUNK; ++c) {
+    float f[8], g[8];
+    unpack8(va[c], f);
+    unpack8(vb[c], g);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float da = f[j] - mean_a, db = g[j] - mean_b;
+      qa = __builtin_fmaf(da, da, qa);
+      qb = __builtin_fmaf(db, db, qb);
+    }
+  }
+  wave_sum2(qa, qb, ta, tb);
+  rstd_a = __fdiv_rn(1.0f, __builtin_sqrtf(__fdiv_rn(ta, fD) + eps));
+  rstd_b = __fdiv_rn(1.0f, __builtin_sqrtf(__fdiv_rn(tb, fD) + eps));
+}
+
 template <int E, int NCHUNK, bool QUANT, bool LN = false>
-__global__ __launch_bounds__(WAVES_PER_BLOCK * 64, 3) void gate_top2_reg_kernel(
+__global__ __launch_bounds__(WAVES_PER_BLOCK * 64, 2) void gate_top2_reg_kernel(
     const uint4* __restrict__ x, const uint4* __restrict__ wg, int T, int tpb, int32_t* __restrict__ idx,
     uint16_t* __restrict__ wout, int32_t* __restrict__ block_hist, GateQuant q) {
   const int lane = threadIdx.x & 63;
+  const int wv = threadIdx.x >> 6;
   constexpr int ROW16 = NCHUNK * 64;  // 16-byte units per row
-  const TokenWalk walk = token_walk(T, tpb);
-  int t = walk.first;
-  const int t_end = walk.end;
-  // the wave's first token is requested before the block copies the gate weight: the two latencies overlap
-  uint4 cur[NCHUNK], nxt[NCHUNK];
-  if (t < t_end) {
-#pragma unroll
-    for (int c = 0; c < NCHUNK; ++c) cur[c] = x[(size_t)t * ROW16 + c * 64 + lane];
+  // Pairs of consecutive tokens. tpb > 0: block b owns tokens [b * tpb, (b + 1) * tpb) and its waves take the pairs
+  // of that range in turn; tpb == 0: the waves of the grid stride over the pairs of all tokens (see TokenWalk).
+  int t0, t_end, step;
+  if (tpb > 0) {
+    t0 = (int)blockIdx.x * tpb + 2 * wv;
+    t_end = min(T, (int)(blockIdx.x + 1) * tpb);
+    step = 2 * WAVES_PER_BLOCK;
+  } else {
+    t0 = 2 * ((int)blockIdx.x * WAVES_PER_BLOCK + wv);
+    t_end = T;
+    step = 2 * (int)gridDim.x * WAVES_PER_BLOCK;
   }
-  // The gate weight (E rows) sits in LDS, not in registers: 80 registers less per lane, i.e. four waves per SIMD
-  // instead of two, which is what a kernel that only streams needs. A lane reads the same 16-byte units of every
-  // row for every token (lane-contiguous, conflict-free).
-  __shared__ uint4 w[E * ROW16];
-  for (int i = threadIdx.x; i < E * ROW16; i += WAVES_PER_BLOCK * 64) w[i] = wg[i];
+  // the wave's first pair is requested before the block fills LDS with the gate weight: the two latencies overlap.
+  // A pair whose second token lies past the end reads its first token twice and drops the copy's results.
+  uint4 cur0[NCHUNK], cur1[NCHUNK], nxt0[NCHUNK], nxt1[NCHUNK];
+  auto load_pair = [&](int t, uint4 (&a)[NCHUNK], uint4 (&b)[NCHUNK]) {
+    const int tb = t + 1 < t_end ? t + 1 : t;
+#pragma unroll
+    for (int c = 0; c < NCHUNK; ++c) a[c] = x[(size_t)t * ROW16 + c * 64 + lane];
+#pragma unroll
+    for (int c = 0; c < NCHUNK; ++c) b[c] = x[(size_t)tb * ROW16 + c * 64 + lane];
+  };
+  if (t0 < t_end) load_pair(t0, cur0, cur1);
+  // gate weight -> LDS as fp32. Unit (e, c, lane) of the bf16 weight (8 elements) becomes the two float4 at
+  // [(e * NCHUNK + c) * 2 + half][lane]: a lane's reads are 16 bytes wide and lane-contiguous (no bank conflicts).
+  __shared__ float4 wf[E * NCHUNK * 2 * 64];
+  for (int i = threadIdx.x; i < E * ROW16; i += WAVES_PER_BLOCK * 64) {
+    const uint4 v = wg[i];
+    const int unit = i >> 6, l = i & 63;
+    wf[(unit * 2 + 0) * 64 + l] = make_float4(bf16_lo(v.x), bf16_hi(v.x), bf16_lo(v.y), bf16_hi(v.y));
+    wf[(unit * 2 + 1) * 64 + l] = make_float4(bf16_lo(v.z), bf16_hi(v.z), bf16_lo(v.w), bf16_hi(v.w));
+  }
   __syncthreads();
 
   int cnt[E];
@@ -309,66 +449,92 @@ __global__ __launch_bounds__(WAVES_PER_BLOCK * 64, 3) void gate_top2_reg_kernel(
       if (!ok13 && q.scale_check != nullptr) *q.scale_check = 1;
     }
   }
-  for (; t < t_end; t += walk.step) {
-    const int tn = t + walk.step;
-    if (tn < t_end) {
-#pragma unroll
-      for (int c = 0; c < NCHUNK; ++c) nxt[c] = x[(size_t)tn * ROW16 + c * 64 + lane];
+  auto write_token = [&](int t, const uint4 (&row)[NCHUNK], int i0, int i1, float s0, float s1) {
+    if (lane == 0) {
+      reinterpret_cast<int2*>(idx)[t] = make_int2(i0, i1);
+      reinterpret_cast<uint32_t*>(wout)[t] = GateBf16::pack(s0, s1);
     }
-    if constexpr (LN) {
-      float mean, rstd;
-      ln_stats<NCHUNK>(cur, (float)(NCHUNK * 512), q.ln_eps, mean, rstd);
-      const size_t brow = (size_t)(t / q.tokens_per_batch) * ROW16;
-#pragma unroll
-      for (int c = 0; c < NCHUNK; ++c)
-        cur[c] = modulate8(cur[c], q.mod_scale[brow + c * 64 + lane], q.mod_shift[brow + c * 64 + lane], mean, rstd);
-    }
-    float logit[E];
-    // opaque per token, or the compiler hoists the E * NCHUNK weight reads out of the token loop and keeps the
-    // slice in registers after all
-    int wlane = lane;
-    asm volatile("" : "+v"(wlane));
-#pragma unroll
-    for (int e = 0; e < E; ++e) {
-      float acc = 0.0f;
-#pragma unroll
-      for (int c = 0; c < NCHUNK; ++c) {
-        acc = dot8(cur[c], w[e * ROW16 + c * 64 + wlane], acc);
-      }
-      logit[e] = acc;
-    }
-    int i0, i1;
-    finish_token<E>(logit, lane, t, idx, wout, i0, i1);
 #pragma unroll
     for (int e = 0; e < E; ++e) cnt[e] += (i0 == e) + (i1 == e);
     if constexpr (QUANT) {
-      float inv0 = inv_e[0], inv1 = inv_e[0];
-#pragma unroll
-      for (int e = 1; e < E; ++e) {
-        inv0 = i0 == e ? inv_e[e] : inv0;
-        inv1 = i1 == e ? inv_e[e] : inv1;
-      }
-      inv0 = hdmoe_q_uniform(inv0);
-      inv1 = hdmoe_q_uniform(inv1);
       if (one_row) {
         // one scale_input for all: one row per token
 #pragma unroll
-        for (int c = 0; c < NCHUNK; ++c) q.xq_shared[(size_t)t * ROW16 + c * 64 + lane] = hdmoe_q_8(cur[c], invs);
+        for (int c = 0; c < NCHUNK; ++c) q.xq_shared[(size_t)t * ROW16 + c * 64 + lane] = hdmoe_q_8(row[c], invs);
       } else {
+        float inv0 = inv_e[0], inv1 = inv_e[0];
+#pragma unroll
+        for (int e = 1; e < E; ++e) {
+          inv0 = i0 == e ? inv_e[e] : inv0;
+          inv1 = i1 == e ? inv_e[e] : inv1;
+        }
+        inv0 = hdmoe_q_uniform(inv0);
+        inv1 = hdmoe_q_uniform(inv1);
         uint2* r0 = q.xq_routed + (size_t)(2 * t) * ROW16;
         const bool same01 = inv0 == inv1, same0s = inv0 == invs;  // equal scales: cast once, store again
 #pragma unroll
         for (int c = 0; c < NCHUNK; ++c) {
-          const uint2 v0 = hdmoe_q_8(cur[c], inv0);
+          const uint2 v0 = hdmoe_q_8(row[c], inv0);
           r0[c * 64 + lane] = v0;
-          r0[ROW16 + c * 64 + lane] = same01 ? v0 : hdmoe_q_8(cur[c], inv1);
+          r0[ROW16 + c * 64 + lane] = same01 ? v0 : hdmoe_q_8(row[c], inv1);
           if (with_shared)
-            q.xq_shared[(size_t)t * ROW16 + c * 64 + lane] = same0s ? v0 : hdmoe_q_8(cur[c], invs);
+            q.xq_shared[(size_t)t * ROW16 + c * 64 + lane] = same0s ? v0 : hdmoe_q_8(row[c], invs);
         }
       }
     }
+  };
+  for (; t0 < t_end; t0 += step) {
+    const int tn = t0 + step;
+    if (tn < t_end) load_pair(tn, nxt0, nxt1);
+    const bool has1 = t0 + 1 < t_end;
+    if constexpr (LN) {
+      float m0, r0, m1, r1;
+      ln_stats2<NCHUNK>(cur0, cur1, (float)(NCHUNK * 512), q.ln_eps, m0, r0, m1, r1);
+      const int t1 = has1 ? t0 + 1 : t0;
+      const size_t b0 = (size_t)(t0 / q.tokens_per_batch) * ROW16, b1 = (size_t)(t1 / q.tokens_per_batch) * ROW16;
 #pragma unroll
-    for (int c = 0; c < NCHUNK; ++c) cur[c] = nxt[c];
+      for (int c = 0; c < NCHUNK; ++c) {
+        cur0[c] = modulate8(cur0[c], q.mod_scale[b0 + c * 64 + lane], q.mod_shift[b0 + c * 64 + lane], m0, r0);
+        cur1[c] = modulate8(cur1[c], q.mod_scale[b1 + c * 64 + lane], q.mod_shift[b1 + c * 64 + lane], m1, r1);
+      }
+    }
+    float acc0[E], acc1[E];
+#pragma unroll
+    for (int e = 0; e < E; ++e) acc0[e] = acc1[e] = 0.0f;
+    // opaque per trip, or the compiler hoists the weight reads out of the token loop and keeps the slice in registers
+    int wlane = lane;
+    asm volatile("" : "+v"(wlane));
+#pragma unroll
+    for (int c = 0; c < NCHUNK; ++c) {
+      float xa[8], xb[8];
+      unpack8(cur0[c], xa);
+      unpack8(cur1[c], xb);
+#pragma unroll
+      for (int e = 0; e < E; ++e) {
+        const float4 wlo = wf[((e * NCHUNK + c) * 2 + 0) * 64 + wlane], whi = wf[((e * NCHUNK + c) * 2 + 1) * 64 + wlane];
+        const float w8[8] = {wlo.x, wlo.y, wlo.z, wlo.w, whi.x, whi.y, whi.z, whi.w};
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          acc0[e] = __builtin_fmaf(xa[j], w8[j], acc0[e]);
+          acc1[e] = __builtin_fmaf(xb[j], w8[j], acc1[e]);
+        }
+      }
+      // nothing moves across: the scheduler would otherwise issue the weight reads of every chunk up front and keep
+      // E * D / 64 values live
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // both tokens' sums are formed here: left to itself the compiler sinks the second token's arithmetic into the
+    // branch that stores its results and keeps the whole weight slice in registers until then
+#pragma unroll
+    for (int e = 0; e < E; ++e) asm volatile("" : "+v"(acc0[e]), "+v"(acc1[e]));
+    int i0, i1, j0, j1;
+    float s0, s1, u0, u1;
+    finish_rows<E>(expert_rows<E>(acc0), i0, i1, s0, s1);
+    finish_rows<E>(expert_rows<E>(acc1), j0, j1, u0, u1);
+    write_token(t0, cur0, i0, i1, s0, s1);
+    if (has1) write_token(t0 + 1, cur1, j0, j1, u0, u1);
+#pragma unroll
+    for (int c = 0; c < NCHUNK; ++c) { cur0[c] = nxt0[c]; cur1[c] = nxt1[c]; }
   }
   write_block_hist<E>(cnt, block_hist);
 }
@@ -437,11 +603,13 @@ __global__ __launch_bounds__(WAVES_PER_BLOCK * 64) void gate_top2_generic_kernel
 template <int E>
 int launch_gate(const void* x, const void* wg, int T, int D, int32_t* idx, void* w, const GateQuant* quant,
                 int32_t* block_hist, hipStream_t s, const char* what, bool f16) {
-  // with histograms: block ranges; without: waves strided over the tokens, at least two tokens per wave to pay for
-  // the block's copy of the gate weight into LDS and at most three blocks per CU (all resident)
-  const int tpb = block_hist != nullptr ? hdmoe_gate_tokens_per_block(T) : 0;
+  // with histograms: block ranges; without: waves strided over the tokens (the register kernel: over token pairs),
+  // at least two tokens per wave, and no more blocks than are resident at once
+  const bool reg_kernel = !f16 && E <= 4 && D == 2560;
+  const int tpb = block_hist != nullptr ? hdmoe_gate_tokens_per_block(T, D, E) : 0;
   int blocks = tpb > 0 ? (T + tpb - 1) / tpb : (T + WAVES_PER_BLOCK * 2 - 1) / (WAVES_PER_BLOCK * 2);
-  if (tpb == 0 && blocks > HDMOE_NUM_CU * 3) blocks = HDMOE_NUM_CU * 3;
+  const int resident = HDMOE_NUM_CU * (reg_kernel ? GATE_BLOCKS_PER_CU : 3);
+  if (tpb == 0 && blocks > resident) blocks = resident;
   dim3 grid(blocks < 1 ? 1 : blocks), block(WAVES_PER_BLOCK * 64);
   const uint4* xp = static_cast<const uint4*>(x);
   const uint4* wp = static_cast<const uint4*>(wg);
@@ -564,22 +732,25 @@ extern "C" int hdmoe_gate_top2_f16(const void* x_f16, const void* gate_w_f16, in
                        static_cast<hipStream_t>(stream), "hdmoe_gate_top2_f16", true);
 }
 
-// Tokens per block of the gate kernels, a pure function of T: the grid is three blocks per CU, all resident at once
-// (the register kernels hold 12 waves per CU), with at least one token per wave (a few hundred tokens then spread over
-// more blocks: 2 us off the 256-token gate against two tokens per wave, nothing lost at 4096 tokens, where a block
-// holds 6 tokens instead of 8); very large T gets more blocks instead of more than 1024 tokens each (the
-// dispatch's scatter pass handles one or several whole blocks per chunk, at most 1024 tokens).
-int hdmoe_gate_tokens_per_block(int T) {
-  const int resident = HDMOE_NUM_CU * 3;
+// Tokens per block of the gate kernels of the one-call layer, a pure function of the sizes. Register kernel (two
+// tokens per wave and trip): two blocks per CU, all resident at once, each block a whole number of token pairs per
+// wave. Generic kernel: three blocks per CU, at least one token per wave. Very large T gets more blocks instead of
+// more than 1024 tokens each (the dispatch's scatter pass handles one or several whole blocks per chunk, at most 1024
+// tokens).
+int hdmoe_gate_tokens_per_block(int T, int D, int E) {
+  const bool reg_kernel = E <= 4 && D == 2560;
+  const int resident = HDMOE_NUM_CU * (reg_kernel ? GATE_BLOCKS_PER_CU : 3);
+  const int unit = reg_kernel ? 2 * WAVES_PER_BLOCK : WAVES_PER_BLOCK;
   int tpb = (T + resident - 1) / resident;
-  if (tpb < WAVES_PER_BLOCK) tpb = WAVES_PER_BLOCK;
+  tpb = (tpb + unit - 1) / unit * unit;
+  if (tpb < unit) tpb = unit;
   if (tpb > 1024) tpb = 1024;
   return tpb;
 }
 
 // Bytes of the per-block expert histograms the gate kernels can leave for the dispatch.
-size_t hdmoe_gate_hist_bytes(int T, int E) {
-  const int tpb = hdmoe_gate_tokens_per_block(T);
+size_t hdmoe_gate_hist_bytes(int T, int D, int E) {
+  const int tpb = hdmoe_gate_tokens_per_block(T, D, E);
   const size_t blocks = T > 0 ? ((size_t)T + tpb - 1) / tpb : 1;
   return hdmoe_align_up(blocks * (size_t)E * sizeof(int32_t), 256);
 }
