@@ -162,7 +162,64 @@ def aux_kernels(dev, module, x):
         flop = tokens * 3 * 2 * 2 * dim * inner
         return {"ms": r["ms"], "tokens": tokens, "TFLOPs": flop / r["ms"] / 1e9, "frac_of_mfma_peak": flop / r["ms"] / 1e9 / PEAK_BF16_TFLOPS}
 
+    def fp8_gemm_vs_vendor():
+        """One plain fp8 Linear, out = bf16((a . w^T) * scale), through this library's kernel (hdmoe_linear: the K loop of
+        the feed-forward kernels with the trivial epilogue) and through torch._scaled_mm (the vendor library) on the same
+        operands: e4m3fn casts of N(0,1) values, the data the matrix cores' clock depends on. M x N x K."""
+        rows = []
+        gg = torch.Generator(device=dev).manual_seed(5)
+        one = torch.ones((), dtype=torch.float32, device=dev)
+        for M, N, K in ((16384, 16384, 2560), (16384, 13824, 2560), (16384, 2560, 6912), (16384, 16384, 16384)):
+            a = torch.randn((M, K), generator=gg, device=dev).to(torch.float8_e4m3fn)
+            w = torch.randn((N, K), generator=gg, device=dev).to(torch.float8_e4m3fn)
+            flop = 2.0 * M * N * K
+            ours = timed(lambda: HF.linear(a, w, one, one), 0, reps=10)
+            entry = {"M": M, "N": N, "K": K, "hdmoe_linear_ms": ours["ms"], "hdmoe_linear_TFLOPs": flop / ours["ms"] / 1e9}
+            try:
+                theirs = timed(lambda: torch._scaled_mm(a, w.t(), scale_a=one, scale_b=one, out_dtype=torch.bfloat16), 0, reps=10)
+                entry.update({"scaled_mm_ms": theirs["ms"], "scaled_mm_TFLOPs": flop / theirs["ms"] / 1e9})
+            except (RuntimeError, NotImplementedError) as e:
+                entry["scaled_mm_error"] = str(e)[:200]
+            rows.append(entry)
+            del a, w
+        return rows
+
+    def mfma_ceiling():
+        """The matrix cores alone: a loop of fp8 MFMAs on register operands (csrc/mfma_probe.hip), one block of 8 waves
+        per CU as the GEMM kernels run, on zeros and on e4m3fn casts of N(0,1) values. Rate from events around the
+        launch; the clock from the kernel's own cycle counter against the device's constant-rate counter."""
+        path = os.path.join(ROOT, "comfyui_amd", "libhdmoe_probe.so")
+        if not os.path.exists(path):
+            return {"error": "libhdmoe_probe.so is not built (python -m comfyui_amd.build)"}
+        probe = ctypes.CDLL(path)
+        probe.hdmoe_probe_mfma_fp8.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
+                                               ctypes.c_void_p, ctypes.c_void_p]
+        blocks, iters, nacc = 256, 4000, probe.hdmoe_probe_accumulators()
+        wall_khz = probe.hdmoe_probe_wall_clock_khz()
+        ticks = torch.zeros(2, dtype=torch.int64, device=dev)
+        sink = torch.zeros(1, dtype=torch.float32, device=dev)
+        gg = torch.Generator(device=dev).manual_seed(6)
+        data = {"zeros": torch.zeros(blocks * 512 * 64, dtype=torch.uint8, device=dev),
+                "normal": torch.randn(blocks * 512 * 64, generator=gg, device=dev).to(torch.float8_e4m3fn).view(torch.uint8)}
+        out = {}
+        stream = torch.cuda.current_stream().cuda_stream
+        for form, name, per in ((0, "32x32x64", 131072), (1, "16x16x128", 65536)):
+            for kind, buf in data.items():
+                run = lambda: probe.hdmoe_probe_mfma_fp8(form, buf.data_ptr(), blocks, iters, ticks.data_ptr(), sink.data_ptr(), stream)
+                r = timed(run, 0, reps=10)
+                flop = float(blocks) * 8 * iters * nacc * per
+                t = ticks.cpu().tolist()
+                entry = {"ms": r["ms"], "TFLOPs": flop / r["ms"] / 1e9, "frac_of_published_peak": flop / r["ms"] / 1e9 / PEAK_FP8_TFLOPS}
+                if wall_khz > 0 and t[1] > 0:
+                    # the first wave's cycle counter against the constant-rate counter over its own run: the clock
+                    # the matrix cores sustained under this instruction on this data
+                    entry["shader_clock_GHz"] = t[0] / t[1] * wall_khz / 1e6
+                out[f"{name}_{kind}"] = entry
+        return out
+
     return {
+        "fp8_gemm_vs_vendor": fp8_gemm_vs_vendor(),
+        "mfma_ceiling": mfma_ceiling(),
         "hunyuan3d_moe_block_bf16": hunyuan_block(torch.bfloat16),
         "hunyuan3d_moe_block_fp16": hunyuan_block(torch.float16),
         "ln_modulate": timed(lambda: HF.ln_modulate(x2, scale, shift, S), 2 * T * D * 2),
@@ -183,7 +240,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--aux-kernels", action="store_true",
                     help="also time the stand-alone kernels outside the layer (LayerNorm+modulation, gated-residual "
-                         "combine, stochastic rounding of one expert weight) and report them under \"aux\"")
+                         "combine, stochastic rounding of one expert weight), the plain fp8 Linear against the vendor "
+                         "library's on the feed-forward's shapes and the matrix cores' own rate, and report them under "
+                         "\"aux\"")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also run one plain 256 MiB device copy, whose FETCH_SIZE/WRITE_SIZE readings calibrate the counters")
     args = ap.parse_args()
@@ -396,6 +455,11 @@ def main():
     }
     if args.aux_kernels:
         out["aux"] = aux_kernels(dev, module, x)
+        ceiling = out["aux"]["mfma_ceiling"].get("32x32x64_normal") if fp8 else None
+        if ceiling:
+            # the dominant kernel against what its own MFMA instruction sustains on this data on this device
+            out["roofline"]["measured_ceiling_TFLOPs"] = ceiling["TFLOPs"]
+            out["roofline"]["frac_of_measured_ceiling"] = gemm1_tflops / ceiling["TFLOPs"]
     if not args.no_cpu_baseline:
         del module
         torch.cuda.empty_cache()

@@ -106,6 +106,9 @@ SIGNATURES = {
     "hdmoe_grouped_linear_f16": (c_int, [c_void_p, c_void_p, c_int, c_int, ctypes.POINTER(LinearWeights), c_void_p,
                                          c_void_p, c_int, ctypes.POINTER(LinearWeights), c_void_p, c_int, c_int, c_int,
                                          c_void_p]),
+    "hdmoe_grouped_linear_tokens": (c_int, [c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, ctypes.POINTER(LinearWeights),
+                                            c_void_p, ctypes.POINTER(LinearWeights), c_void_p, c_int, c_int, c_int,
+                                            c_void_p]),
     "hdmoe_stochastic_round_e4m3fn": (c_int, [c_int, c_void_p, ctypes.c_int64, c_void_p, ctypes.c_uint64, c_void_p,
                                               c_void_p]),
     "hdmoe_ln_modulate_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, ctypes.c_float, c_void_p,

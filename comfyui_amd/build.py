@@ -11,6 +11,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libhdmoe.so")
+PROBE_LIB = os.path.join(HERE, "libhdmoe_probe.so")
 SOURCES = ["gate.hip", "dispatch.hip", "elementwise.hip", "gemm.hip", "layer.hip", "weights.hip"]
 
 HIPCC_FLAGS = [
@@ -55,6 +56,14 @@ def build(verbose=True, extra_flags=()):
     subprocess.check_call(cmd)
     # an unresolved symbol (e.g. a kernel stub the host pass dropped) must fail the build, not the first call
     subprocess.check_call([sys.executable, "-c", f"import ctypes; ctypes.CDLL({LIB!r})"])
+    # measurement support for bench.py --aux-kernels (the matrix cores' own rate); not part of the product library
+    cmd = [hipcc, *HIPCC_FLAGS, *extra_flags, "-shared", "-o", PROBE_LIB, os.path.join(CSRC, "mfma_probe.hip")]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    out = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if out.returncode != 0:
+        print(out.stdout, file=sys.stderr)
+        raise RuntimeError("hipcc failed: mfma_probe.hip")
     return LIB
 
 

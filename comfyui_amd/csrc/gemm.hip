@@ -1524,7 +1524,11 @@ int hdmoe_down_parts(int rows_dyn, int n_dyn, int rows_static, int N, int K_dyn,
 int hdmoe_launch_linear_groups(const uint8_t* a_dyn, const int32_t* offsets, int rows_dyn, int n_dyn,
                                const hdmoe_linear_weights* experts, uint8_t* out_dyn, const uint8_t* a_static,
                                int rows_static, const hdmoe_linear_weights* shared, uint8_t* out_static, int K, int N,
-                               int act, hipStream_t s, const char* what, bool f16 = false) {
+                               int act, hipStream_t s, const char* what, bool f16 = false,
+                               const int32_t* gather = nullptr, int gather_rows = 0, int gather_shift = 0) {
+  if (gather != nullptr && (unsigned long long)gather_rows * K * 2 >= (1ull << 31))
+    return hdmoe_fail(HDMOE_E_SHAPE, "%s: %d gathered rows of %d bytes exceed the 2 GiB offset range", what, gather_rows,
+                      K * 2);
   GemmArgs args;
   memset(&args, 0, sizeof(args));
   args.nparts = 1;
@@ -1542,6 +1546,9 @@ int hdmoe_launch_linear_groups(const uint8_t* a_dyn, const int32_t* offsets, int
     GemmGroup& gg = args.g[G];
     fill(gg, experts[e]);
     gg.a = a_dyn;
+    gg.gather = gather;
+    gg.gather_shift = gather_shift;
+    gg.a_rows = gather_rows;
     gg.out = out_dyn;
     gg.row_begin = -1;
     gg.dyn = e;
@@ -1692,7 +1699,9 @@ namespace {
 int grouped_linear_entry(const char* what, bool f16, const void* a_bf16, const int32_t* offsets, int rows_total, int E,
                          const hdmoe_linear_weights* experts, void* out_bf16, const void* a_static_bf16,
                          int rows_static, const hdmoe_linear_weights* shared, void* out_static_bf16, int K, int N, int act,
-                         hdmoe_stream_t stream) {
+                         hdmoe_stream_t stream, const int32_t* perm = nullptr, int T = 0) {
+  if (perm != nullptr && (T <= 0 || rows_total != T * HDMOE_TOPK))
+    return hdmoe_fail(HDMOE_E_SHAPE, "%s: rows_total=%d is not %d slots of T=%d tokens", what, rows_total, HDMOE_TOPK, T);
   if (E < 0 || E > HDMOE_MAX_EXPERTS) return hdmoe_fail(HDMOE_E_SHAPE, "%s: E=%d", what, E);
   if (act != HDMOE_ACT_NONE && act != HDMOE_ACT_GELU) return hdmoe_fail(HDMOE_E_SHAPE, "%s: act=%d", what, act);
   if (E > 0) {
@@ -1713,7 +1722,7 @@ int grouped_linear_entry(const char* what, bool f16, const void* a_bf16, const i
   return hdmoe_launch_linear_groups(static_cast<const uint8_t*>(a_bf16), offsets, rows_total, rows_total > 0 ? E : 0,
                                     experts, static_cast<uint8_t*>(out_bf16), static_cast<const uint8_t*>(a_static_bf16),
                                     rows_static, shared, static_cast<uint8_t*>(out_static_bf16), K, N, act,
-                                    static_cast<hipStream_t>(stream), what, f16);
+                                    static_cast<hipStream_t>(stream), what, f16, perm, T, perm != nullptr ? 1 : 0);
 }
 }  // namespace
 
@@ -1731,4 +1740,20 @@ extern "C" int hdmoe_grouped_linear_f16(const void* a_f16, const int32_t* offset
                                         int K, int N, int act, hdmoe_stream_t stream) {
   return grouped_linear_entry("hdmoe_grouped_linear_f16", true, a_f16, offsets, rows_total, E, experts, out_f16,
                               a_static_f16, rows_static, shared, out_static_f16, K, N, act, stream);
+}
+
+// The first Linear of the experts on the tokens themselves: sorted row r is token perm[r] / 2 (the rows the boolean
+// masks of the reference select, read through the dispatch permutation instead of from a copy in expert order).
+extern "C" int hdmoe_grouped_linear_tokens(int act_dtype, const void* x, int T, const int32_t* perm,
+                                           const int32_t* offsets, int E, const hdmoe_linear_weights* experts, void* out,
+                                           const hdmoe_linear_weights* shared, void* out_shared, int K, int N, int act,
+                                           hdmoe_stream_t stream) {
+  HDMOE_REQUIRE_PTR(perm);
+  if (act_dtype != HDMOE_W_BF16 && act_dtype != HDMOE_W_F16)
+    return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_grouped_linear_tokens: act_dtype=%d is neither HDMOE_W_BF16 nor HDMOE_W_F16",
+                      act_dtype);
+  if (T < 0 || E < 1) return hdmoe_fail(HDMOE_E_SHAPE, "hdmoe_grouped_linear_tokens: T=%d E=%d", T, E);
+  if (T == 0) return HDMOE_OK;
+  return grouped_linear_entry("hdmoe_grouped_linear_tokens", act_dtype == HDMOE_W_F16, x, offsets, T * HDMOE_TOPK, E,
+                              experts, out, x, shared != nullptr ? T : 0, shared, out_shared, K, N, act, stream, perm, T);
 }

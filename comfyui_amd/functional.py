@@ -237,6 +237,29 @@ def grouped_linear(a_sorted, offsets, experts, a_static=None, shared=None, act="
     return out, out_static
 
 
+def grouped_linear_tokens(x2d, perm, offsets, experts, shared=None, act="none"):
+    """The first Linear (+ bias, + erf GELU) of every expert on the rows of `x2d` [T, K] its segment selects through
+    the dispatch permutation (sorted row r = token perm[r] // 2; nothing is copied into expert order), and of
+    `shared` (weight, bias) on all T rows, in one launch. Returns (out_sorted [2T, N], out_shared [T, N] or None)."""
+    code = {"none": _lib.ACT_NONE, "gelu": _lib.ACT_GELU}[act]
+    dt = _act_dtype(x2d, "grouped_linear_tokens x")
+    _need_hip(x2d, "grouped_linear_tokens x", dt)
+    T, K = x2d.shape
+    N = experts[0][0].shape[0]
+    E = len(experts)
+    arr = (LinearWeights * E)(*[_linear_weights(w, b, K, N, f"grouped_linear_tokens expert {i}", dt)
+                                for i, (w, b) in enumerate(experts)])
+    out = torch.empty((T * _lib.TOPK, N), dtype=dt, device=x2d.device)
+    out_shared, sh = None, None
+    if shared is not None:
+        sh = _linear_weights(shared[0], shared[1], K, N, "grouped_linear_tokens shared", dt)
+        out_shared = torch.empty((T, N), dtype=dt, device=x2d.device)
+    check(lib.hdmoe_grouped_linear_tokens(_lib.W_BF16 if dt == BF16 else _lib.W_F16, ptr(x2d), T, ptr(perm), ptr(offsets), E,
+                                          arr, ptr(out), ctypes.byref(sh) if sh is not None else None, ptr(out_shared),
+                                          K, N, code, _stream(x2d)))
+    return out, out_shared
+
+
 def stochastic_round_e4m3fn(weight, scale=None, seed=0):
     """weight (fp32 or bf16, HIP) / scale (fp32 scalar tensor or None) -> float8_e4m3fn by stochastic rounding
     (comfy/float.py:14-67 behind comfy/ops.py:419-426), one kernel."""

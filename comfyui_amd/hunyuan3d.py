@@ -155,8 +155,8 @@ class MoEBlock(nn.Module):
         gate_w = amd_ops.cast_to(self.gate.weight, dtype=x2.dtype, device=x2.device).contiguous()
         idx, w = HF.gate_top2(x2, gate_w)
         _, offsets, perm, inv_perm = HF.dispatch(idx, self.num_experts)
-        xs = HF.permute_bf16(x2, perm)
         if not (all(e.fusable(x2) for e in self.experts) and self.shared_experts.fusable(x2)):
+            xs = HF.permute_bf16(x2, perm)
             y = torch.empty_like(xs)
             bounds = offsets.tolist()  # host sync: segment sizes steer the per-expert calls
             for i, expert in enumerate(self.experts):
@@ -167,6 +167,7 @@ class MoEBlock(nn.Module):
         stage1 = [e.stage_weights()[0] for e in self.experts]
         stage2 = [e.stage_weights()[1] for e in self.experts]
         sh1, sh2 = self.shared_experts.stage_weights()
-        h, h_sh = HF.grouped_linear(xs, offsets, stage1, a_static=x2, shared=sh1, act="gelu")
+        # the experts' first Linear reads the routed rows through the permutation: no copy in expert order
+        h, h_sh = HF.grouped_linear_tokens(x2, perm, offsets, stage1, shared=sh1, act="gelu")
         y, y_sh = HF.grouped_linear(h, offsets, stage2, a_static=h_sh, shared=sh2, act="none")
         return HF.combine(y, inv_perm, w, y_sh).view(*orig_shape)

@@ -262,6 +262,15 @@ int hdmoe_grouped_linear_f16(const void* a_f16, const int32_t* offsets, int rows
                              int rows_static, const hdmoe_linear_weights* shared, void* out_static_f16, int K,
                              int N, int act, hdmoe_stream_t stream);
 
+/* The same Linear as the first stage of a block, on the tokens themselves: expert e multiplies the rows its segment of
+ * the dispatch holds, sorted row r being token perm[r] / 2 of x [T,K] (the rows `hidden_states[idx]` of
+ * comfy/ldm/hunyuan3dv2_1/hunyuandit.py:176-186 select, read through the permutation instead of from a copy in
+ * expert order), and the shared expert (NULL = none) all T rows. out [2T,N], out_shared [T,N]; act_dtype
+ * HDMOE_W_BF16 or HDMOE_W_F16 is the element type of x, weights, biases and outputs. */
+int hdmoe_grouped_linear_tokens(int act_dtype, const void* x, int T, const int32_t* perm, const int32_t* offsets, int E,
+                                const hdmoe_linear_weights* experts, void* out, const hdmoe_linear_weights* shared,
+                                void* out_shared, int K, int N, int act, hdmoe_stream_t stream);
+
 /* Weight maintenance of a scaled-fp8 Linear (comfy/ops.py:419-426 set_weight, comfy/float.py:14-67):
  * out[i] = stochastic_round_e4m3fn( float16( src[i] / *scale_dev ) ), scale_dev NULL = 1. Each value lands on one of
  * its two e4m3fn neighbours, the upper one with probability equal to its position between them; |v| >= 448
