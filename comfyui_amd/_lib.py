@@ -60,7 +60,7 @@ class LayerArgs(ctypes.Structure):
         ("stage_events", ctypes.POINTER(c_void_p)),
         ("mod_scale", c_void_p), ("mod_shift", c_void_p), ("mod_gate", c_void_p),
         ("tokens_per_batch", c_int), ("ln_eps", ctypes.c_float), ("uniform_scale_in", c_int),
-        ("scale_check", c_void_p),
+        ("scale_check", c_void_p), ("fixed_k_cut", c_int),
     ]
 
 

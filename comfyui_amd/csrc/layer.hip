@@ -272,6 +272,11 @@ extern "C" int hdmoe_moe_ffn(const hdmoe_layer_args* p, hdmoe_stream_t stream) {
   // down projections, both in one launch
   HdmoeSplitPlan plan;  // candidate cuts; the kernels pick one by the real segment sizes
   const int parts = hdmoe_down_parts((int)n, E, Hs > 0 ? T : 0, D, H, Hs, wd, &plan);
+  if (p->fixed_k_cut != 0 && plan.n > 1) {  // the cost model's entry, whatever the routing
+    plan.pd[0] = plan.pd[plan.n - 1];
+    plan.ps[0] = plan.ps[plan.n - 1];
+    plan.n = 1;
+  }
   if (int rc = hdmoe_launch_ffn_gemm(false, wd, h_routed, offsets, (int)n, E, p->experts, y_routed, h_shared,
                                      Hs > 0 ? T : 0, p->shared, y_shared, H, D, Hs, D, s, "hdmoe_moe_ffn (down)",
                                      nullptr, 0, parts > 1 ? reinterpret_cast<float*>(ws + l.partials) : nullptr, parts,

@@ -390,12 +390,14 @@ def layer_layout(T, D, H, Hs, E, code):
 
 def moe_ffn(x2d, gate_w, experts, shared, H, Hs, weight_dtype, out=None, workspace=None, want_routing=False,
             stage_events=None, modulation=None, tokens_per_batch=None, ln_eps=1e-6, uniform_scale_in=False,
-            scale_check=None):
+            scale_check=None, fixed_k_cut=False):
     """The whole layer as one enqueue. experts: list of FfnWeights, shared: FfnWeights or None.
     modulation=(shift, scale, gate), each [B, D] bf16, turns the call into the block's feed-forward branch:
     out = x + gate * layer(LayerNorm(x) * (1 + scale) + shift), with T == B * tokens_per_batch.
     uniform_scale_in: accepted and not used (the casting kernel compares the scale_input values on the device and
     casts the tokens once when they agree).
+    fixed_k_cut: the K cut of the down projection (small token counts) is taken from the sizes alone instead of from
+    the segment sizes of the call, so that a row's bytes do not depend on the routing of the other rows.
     scale_check: optional pinned int32 tensor of one element that the casting kernel sets to 1 when w1 and w3 of a
     feed-forward turn out to cast the tokens differently (the output is then NaN).
     Returns out [T,D] bf16 (and topk_idx int32, topk_weight bf16 when want_routing)."""
@@ -423,6 +425,7 @@ def moe_ffn(x2d, gate_w, experts, shared, H, Hs, weight_dtype, out=None, workspa
         args.shared = ctypes.pointer(sh)
     args.out, args.workspace, args.workspace_bytes = ptr(out), ptr(workspace), workspace.numel()
     args.uniform_scale_in = 1 if uniform_scale_in else 0
+    args.fixed_k_cut = 1 if fixed_k_cut else 0
     if scale_check is not None:
         if scale_check.dtype != torch.int32 or scale_check.numel() < 1 or not (scale_check.is_cuda or scale_check.is_pinned()):
             raise TypeError("moe_ffn: scale_check must be an int32 tensor on the device or in pinned host memory")

@@ -228,6 +228,11 @@ class MOEFeedForwardSwiGLU(nn.Module):
                             operations=operations)
         self.num_activated_experts = num_activated_experts
 
+    # Not an attribute of the reference class. Set `module.batch_invariant = True` to have every token's output bytes
+    # independent of how the other tokens of the batch are routed: between a few hundred and about two thousand tokens
+    # the down projection is cut along K and the cut that runs is otherwise picked from the experts' segment sizes,
+    # which changes the fp32 summation order (the last bit of an output) with the rest of the batch.
+
     # ---- fused path ----------------------------------------------------------------
 
     def _collect(self, x):
@@ -281,7 +286,8 @@ class MOEFeedForwardSwiGLU(nn.Module):
             H = self.experts[0].w1.weight.shape[0]
             Hs = self.shared_experts.w1.weight.shape[0]
             y = HF.moe_ffn(x2, gate_w, experts, shared, H, Hs, wdt, stage_events=stage_events,
-                           scale_check=amd_ops.scale_check_word(x2.device) if wdt == FP8 else None)
+                           scale_check=amd_ops.scale_check_word(x2.device) if wdt == FP8 else None,
+                           fixed_k_cut=self.__dict__.get("batch_invariant", False))
             del keep
             return y.view(*orig_shape)
         return self._forward_composed(x2, gate_w).view(*orig_shape)
@@ -306,6 +312,7 @@ class MOEFeedForwardSwiGLU(nn.Module):
             Hs = self.shared_experts.w1.weight.shape[0]
             y = HF.moe_ffn(x2, gate_w, experts, shared, H, Hs, wdt, stage_events=stage_events, modulation=mods,
                            scale_check=amd_ops.scale_check_word(x2.device) if wdt == FP8 else None,
+                           fixed_k_cut=self.__dict__.get("batch_invariant", False),
                            tokens_per_batch=S, ln_eps=eps)
             del keep
             return y.view(B, S, D)

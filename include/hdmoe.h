@@ -347,6 +347,13 @@ typedef struct hdmoe_layer_args {
    * two factors differ it writes NaN rows (the output of the call is then NaN, not a wrong number) and sets this
    * word to 1. A caller that caches its comparison of the values can poll the word and drop the cache. */
   int32_t* scale_check;
+  /* With a few hundred to about two thousand tokens the down projection is cut along K, and which of the candidate
+   * cuts runs is chosen on the device from the experts' segment sizes (the cut that fills one round of blocks). The
+   * fp32 summation order of a row then depends on how the OTHER tokens of the batch were routed: the same token can
+   * differ in the last bit of its output between two batches. Nonzero here fixes the cut from the sizes alone (the
+   * cost model's choice), which makes every row's bytes a function of that row, its expert's weights and T only, at
+   * 2 to 10 % of the layer's time at those sizes. */
+  int fixed_k_cut;
 } hdmoe_layer_args;
 
 #define HDMOE_NUM_STAGES 6

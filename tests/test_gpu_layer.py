@@ -543,3 +543,38 @@ def test_combine_over_the_partial_sums_of_a_cut_down_projection(dev, weights, to
     assert bool(torch.isfinite(out.float()).all()) and float(out.float().abs().max()) > 0
     assert torch.equal(out.view(torch.int16), want.view(torch.int16))
     del keep
+
+
+def test_rows_do_not_depend_on_the_rest_of_the_batch_when_asked(dev):
+    """At 1024 tokens of HiDream's width the down projection is cut along K and the entry of the plan that runs is
+    picked on the device from the experts' segment sizes, so the fp32 summation order of a token's rows may follow the
+    routing of the other tokens. Two batches that share their first 256 tokens and route the other 768 differently
+    (evenly, with segments that do not fit the first candidate cut / all to the experts of one token, where it fits):
+    with `batch_invariant` set the cut is the same whatever the routing and the shared tokens come out byte for byte
+    the same. (Where both entries happen to hold the same cut they do so without the flag as well; the count printed
+    below says which.)"""
+    cfg = synth.make_config("cfg2")
+    sd = synth.to_state_dict(cfg["master"], "fp8")
+    m = synth.build_module({k: v.to(dev) for k, v in sd.items()}, "fp8", dev)
+    xall = cfg["x"].reshape(-1, synth.DIM)
+    tiles = lambda xs: int(sum(-(-int(c) // 256) for c in torch.bincount(
+        O.gate_fixed_order(xs, sd["gate.weight"])[0].reshape(-1).long(), minlength=4)))
+    # a batch whose experts' segments make 11 or more 256-token tiles (three experts above 512 rows): the cut in
+    # (2, 1) parts then does not fit one round of blocks and another runs; and one with 10 or fewer, where it does
+    start = next(s0 for s0 in range(0, 3072, 64) if tiles(xall[s0:s0 + 1024]) >= 11)
+    xa = xall[start:start + 1024].clone()
+    xb = xa.clone()
+    xb[256:] = xa[300]                                 # 768 copies of one token: two experts take them all
+    assert tiles(xa) >= 11 and tiles(xb) <= 10, (tiles(xa), tiles(xb))
+    outs = {}
+    for flag in (False, True):
+        m.batch_invariant = flag
+        ya = m(xa.to(dev).unsqueeze(0))[0, :256].cpu()
+        yb = m(xb.to(dev).unsqueeze(0))[0, :256].cpu()
+        outs[flag] = (ya, yb)
+    differ = int((outs[False][0].view(torch.int16) != outs[False][1].view(torch.int16)).sum())
+    print(f"\n{differ} of {256 * synth.DIM} outputs of the shared tokens differ between the batches without the flag")
+    assert torch.equal(outs[True][0].view(torch.int16), outs[True][1].view(torch.int16))
+    ref = O.moe_forward(xa[:256].unsqueeze(0), oracle_params(sd, 4), "fp8mm")[0]
+    met = O.error_metrics(outs[True][0], ref)
+    assert met["rel_rms"] <= TOL_RMS_SAME_DATAFLOW["fp8"] and met["max_over_max"] <= TOL["fp8"], met
