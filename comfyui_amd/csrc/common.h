@@ -44,9 +44,11 @@ static inline int hdmoe_check_scale_in13(const char* what, const hdmoe_ffn_weigh
 
 static inline size_t hdmoe_align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
-// gate kernels: tokens per block (a pure function of T) and the bytes of the per-block expert histograms
-int hdmoe_gate_tokens_per_block(int T, int D, int E);
-size_t hdmoe_gate_hist_bytes(int T, int D, int E);
+// gate kernels: which kernel casts (with_cast: fp8 experts; with_ln: LayerNorm + modulation inside the kernel), its
+// tokens per block (a pure function of the sizes) and the bytes of the per-block expert histograms
+bool hdmoe_gate_splits_roles(int D, int E, bool with_cast, bool with_ln);
+int hdmoe_gate_tokens_per_block(int T, int D, int E, bool with_cast, bool with_ln);
+size_t hdmoe_gate_hist_bytes(int T, int D, int E, bool with_cast);
 
 // Few rows per segment: one m-tile per group and the experts' 256-token tiles half empty on average (up to 256 tokens
 // in a top-2 layer of 4 experts). Such launches run in the forms of the GEMM kernels that skip padding, and their down

@@ -539,6 +539,213 @@ __global__ __launch_bounds__(WAVES_PER_BLOCK * 64, 2) void gate_top2_reg_kernel(
   write_block_hist<E>(cnt, block_hist);
 }
 
+// ---- routing and cast by different waves ------------------------------------------------------------------
+// Eight waves per block, two blocks per CU. Waves 0-3 route: one token per trip, the next token's row requested a
+// trip ahead, the dot products as above (fp32 gate weight in LDS, folded wave sums); their only stores are the 12
+// bytes of routing per token. Waves 4-7 cast: they load the same tokens, cast them and store the fp8 rows, two rows
+// in flight, and never touch the gate weight (they pass the fill barrier at once). A wave that does both computes,
+// then casts and stores, and while its stores and the next loads queue up behind those of every other wave its
+// arithmetic cannot issue (instructions issue in order); with two kinds of wave the arithmetic of one overlaps the
+// memory traffic of the other, and sixteen waves per CU instead of eight cover each other's waits. The second read
+// of a row comes from cache: both waves of a token sit on one CU and ask for it at about the same time.
+// Measured inside the layer (kernel start to last store, 8192 / 4096 / 256 tokens): 19 / 12 / 7 us against
+// 24 / 18 / 11 us of the kernel above doing both in every wave.
+// The split needs a cast that does not depend on the routing, i.e. one cast factor for every expert. Where the
+// scale values say otherwise (decided here, on the device) the cast waves wait, and behind a barrier all eight
+// waves write the per-slot rows from the routing the first four have left in idx.
+// Every floating-point operation of the routing has the operands and the order of the one-token form: same bits.
+constexpr int ROLE_WAVES = 4;          // waves per role and block
+constexpr int ROLES_BLOCKS_PER_CU = 2;
+constexpr int WEIGHT_READAHEAD = 3;    // (chunk, expert) steps the LDS reads run ahead of the arithmetic
+
+template <int E, int NCHUNK>
+__global__ __launch_bounds__(2 * ROLE_WAVES * 64, 2 * ROLES_BLOCKS_PER_CU) void gate_cast_roles_kernel(
+    const uint4* __restrict__ x, const uint4* __restrict__ wg, int T, int tpb, int32_t* __restrict__ idx,
+    uint16_t* __restrict__ wout, int32_t* __restrict__ block_hist, GateQuant q) {
+  const int lane = threadIdx.x & 63;
+  const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int rw = wv % ROLE_WAVES;
+  const bool caster = wv >= ROLE_WAVES;
+  constexpr int ROW16 = NCHUNK * 64;
+  // the tokens of wave rw of either role: block ranges or grid-strided (see TokenWalk)
+  int t0, t_end, step;
+  if (tpb > 0) {
+    t0 = (int)blockIdx.x * tpb + rw;
+    t_end = min(T, (int)(blockIdx.x + 1) * tpb);
+    step = ROLE_WAVES;
+  } else {
+    t0 = (int)blockIdx.x * ROLE_WAVES + rw;
+    t_end = T;
+    step = (int)gridDim.x * ROLE_WAVES;
+  }
+  const int t_first = t0;
+  uint4 row[NCHUNK], nxt[NCHUNK];
+  auto load_row = [&](int t, uint4 (&r)[NCHUNK]) {
+#pragma unroll
+    for (int c = 0; c < NCHUNK; ++c) r[c] = x[(size_t)t * ROW16 + c * 64 + lane];
+  };
+  // gate weight -> LDS as fp32 (layout as in gate_top2_reg_kernel), by the routing waves, requested in front of
+  // their first row
+  __shared__ float4 wf[E * NCHUNK * 2 * 64];
+  constexpr int FILL = (E * ROW16 + ROLE_WAVES * 64 - 1) / (ROLE_WAVES * 64);
+  uint4 wpart[FILL];
+  if (!caster) {
+#pragma unroll
+    for (int k = 0; k < FILL; ++k) {
+      const int i = threadIdx.x + k * ROLE_WAVES * 64;
+      wpart[k] = i < E * ROW16 ? wg[i] : make_uint4(0, 0, 0, 0);
+    }
+  }
+  if (t0 < t_end) load_row(t0, row);
+  // the scale values are asked for before the barrier, so that their latency passes behind it
+  float sc1[E], sc3[E];
+#pragma unroll
+  for (int e = 0; e < E; ++e) {
+    sc1[e] = q.scale_in.p[e] != nullptr ? *q.scale_in.p[e] : 0.0f;
+    sc3[e] = q.scale_in3.p[e] != nullptr ? *q.scale_in3.p[e] : 0.0f;
+  }
+  const float scs1 = q.shared_scale != nullptr ? *q.shared_scale : 0.0f;
+  const float scs3 = q.shared_scale3 != nullptr ? *q.shared_scale3 : 0.0f;
+  if (!caster) {
+#pragma unroll
+    for (int k = 0; k < FILL; ++k) {
+      const int i = threadIdx.x + k * ROLE_WAVES * 64;
+      if (i < E * ROW16) {
+        const uint4 v = wpart[k];
+        const int unit = i >> 6, l = i & 63;
+        wf[(unit * 2 + 0) * 64 + l] = make_float4(bf16_lo(v.x), bf16_hi(v.x), bf16_lo(v.y), bf16_hi(v.y));
+        wf[(unit * 2 + 1) * 64 + l] = make_float4(bf16_lo(v.z), bf16_hi(v.z), bf16_lo(v.w), bf16_hi(v.w));
+      }
+    }
+  }
+  __syncthreads();
+
+  // decisions and checks on the scale values (see GateQuant); NULL pointer: the clamp rule's marker
+  auto inv_of = [](const float* p, float v) { return p == nullptr ? -1.0f : hdmoe_dev_round_bf16(__fdiv_rn(1.0f, v)); };
+  float inv_e[E];
+  bool ok13 = true, same = true;
+#pragma unroll
+  for (int e = 0; e < E; ++e) {
+    inv_e[e] = hdmoe_q_uniform(inv_of(q.scale_in.p[e], sc1[e]));
+    if (q.scale_in3.p[e] != q.scale_in.p[e]) ok13 = ok13 && inv_of(q.scale_in3.p[e], sc3[e]) == inv_e[e];
+  }
+  float invs = hdmoe_q_uniform(inv_of(q.shared_scale, scs1));
+  if (q.shared_scale3 != q.shared_scale) ok13 = ok13 && inv_of(q.shared_scale3, scs3) == invs;
+#pragma unroll
+  for (int e = 0; e < E; ++e) same = same && inv_e[e] == invs;
+  const bool one_row = q.decide ? same : q.xq_routed == nullptr;
+  const bool with_shared = q.decide ? q.with_shared != 0 : q.xq_shared != nullptr;
+  if (!ok13) {
+    invs = __builtin_nanf("");   // every product and so every byte written below is NaN
+#pragma unroll
+    for (int e = 0; e < E; ++e) inv_e[e] = invs;
+  }
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    if (q.decide) *q.layout_flag = same ? 1 : 0;
+    if (!ok13 && q.scale_check != nullptr) *q.scale_check = 1;
+  }
+  int cnt[E];
+#pragma unroll
+  for (int e = 0; e < E; ++e) cnt[e] = 0;
+  if (!caster) {
+    for (; t0 < t_end; t0 += step) {
+      const int tn = t0 + step;
+      if (tn < t_end) load_row(tn, nxt);
+      float acc[E];
+#pragma unroll
+      for (int e = 0; e < E; ++e) acc[e] = 0.0f;
+      // Step s = c * E + e multiplies chunk c with the weight unit of expert e. The LDS reads run WEIGHT_READAHEAD
+      // steps ahead of the arithmetic and no further: each step's empty statement defines the lane offset the next
+      // reads use and consumes the sum of the step before, so the compiler can neither gather the reads at the top
+      // of the trip (the whole slice in registers) nor hoist them out of the token loop.
+      constexpr int RA = WEIGHT_READAHEAD, STEPS = NCHUNK * E;
+      int wlane = lane;
+      asm volatile("" : "+v"(wlane));
+      float4 wlo[RA], whi[RA];
+#pragma unroll
+      for (int s = 0; s < RA && s < STEPS; ++s) {
+        const int u = (s % E) * NCHUNK + s / E;
+        wlo[s] = wf[(u * 2 + 0) * 64 + wlane];
+        whi[s] = wf[(u * 2 + 1) * 64 + wlane];
+      }
+#pragma unroll
+      for (int c = 0; c < NCHUNK; ++c) {
+        float xa[8];
+        unpack8(row[c], xa);
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+          const int st = c * E + e;
+          const float4 lo = wlo[st % RA], hi = whi[st % RA];
+          if (st + RA < STEPS) {
+            const int u = ((st + RA) % E) * NCHUNK + (st + RA) / E;
+            asm volatile("" : "+v"(wlane), "+v"(acc[e == 0 ? E - 1 : e - 1]));
+            wlo[st % RA] = wf[(u * 2 + 0) * 64 + wlane];
+            whi[st % RA] = wf[(u * 2 + 1) * 64 + wlane];
+          }
+          const float w8[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+#pragma unroll
+          for (int j = 0; j < 8; ++j) acc[e] = __builtin_fmaf(xa[j], w8[j], acc[e]);
+        }
+      }
+      int i0, i1;
+      float s0, s1;
+      finish_rows<E>(expert_rows<E>(acc), i0, i1, s0, s1);
+      if (lane == 0) {
+        reinterpret_cast<int2*>(idx)[t0] = make_int2(i0, i1);
+        reinterpret_cast<uint32_t*>(wout)[t0] = GateBf16::pack(s0, s1);
+      }
+#pragma unroll
+      for (int e = 0; e < E; ++e) cnt[e] += (i0 == e) + (i1 == e);
+#pragma unroll
+      for (int c = 0; c < NCHUNK; ++c) row[c] = nxt[c];
+    }
+  } else if (one_row) {
+    // two rows in flight: the cast itself is a few instructions, the wave's time is memory latency
+    if (t0 + step < t_end) load_row(t0 + step, nxt);
+    for (; t0 < t_end; t0 += 2 * step) {
+      auto cast_row = [&](int t, uint4 (&r)[NCHUNK]) {
+        if (t >= t_end) return;
+        uint2 o[NCHUNK];
+#pragma unroll
+        for (int c = 0; c < NCHUNK; ++c) o[c] = hdmoe_q_8(r[c], invs);
+        if (t + 2 * step < t_end) load_row(t + 2 * step, r);
+#pragma unroll
+        for (int c = 0; c < NCHUNK; ++c) q.xq_shared[(size_t)t * ROW16 + c * 64 + lane] = o[c];
+      };
+      cast_row(t0, row);
+      cast_row(t0 + step, nxt);
+    }
+  }
+  if (!one_row) {
+    // a cast per slot: all eight waves, from the routing the first four have written (the barrier makes a block's
+    // own global stores visible to its waves)
+    __syncthreads();
+    for (int t = t_first + (wv / ROLE_WAVES) * step; t < t_end; t += 2 * step) {
+      load_row(t, row);
+      const int2 r = reinterpret_cast<const int2*>(idx)[t];
+      const int i0 = __builtin_amdgcn_readfirstlane(r.x), i1 = __builtin_amdgcn_readfirstlane(r.y);
+      float inv0 = inv_e[0], inv1 = inv_e[0];
+#pragma unroll
+      for (int e = 1; e < E; ++e) {
+        inv0 = i0 == e ? inv_e[e] : inv0;
+        inv1 = i1 == e ? inv_e[e] : inv1;
+      }
+      inv0 = hdmoe_q_uniform(inv0);
+      inv1 = hdmoe_q_uniform(inv1);
+      uint2* r0 = q.xq_routed + (size_t)(2 * t) * ROW16;
+      const bool same01 = inv0 == inv1, same0s = inv0 == invs;  // equal scales: cast once, store again
+#pragma unroll
+      for (int c = 0; c < NCHUNK; ++c) {
+        const uint2 v0 = hdmoe_q_8(row[c], inv0);
+        r0[c * 64 + lane] = v0;
+        r0[ROW16 + c * 64 + lane] = same01 ? v0 : hdmoe_q_8(row[c], inv1);
+        if (with_shared) q.xq_shared[(size_t)t * ROW16 + c * 64 + lane] = same0s ? v0 : hdmoe_q_8(row[c], invs);
+      }
+    }
+  }
+  write_block_hist<E, 2 * ROLE_WAVES>(cnt, block_hist);
+}
+
 // Any D that is a multiple of 8: Wg is re-read through the cache hierarchy.
 template <int E, bool QUANT, class A = GateBf16>
 __global__ __launch_bounds__(WAVES_PER_BLOCK * 64) void gate_top2_generic_kernel(
@@ -603,34 +810,38 @@ __global__ __launch_bounds__(WAVES_PER_BLOCK * 64) void gate_top2_generic_kernel
 template <int E>
 int launch_gate(const void* x, const void* wg, int T, int D, int32_t* idx, void* w, const GateQuant* quant,
                 int32_t* block_hist, hipStream_t s, const char* what, bool f16) {
-  // with histograms: block ranges; without: waves strided over the tokens (the register kernel: over token pairs),
+  // with histograms: block ranges; without: waves strided over the tokens (gate_top2_reg_kernel: over token pairs),
   // at least two tokens per wave, and no more blocks than are resident at once
   const bool reg_kernel = !f16 && E <= 4 && D == 2560;
-  const int tpb = block_hist != nullptr ? hdmoe_gate_tokens_per_block(T, D, E) : 0;
-  int blocks = tpb > 0 ? (T + tpb - 1) / tpb : (T + WAVES_PER_BLOCK * 2 - 1) / (WAVES_PER_BLOCK * 2);
-  const int resident = HDMOE_NUM_CU * (reg_kernel ? GATE_BLOCKS_PER_CU : 3);
+  const bool ln = quant != nullptr && quant->mod_scale != nullptr;
+  const bool roles = !f16 && hdmoe_gate_splits_roles(D, E, quant != nullptr, ln);
+  const int tpb = block_hist != nullptr ? hdmoe_gate_tokens_per_block(T, D, E, quant != nullptr, ln) : 0;
+  const int per_trip = roles ? ROLE_WAVES : 2 * WAVES_PER_BLOCK;
+  int blocks = tpb > 0 ? (T + tpb - 1) / tpb : (T + per_trip - 1) / per_trip;
+  const int resident = HDMOE_NUM_CU * (roles ? ROLES_BLOCKS_PER_CU : reg_kernel ? GATE_BLOCKS_PER_CU : 3);
   if (tpb == 0 && blocks > resident) blocks = resident;
-  dim3 grid(blocks < 1 ? 1 : blocks), block(WAVES_PER_BLOCK * 64);
+  dim3 grid(blocks < 1 ? 1 : blocks), block((roles ? 2 * ROLE_WAVES : WAVES_PER_BLOCK) * 64);
   const uint4* xp = static_cast<const uint4*>(x);
   const uint4* wp = static_cast<const uint4*>(wg);
   uint16_t* wo = static_cast<uint16_t*>(w);
   GateQuant q;
   memset(&q, 0, sizeof(q));
   if (quant) q = *quant;
-  constexpr int ER = E <= 4 ? E : 4;  // the register kernel is only instantiated for up to 4 experts
+  constexpr int ER = E <= 4 ? E : 4;  // the register kernels are only instantiated for up to 4 experts
   if (f16) {
     if (quant) return hdmoe_fail(HDMOE_E_SHAPE, "%s: the fp8 cast takes bf16 activations", what);
     hipLaunchKernelGGL((gate_top2_generic_kernel<E, false, GateF16>), grid, block, 0, s, xp, wp, T, D, tpb, idx, wo,
                        block_hist, q);
-  } else if (E <= 4 && D == 2560) {
-    if (quant && q.mod_scale != nullptr)
+  } else if (roles) {
+    hipLaunchKernelGGL((gate_cast_roles_kernel<ER, 5>), grid, block, 0, s, xp, wp, T, tpb, idx, wo, block_hist, q);
+  } else if (reg_kernel) {
+    // the cast without the LayerNorm goes to gate_cast_roles_kernel
+    if (quant)
       hipLaunchKernelGGL((gate_top2_reg_kernel<ER, 5, true, true>), grid, block, 0, s, xp, wp, T, tpb, idx, wo, block_hist, q);
-    else if (quant)
-      hipLaunchKernelGGL((gate_top2_reg_kernel<ER, 5, true>), grid, block, 0, s, xp, wp, T, tpb, idx, wo, block_hist, q);
     else
       hipLaunchKernelGGL((gate_top2_reg_kernel<ER, 5, false>), grid, block, 0, s, xp, wp, T, tpb, idx, wo, block_hist, q);
   } else {
-    if (q.mod_scale != nullptr) return hdmoe_fail(HDMOE_E_SHAPE, "%s: the LayerNorm variant needs D = 2560 and E <= 4", what);
+    if (ln) return hdmoe_fail(HDMOE_E_SHAPE, "%s: the LayerNorm variant needs D = 2560 and E <= 4", what);
     if (quant)
       hipLaunchKernelGGL((gate_top2_generic_kernel<E, true>), grid, block, 0, s, xp, wp, T, D, tpb, idx, wo, block_hist, q);
     else
@@ -732,15 +943,23 @@ extern "C" int hdmoe_gate_top2_f16(const void* x_f16, const void* gate_w_f16, in
                        static_cast<hipStream_t>(stream), "hdmoe_gate_top2_f16", true);
 }
 
-// Tokens per block of the gate kernels of the one-call layer, a pure function of the sizes. Register kernel (two
-// tokens per wave and trip): two blocks per CU, all resident at once, each block a whole number of token pairs per
-// wave. Generic kernel: three blocks per CU, at least one token per wave. Very large T gets more blocks instead of
-// more than 1024 tokens each (the dispatch's scatter pass handles one or several whole blocks per chunk, at most 1024
-// tokens).
-int hdmoe_gate_tokens_per_block(int T, int D, int E) {
+// Which of the gate + cast kernels a launch gets: the one with routing and cast waves takes the cast without the
+// LayerNorm at the register kernels' shape (with the LayerNorm both kinds of wave would compute it, and at 32768
+// tokens, where the kernel is bound by its arithmetic, that costs 20 us).
+bool hdmoe_gate_splits_roles(int D, int E, bool with_cast, bool with_ln) {
+  return E <= 4 && D == 2560 && with_cast && !with_ln;
+}
+
+// Tokens per block of the gate kernels of the one-call layer, a pure function of the sizes and of the kernel.
+// Register kernel (two tokens per wave and trip) and the kernel with routing and cast waves (one token per routing
+// wave and trip): two blocks per CU, all resident at once, each block a whole number of trips. Generic kernel: three
+// blocks per CU, at least one token per wave. Very large T gets more blocks instead of more than 1024 tokens each
+// (the dispatch's scatter pass handles one or several whole blocks per chunk, at most 1024 tokens).
+int hdmoe_gate_tokens_per_block(int T, int D, int E, bool with_cast, bool with_ln) {
   const bool reg_kernel = E <= 4 && D == 2560;
-  const int resident = HDMOE_NUM_CU * (reg_kernel ? GATE_BLOCKS_PER_CU : 3);
-  const int unit = reg_kernel ? 2 * WAVES_PER_BLOCK : WAVES_PER_BLOCK;
+  const bool roles = hdmoe_gate_splits_roles(D, E, with_cast, with_ln);
+  const int resident = HDMOE_NUM_CU * (roles ? ROLES_BLOCKS_PER_CU : reg_kernel ? GATE_BLOCKS_PER_CU : 3);
+  const int unit = roles ? ROLE_WAVES : (reg_kernel ? 2 * WAVES_PER_BLOCK : WAVES_PER_BLOCK);
   int tpb = (T + resident - 1) / resident;
   tpb = (tpb + unit - 1) / unit * unit;
   if (tpb < unit) tpb = unit;
@@ -748,11 +967,16 @@ int hdmoe_gate_tokens_per_block(int T, int D, int E) {
   return tpb;
 }
 
-// Bytes of the per-block expert histograms the gate kernels can leave for the dispatch.
-size_t hdmoe_gate_hist_bytes(int T, int D, int E) {
-  const int tpb = hdmoe_gate_tokens_per_block(T, D, E);
-  const size_t blocks = T > 0 ? ((size_t)T + tpb - 1) / tpb : 1;
-  return hdmoe_align_up(blocks * (size_t)E * sizeof(int32_t), 256);
+// Bytes of the per-block expert histograms the gate kernels can leave for the dispatch: enough for either kernel
+// a layer of these sizes may get.
+size_t hdmoe_gate_hist_bytes(int T, int D, int E, bool with_cast) {
+  size_t most = 0;
+  for (int ln = 0; ln < (with_cast ? 2 : 1); ++ln) {
+    const int tpb = hdmoe_gate_tokens_per_block(T, D, E, with_cast, ln != 0);
+    const size_t blocks = T > 0 ? ((size_t)T + tpb - 1) / tpb : 1;
+    if (blocks > most) most = blocks;
+  }
+  return hdmoe_align_up(most * (size_t)E * sizeof(int32_t), 256);
 }
 
 // The same gate for the one-call layer, which also takes the histograms.

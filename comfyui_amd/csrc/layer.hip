@@ -69,7 +69,7 @@ extern "C" int hdmoe_layer_layout_get(int T, int D, int H, int Hs, int E, int we
   out->inv_perm = take(n * 4);
   // per-block expert histograms of the gate kernel (the first pass of the dispatch)
   {
-    const size_t a = hdmoe_gate_hist_bytes(T, D, E), b = hdmoe_dispatch_workspace_bytes(T, E);
+    const size_t a = hdmoe_gate_hist_bytes(T, D, E, fp8), b = hdmoe_dispatch_workspace_bytes(T, E);
     out->dispatch_ws = take(a > b ? a : b);
   }
   // a (fp8 only; bf16 weights multiply the tokens themselves): the tokens' e4m3fn rows per flat slot [2T,D], then
@@ -234,7 +234,7 @@ extern "C" int hdmoe_moe_ffn(const hdmoe_layer_args* p, hdmoe_stream_t stream) {
   mark();
   if (hist != nullptr) {
     if (int rc = hdmoe_launch_dispatch_scatter(idx, T, E, counts, offsets, perm, inv_perm, hist,
-                                               hdmoe_gate_tokens_per_block(T, D, E), s, "hdmoe_moe_ffn (dispatch)"))
+                                               hdmoe_gate_tokens_per_block(T, D, E, fp8, ln_in_gate), s, "hdmoe_moe_ffn (dispatch)"))
       return rc;
   } else {
     if (int rc = hdmoe_dispatch(idx, T, E, counts, offsets, perm, inv_perm, dispatch_ws,
