@@ -46,7 +46,6 @@ static inline size_t hdmoe_align_up(size_t v, size_t a) { return (v + a - 1) / a
 
 // gate kernels: which kernel casts (with_cast: fp8 experts; with_ln: LayerNorm + modulation inside the kernel), its
 // tokens per block (a pure function of the sizes) and the bytes of the per-block expert histograms
-bool hdmoe_gate_splits_roles(int D, int E, bool with_cast, bool with_ln);
 int hdmoe_gate_tokens_per_block(int T, int D, int E, bool with_cast, bool with_ln);
 size_t hdmoe_gate_hist_bytes(int T, int D, int E, bool with_cast);
 

@@ -22,7 +22,6 @@
 namespace {
 
 constexpr int WAVES_PER_BLOCK = 4;
-constexpr int GATE_BLOCKS_PER_CU = 2;   // resident blocks per CU the grids are sized for
 
 __device__ __forceinline__ float exp_neg(float x) {
   // exp(x), x <= 0: ln2 split range reduction, degree-5 polynomial, exponent
@@ -257,18 +256,18 @@ __device__ __forceinline__ void write_block_hist(const int (&cnt)[E], int32_t* _
   }
 }
 
-// ---- the kernel for D = NCHUNK * 512 and up to 4 experts ------------------------------------------------------
-// Two tokens per wave and trip. The gate weight sits in LDS as fp32 (E * D * 4 bytes: 40 KiB for HiDream), written
-// once per block, so that the dot products are fused multiply-adds on LDS operands with nothing to unpack but the
-// tokens, and one read of a weight slice serves both tokens. The 2 * E partial sums per lane are added up across the
-// wave in the butterfly order of wave_sum, but folded: at the step with offset 32 the lower half of the wave keeps
-// the sums of one expert and the upper half those of another (v[l] + v[l ^ 32] is the same number in both lanes, so
-// computing it once loses nothing), at offset 16 the four 16-lane rows end up with the four experts, and the last
-// four steps run on one register instead of four. Row e of that register then holds logit e; softmax is evaluated
-// once on the rows (its exponential and division once per token instead of once per expert), the E scores come
-// back through lane reads, and the top-2 selection and everything after it is wave-uniform.
-// Every floating-point operation has the operands and the order of the one-token form, so the results are the same
-// bit for bit.
+// ---- the kernels for D = NCHUNK * 512 and up to 4 experts -----------------------------------------------------
+// One token per wave and trip, sixteen waves per CU. The gate weight sits in LDS as fp32 (E * D * 4 bytes: 40 KiB
+// for HiDream), written once per block, so that the dot products are fused multiply-adds on LDS operands with
+// nothing to unpack but the token. The E partial sums per lane are added up across the wave in the butterfly order
+// of wave_sum, but folded: at the step with offset 32 the lower half of the wave keeps the sums of one expert and
+// the upper half those of another (v[l] + v[l ^ 32] is the same number in both lanes, so computing it once loses
+// nothing), at offset 16 the four 16-lane rows end up with the four experts, and the last four steps run on one
+// register instead of four. Row e of that register then holds logit e; softmax is evaluated once on the rows (its
+// exponential and division once per token instead of once per expert), the E scores come back through lane reads,
+// and the top-2 selection and everything after it is wave-uniform.
+// Every floating-point operation has the operands and the order of the plain one-token form (dot8, wave_sum,
+// finish_token), so the results are the same bit for bit.
 __device__ __forceinline__ float fold32(float a, float b) {
   auto h = __builtin_amdgcn_permlane32_swap(__float_as_uint(a), __float_as_uint(b), false, false);
   return __uint_as_float(h[0]) + __uint_as_float(h[1]);   // lanes 0-31: a[l] + a[l + 32]; lanes 32-63: the same for b
@@ -331,252 +330,170 @@ __device__ __forceinline__ void finish_rows(float rows, int& i0, int& i1, float&
   }
 }
 
-// Wave totals of a and of b (what wave_sum returns for each), as wave-uniform values: a in the lower half of the
-// wave, b in the upper half from the first step on.
-__device__ __forceinline__ void wave_sum2(float a, float b, float& ta, float& tb) {
-  float v = fold32(a, b);
-  const uint32_t u = __float_as_uint(v);
-  auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
-  v = row_sum(__uint_as_float(r[0]) + __uint_as_float(r[1]));
-  ta = lane_value(v, 0);
-  tb = lane_value(v, 32);
-}
-
-// LayerNorm statistics of two rows held in registers: ln_stats for each, the wave sums taken together
-template <int NCHUNK>
-__device__ __forceinline__ void ln_stats2(const uint4 (&va)[NCHUNK], const uint4 (&vb)[NCHUNK], float fD, float eps,
-                                          float& mean_a, float& rstd_a, float& mean_b, float& rstd_b) {
-  float sa = 0.0f, sb = 0.0f;
+// E dot products of one token row with the fp32 gate weight in LDS. Unit (e, c, lane) of the bf16 weight (8
+// elements) is the two float4 at [(e * NCHUNK + c) * 2 + half][lane]: a lane's reads are 16 bytes wide and
+// lane-contiguous (no bank conflicts). Step s = c * E + e multiplies chunk c with the unit of expert e. The LDS reads
+// run RA steps ahead of the arithmetic and no further: each step's empty statement defines the lane offset the next
+// reads use and consumes the sum of the step before, so the compiler can neither gather all reads at the top (the
+// whole slice, E * D / 64 values, in registers: that is what it does when left alone, and it costs the occupancy
+// these kernels live on) nor hoist them out of the token loop.
+template <int E, int NCHUNK, int RA>
+__device__ __forceinline__ void dot_rows(const uint4 (&row)[NCHUNK], const float4* wf, int lane, float (&acc)[E]) {
+  constexpr int STEPS = NCHUNK * E;
+#pragma unroll
+  for (int e = 0; e < E; ++e) acc[e] = 0.0f;
+  int wlane = lane;
+  asm volatile("" : "+v"(wlane));
+  float4 wlo[RA], whi[RA];
+#pragma unroll
+  for (int s = 0; s < RA && s < STEPS; ++s) {
+    const int u = (s % E) * NCHUNK + s / E;
+    wlo[s] = wf[(u * 2 + 0) * 64 + wlane];
+    whi[s] = wf[(u * 2 + 1) * 64 + wlane];
+  }
 #pragma unroll
   for (int c = 0; c < NCHUNK; ++c) {
-    float f[8], g[8];
-    unpack8(va[c], f);
-    unpack8(vb[c], g);
-#pragma unroll
-    for (int j = 0; j < 8; ++j) { sa = sa + f[j]; sb = sb + g[j]; }
-  }
-  float ta, tb;
-  wave_sum2(sa, sb, ta, tb);
-  mean_a = __fdiv_rn(ta, fD);
-  mean_b = __fdiv_rn(tb, fD);
-  float qa = 0.0f, qb = 0.0f;
-#pragma unroll
-  for (int c = 0; c < NCHUNK; ++c) {
-    float f[8], g[8];
-    unpack8(va[c], f);
-    unpack8(vb[c], g);
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const float da = f[j] - mean_a, db = g[j] - mean_b;
-      qa = __builtin_fmaf(da, da, qa);
-      qb = __builtin_fmaf(db, db, qb);
-    }
-  }
-  wave_sum2(qa, qb, ta, tb);
-  rstd_a = __fdiv_rn(1.0f, __builtin_sqrtf(__fdiv_rn(ta, fD) + eps));
-  rstd_b = __fdiv_rn(1.0f, __builtin_sqrtf(__fdiv_rn(tb, fD) + eps));
-}
-
-template <int E, int NCHUNK, bool QUANT, bool LN = false>
-__global__ __launch_bounds__(WAVES_PER_BLOCK * 64, 2) void gate_top2_reg_kernel(
-    const uint4* __restrict__ x, const uint4* __restrict__ wg, int T, int tpb, int32_t* __restrict__ idx,
-    uint16_t* __restrict__ wout, int32_t* __restrict__ block_hist, GateQuant q) {
-  const int lane = threadIdx.x & 63;
-  const int wv = threadIdx.x >> 6;
-  constexpr int ROW16 = NCHUNK * 64;  // 16-byte units per row
-  // Pairs of consecutive tokens. tpb > 0: block b owns tokens [b * tpb, (b + 1) * tpb) and its waves take the pairs
-  // of that range in turn; tpb == 0: the waves of the grid stride over the pairs of all tokens (see TokenWalk).
-  int t0, t_end, step;
-  if (tpb > 0) {
-    t0 = (int)blockIdx.x * tpb + 2 * wv;
-    t_end = min(T, (int)(blockIdx.x + 1) * tpb);
-    step = 2 * WAVES_PER_BLOCK;
-  } else {
-    t0 = 2 * ((int)blockIdx.x * WAVES_PER_BLOCK + wv);
-    t_end = T;
-    step = 2 * (int)gridDim.x * WAVES_PER_BLOCK;
-  }
-  // the wave's first pair is requested before the block fills LDS with the gate weight: the two latencies overlap.
-  // A pair whose second token lies past the end reads its first token twice and drops the copy's results.
-  uint4 cur0[NCHUNK], cur1[NCHUNK], nxt0[NCHUNK], nxt1[NCHUNK];
-  auto load_pair = [&](int t, uint4 (&a)[NCHUNK], uint4 (&b)[NCHUNK]) {
-    const int tb = t + 1 < t_end ? t + 1 : t;
-#pragma unroll
-    for (int c = 0; c < NCHUNK; ++c) a[c] = x[(size_t)t * ROW16 + c * 64 + lane];
-#pragma unroll
-    for (int c = 0; c < NCHUNK; ++c) b[c] = x[(size_t)tb * ROW16 + c * 64 + lane];
-  };
-  if (t0 < t_end) load_pair(t0, cur0, cur1);
-  // gate weight -> LDS as fp32. Unit (e, c, lane) of the bf16 weight (8 elements) becomes the two float4 at
-  // [(e * NCHUNK + c) * 2 + half][lane]: a lane's reads are 16 bytes wide and lane-contiguous (no bank conflicts).
-  __shared__ float4 wf[E * NCHUNK * 2 * 64];
-  for (int i = threadIdx.x; i < E * ROW16; i += WAVES_PER_BLOCK * 64) {
-    const uint4 v = wg[i];
-    const int unit = i >> 6, l = i & 63;
-    wf[(unit * 2 + 0) * 64 + l] = make_float4(bf16_lo(v.x), bf16_hi(v.x), bf16_lo(v.y), bf16_hi(v.y));
-    wf[(unit * 2 + 1) * 64 + l] = make_float4(bf16_lo(v.z), bf16_hi(v.z), bf16_lo(v.w), bf16_hi(v.w));
-  }
-  __syncthreads();
-
-  int cnt[E];
-#pragma unroll
-  for (int e = 0; e < E; ++e) cnt[e] = 0;
-  // the 1/scale_input of every expert, read once: a load that depends on the routing inside the token loop
-  // would make every token wait for its predecessor's stores (loads and stores retire in order)
-  float inv_e[E], invs = -1.0f;
-  bool one_row = false, with_shared = false;
-  if constexpr (QUANT) {
-    bool ok13 = true, same = true;
+    float xa[8];
+    unpack8(row[c], xa);
 #pragma unroll
     for (int e = 0; e < E; ++e) {
-      inv_e[e] = hdmoe_q_inv_scale(q.scale_in.p[e]);
-      if (q.scale_in3.p[e] != q.scale_in.p[e]) ok13 = ok13 && hdmoe_q_inv_scale(q.scale_in3.p[e]) == inv_e[e];
-    }
-    invs = hdmoe_q_uniform(hdmoe_q_inv_scale(q.shared_scale));
-    if (q.shared_scale3 != q.shared_scale) ok13 = ok13 && hdmoe_q_inv_scale(q.shared_scale3) == invs;
+      const int st = c * E + e;
+      const float4 lo = wlo[st % RA], hi = whi[st % RA];
+      if (st + RA < STEPS) {
+        const int u = ((st + RA) % E) * NCHUNK + (st + RA) / E;
+        asm volatile("" : "+v"(wlane), "+v"(acc[e == 0 ? E - 1 : e - 1]));
+        wlo[st % RA] = wf[(u * 2 + 0) * 64 + wlane];
+        whi[st % RA] = wf[(u * 2 + 1) * 64 + wlane];
+      }
+      const float w8[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
 #pragma unroll
-    for (int e = 0; e < E; ++e) same = same && inv_e[e] == invs;
-    one_row = q.decide ? same : q.xq_routed == nullptr;
-    with_shared = q.decide ? q.with_shared != 0 : q.xq_shared != nullptr;
-    if (!ok13) {
-      // the factors are NaN from here on: every product and so every byte written below is NaN
-      invs = __builtin_nanf("");
-#pragma unroll
-      for (int e = 0; e < E; ++e) inv_e[e] = invs;
-    }
-    if (blockIdx.x == 0 && threadIdx.x == 0) {
-      if (q.decide) *q.layout_flag = same ? 1 : 0;
-      if (!ok13 && q.scale_check != nullptr) *q.scale_check = 1;
+      for (int j = 0; j < 8; ++j) acc[e] = __builtin_fmaf(xa[j], w8[j], acc[e]);
     }
   }
-  auto write_token = [&](int t, const uint4 (&row)[NCHUNK], int i0, int i1, float s0, float s1) {
-    if (lane == 0) {
-      reinterpret_cast<int2*>(idx)[t] = make_int2(i0, i1);
-      reinterpret_cast<uint32_t*>(wout)[t] = GateBf16::pack(s0, s1);
-    }
-#pragma unroll
-    for (int e = 0; e < E; ++e) cnt[e] += (i0 == e) + (i1 == e);
-    if constexpr (QUANT) {
-      if (one_row) {
-        // one scale_input for all: one row per token
-#pragma unroll
-        for (int c = 0; c < NCHUNK; ++c) q.xq_shared[(size_t)t * ROW16 + c * 64 + lane] = hdmoe_q_8(row[c], invs);
-      } else {
-        float inv0 = inv_e[0], inv1 = inv_e[0];
-#pragma unroll
-        for (int e = 1; e < E; ++e) {
-          inv0 = i0 == e ? inv_e[e] : inv0;
-          inv1 = i1 == e ? inv_e[e] : inv1;
-        }
-        inv0 = hdmoe_q_uniform(inv0);
-        inv1 = hdmoe_q_uniform(inv1);
-        uint2* r0 = q.xq_routed + (size_t)(2 * t) * ROW16;
-        const bool same01 = inv0 == inv1, same0s = inv0 == invs;  // equal scales: cast once, store again
-#pragma unroll
-        for (int c = 0; c < NCHUNK; ++c) {
-          const uint2 v0 = hdmoe_q_8(row[c], inv0);
-          r0[c * 64 + lane] = v0;
-          r0[ROW16 + c * 64 + lane] = same01 ? v0 : hdmoe_q_8(row[c], inv1);
-          if (with_shared)
-            q.xq_shared[(size_t)t * ROW16 + c * 64 + lane] = same0s ? v0 : hdmoe_q_8(row[c], invs);
-        }
-      }
-    }
-  };
-  for (; t0 < t_end; t0 += step) {
-    const int tn = t0 + step;
-    if (tn < t_end) load_pair(tn, nxt0, nxt1);
-    const bool has1 = t0 + 1 < t_end;
-    if constexpr (LN) {
-      float m0, r0, m1, r1;
-      ln_stats2<NCHUNK>(cur0, cur1, (float)(NCHUNK * 512), q.ln_eps, m0, r0, m1, r1);
-      const int t1 = has1 ? t0 + 1 : t0;
-      const size_t b0 = (size_t)(t0 / q.tokens_per_batch) * ROW16, b1 = (size_t)(t1 / q.tokens_per_batch) * ROW16;
-#pragma unroll
-      for (int c = 0; c < NCHUNK; ++c) {
-        cur0[c] = modulate8(cur0[c], q.mod_scale[b0 + c * 64 + lane], q.mod_shift[b0 + c * 64 + lane], m0, r0);
-        cur1[c] = modulate8(cur1[c], q.mod_scale[b1 + c * 64 + lane], q.mod_shift[b1 + c * 64 + lane], m1, r1);
-      }
-    }
-    float acc0[E], acc1[E];
-#pragma unroll
-    for (int e = 0; e < E; ++e) acc0[e] = acc1[e] = 0.0f;
-    // opaque per trip, or the compiler hoists the weight reads out of the token loop and keeps the slice in registers
-    int wlane = lane;
-    asm volatile("" : "+v"(wlane));
-#pragma unroll
-    for (int c = 0; c < NCHUNK; ++c) {
-      float xa[8], xb[8];
-      unpack8(cur0[c], xa);
-      unpack8(cur1[c], xb);
-#pragma unroll
-      for (int e = 0; e < E; ++e) {
-        const float4 wlo = wf[((e * NCHUNK + c) * 2 + 0) * 64 + wlane], whi = wf[((e * NCHUNK + c) * 2 + 1) * 64 + wlane];
-        const float w8[8] = {wlo.x, wlo.y, wlo.z, wlo.w, whi.x, whi.y, whi.z, whi.w};
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          acc0[e] = __builtin_fmaf(xa[j], w8[j], acc0[e]);
-          acc1[e] = __builtin_fmaf(xb[j], w8[j], acc1[e]);
-        }
-      }
-      // nothing moves across: the scheduler would otherwise issue the weight reads of every chunk up front and keep
-      // E * D / 64 values live
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    // both tokens' sums are formed here: left to itself the compiler sinks the second token's arithmetic into the
-    // branch that stores its results and keeps the whole weight slice in registers until then
-#pragma unroll
-    for (int e = 0; e < E; ++e) asm volatile("" : "+v"(acc0[e]), "+v"(acc1[e]));
-    int i0, i1, j0, j1;
-    float s0, s1, u0, u1;
-    finish_rows<E>(expert_rows<E>(acc0), i0, i1, s0, s1);
-    finish_rows<E>(expert_rows<E>(acc1), j0, j1, u0, u1);
-    write_token(t0, cur0, i0, i1, s0, s1);
-    if (has1) write_token(t0 + 1, cur1, j0, j1, u0, u1);
-#pragma unroll
-    for (int c = 0; c < NCHUNK; ++c) { cur0[c] = nxt0[c]; cur1[c] = nxt1[c]; }
-  }
-  write_block_hist<E>(cnt, block_hist);
 }
 
-// ---- routing and cast by different waves ------------------------------------------------------------------
-// Eight waves per block, two blocks per CU. Waves 0-3 route: one token per trip, the next token's row requested a
-// trip ahead, the dot products as above (fp32 gate weight in LDS, folded wave sums); their only stores are the 12
-// bytes of routing per token. Waves 4-7 cast: they load the same tokens, cast them and store the fp8 rows, two rows
-// in flight, and never touch the gate weight (they pass the fill barrier at once). A wave that does both computes,
-// then casts and stores, and while its stores and the next loads queue up behind those of every other wave its
-// arithmetic cannot issue (instructions issue in order); with two kinds of wave the arithmetic of one overlaps the
-// memory traffic of the other, and sixteen waves per CU instead of eight cover each other's waits. The second read
-// of a row comes from cache: both waves of a token sit on one CU and ask for it at about the same time.
-// Measured inside the layer (kernel start to last store, 8192 / 4096 / 256 tokens): 19 / 12 / 7 us against
-// 24 / 18 / 11 us of the kernel above doing both in every wave.
-// The split needs a cast that does not depend on the routing, i.e. one cast factor for every expert. Where the
-// scale values say otherwise (decided here, on the device) the cast waves wait, and behind a barrier all eight
-// waves write the per-slot rows from the routing the first four have left in idx.
-// Every floating-point operation of the routing has the operands and the order of the one-token form: same bits.
-constexpr int ROLE_WAVES = 4;          // waves per role and block
-constexpr int ROLES_BLOCKS_PER_CU = 2;
-constexpr int WEIGHT_READAHEAD = 3;    // (chunk, expert) steps the LDS reads run ahead of the arithmetic
+// What the cast needs to know about the scale values (see GateQuant), the same in every wave of the grid.
+template <int E>
+struct CastFacts {
+  float inv_e[E], invs;        // (1 / scale_input).to(bf16) per expert and for the shared expert; NaN where w1 and
+                               // w3 of a feed-forward disagree: every product and so every byte written is NaN
+  bool one_row, with_shared;   // one row per token for all readers; per-slot rows plus the shared expert's copy
+};
+// The raw values are asked for early (before the weight fill's barrier), the facts derived behind it.
+template <int E>
+struct ScaleValues { float in1[E], in3[E], shared1, shared3; };
+template <int E>
+__device__ __forceinline__ ScaleValues<E> request_scales(const GateQuant& q) {
+  ScaleValues<E> v;
+#pragma unroll
+  for (int e = 0; e < E; ++e) {
+    v.in1[e] = q.scale_in.p[e] != nullptr ? *q.scale_in.p[e] : 0.0f;
+    v.in3[e] = q.scale_in3.p[e] != nullptr ? *q.scale_in3.p[e] : 0.0f;
+  }
+  v.shared1 = q.shared_scale != nullptr ? *q.shared_scale : 0.0f;
+  v.shared3 = q.shared_scale3 != nullptr ? *q.shared_scale3 : 0.0f;
+  return v;
+}
+template <int E>
+__device__ __forceinline__ CastFacts<E> cast_facts(const GateQuant& q, const ScaleValues<E>& v) {
+  // NULL pointer: the clamp rule's marker
+  auto inv_of = [](const float* p, float s) { return p == nullptr ? -1.0f : hdmoe_dev_round_bf16(__fdiv_rn(1.0f, s)); };
+  CastFacts<E> f;
+  bool ok13 = true, same = true;
+#pragma unroll
+  for (int e = 0; e < E; ++e) {
+    f.inv_e[e] = hdmoe_q_uniform(inv_of(q.scale_in.p[e], v.in1[e]));
+    if (q.scale_in3.p[e] != q.scale_in.p[e]) ok13 = ok13 && inv_of(q.scale_in3.p[e], v.in3[e]) == f.inv_e[e];
+  }
+  f.invs = hdmoe_q_uniform(inv_of(q.shared_scale, v.shared1));
+  if (q.shared_scale3 != q.shared_scale) ok13 = ok13 && inv_of(q.shared_scale3, v.shared3) == f.invs;
+#pragma unroll
+  for (int e = 0; e < E; ++e) same = same && f.inv_e[e] == f.invs;
+  f.one_row = q.decide ? same : q.xq_routed == nullptr;
+  f.with_shared = q.decide ? q.with_shared != 0 : q.xq_shared != nullptr;
+  if (!ok13) {
+    f.invs = __builtin_nanf("");
+#pragma unroll
+    for (int e = 0; e < E; ++e) f.inv_e[e] = f.invs;
+  }
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    if (q.decide) *q.layout_flag = same ? 1 : 0;
+    if (!ok13 && q.scale_check != nullptr) *q.scale_check = 1;
+  }
+  return f;
+}
 
+// the fp8 rows of token t: one row for all readers, or a row per slot (and the shared expert's copy)
 template <int E, int NCHUNK>
-__global__ __launch_bounds__(2 * ROLE_WAVES * 64, 2 * ROLES_BLOCKS_PER_CU) void gate_cast_roles_kernel(
+__device__ __forceinline__ void cast_token(const uint4 (&row)[NCHUNK], int t, int i0, int i1, const CastFacts<E>& f,
+                                           const GateQuant& q, int lane) {
+  constexpr int ROW16 = NCHUNK * 64;
+  if (f.one_row) {
+#pragma unroll
+    for (int c = 0; c < NCHUNK; ++c) q.xq_shared[(size_t)t * ROW16 + c * 64 + lane] = hdmoe_q_8(row[c], f.invs);
+    return;
+  }
+  float inv0 = f.inv_e[0], inv1 = f.inv_e[0];
+#pragma unroll
+  for (int e = 1; e < E; ++e) {
+    inv0 = i0 == e ? f.inv_e[e] : inv0;
+    inv1 = i1 == e ? f.inv_e[e] : inv1;
+  }
+  inv0 = hdmoe_q_uniform(inv0);
+  inv1 = hdmoe_q_uniform(inv1);
+  uint2* r0 = q.xq_routed + (size_t)(2 * t) * ROW16;
+  const bool same01 = inv0 == inv1, same0s = inv0 == f.invs;  // equal scales: cast once, store again
+#pragma unroll
+  for (int c = 0; c < NCHUNK; ++c) {
+    const uint2 v0 = hdmoe_q_8(row[c], inv0);
+    r0[c * 64 + lane] = v0;
+    r0[ROW16 + c * 64 + lane] = same01 ? v0 : hdmoe_q_8(row[c], inv1);
+    if (f.with_shared) q.xq_shared[(size_t)t * ROW16 + c * 64 + lane] = same0s ? v0 : hdmoe_q_8(row[c], f.invs);
+  }
+}
+
+// Three forms of one kernel, eight waves per block and two blocks per CU in each:
+//   GATE_ROUTE  routing only (bf16 experts, the stage entry point): eight routing waves.
+//   GATE_SPLIT  routing and the fp8 cast by different waves. Waves 0-3 route; their only stores are the 12 bytes of
+//     routing per token. Waves 4-7 cast: they load the same tokens, cast them and store the fp8 rows, two rows in
+//     flight, never touch the gate weight and pass the fill barrier at once. A wave that does both computes, then
+//     casts and stores, and while its stores and next loads queue up behind those of every other wave its arithmetic
+//     cannot issue (instructions issue in order); with two kinds of wave the arithmetic of one overlaps the memory
+//     traffic of the other. The second read of a row comes from cache: both waves of a token sit on one CU and ask
+//     for it at about the same time. The split needs a cast that does not depend on the routing, i.e. one cast
+//     factor for every expert; where the scale values say otherwise (decided here, on the device) the cast waves
+//     wait, and behind a barrier all eight waves write the per-slot rows from the routing the first four have left
+//     in idx. Measured inside the layer (kernel start to last store, 8192 / 4096 / 256 tokens): 19 / 12 / 7 us
+//     against 24 / 18 / 11 us with eight waves per CU that each route and cast two tokens per trip.
+//   GATE_LN     LayerNorm + modulation in front (the block branch's form): about 800 vector instructions per token,
+//     bound by arithmetic, so every wave does all of it for its tokens and nothing is computed twice (with the split
+//     both kinds of wave would normalise the row: 115 instead of 81 us at 32768 tokens).
+enum GateForm { GATE_ROUTE = 0, GATE_SPLIT = 1, GATE_LN = 2 };
+constexpr int ROW_WAVES = 8;           // waves per block of the register kernels
+constexpr int ROW_BLOCKS_PER_CU = 2;
+
+template <int E, int NCHUNK, int FORM>
+__global__ __launch_bounds__(ROW_WAVES * 64, ROW_WAVES * ROW_BLOCKS_PER_CU / 4) void gate_row_kernel(
     const uint4* __restrict__ x, const uint4* __restrict__ wg, int T, int tpb, int32_t* __restrict__ idx,
     uint16_t* __restrict__ wout, int32_t* __restrict__ block_hist, GateQuant q) {
+  constexpr bool CAST = FORM != GATE_ROUTE, SPLIT = FORM == GATE_SPLIT, LN = FORM == GATE_LN;
+  constexpr int RW = SPLIT ? ROW_WAVES / 2 : ROW_WAVES;   // routing waves per block
+  constexpr int RA = LN ? 2 : 3;                          // LDS read-ahead; a third step spills in the LN form
+  constexpr int ROW16 = NCHUNK * 64;                      // 16-byte units per row
   const int lane = threadIdx.x & 63;
   const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int rw = wv % ROLE_WAVES;
-  const bool caster = wv >= ROLE_WAVES;
-  constexpr int ROW16 = NCHUNK * 64;
-  // the tokens of wave rw of either role: block ranges or grid-strided (see TokenWalk)
+  const int rw = wv % RW;
+  const bool caster = SPLIT && wv >= RW;
+  // the tokens of wave rw (of either kind): block ranges, or strided over the grid (see TokenWalk)
   int t0, t_end, step;
   if (tpb > 0) {
     t0 = (int)blockIdx.x * tpb + rw;
     t_end = min(T, (int)(blockIdx.x + 1) * tpb);
-    step = ROLE_WAVES;
+    step = RW;
   } else {
-    t0 = (int)blockIdx.x * ROLE_WAVES + rw;
+    t0 = (int)blockIdx.x * RW + rw;
     t_end = T;
-    step = (int)gridDim.x * ROLE_WAVES;
+    step = (int)gridDim.x * RW;
   }
   const int t_first = t0;
   uint4 row[NCHUNK], nxt[NCHUNK];
@@ -584,32 +501,25 @@ __global__ __launch_bounds__(2 * ROLE_WAVES * 64, 2 * ROLES_BLOCKS_PER_CU) void 
 #pragma unroll
     for (int c = 0; c < NCHUNK; ++c) r[c] = x[(size_t)t * ROW16 + c * 64 + lane];
   };
-  // gate weight -> LDS as fp32 (layout as in gate_top2_reg_kernel), by the routing waves, requested in front of
-  // their first row
+  // gate weight -> LDS as fp32, by the routing waves, requested in front of their first row; the scale values are
+  // asked for before the barrier too, so that all three latencies pass together
   __shared__ float4 wf[E * NCHUNK * 2 * 64];
-  constexpr int FILL = (E * ROW16 + ROLE_WAVES * 64 - 1) / (ROLE_WAVES * 64);
+  constexpr int FILL = (E * ROW16 + RW * 64 - 1) / (RW * 64);
   uint4 wpart[FILL];
   if (!caster) {
 #pragma unroll
     for (int k = 0; k < FILL; ++k) {
-      const int i = threadIdx.x + k * ROLE_WAVES * 64;
+      const int i = threadIdx.x + k * RW * 64;
       wpart[k] = i < E * ROW16 ? wg[i] : make_uint4(0, 0, 0, 0);
     }
   }
   if (t0 < t_end) load_row(t0, row);
-  // the scale values are asked for before the barrier, so that their latency passes behind it
-  float sc1[E], sc3[E];
-#pragma unroll
-  for (int e = 0; e < E; ++e) {
-    sc1[e] = q.scale_in.p[e] != nullptr ? *q.scale_in.p[e] : 0.0f;
-    sc3[e] = q.scale_in3.p[e] != nullptr ? *q.scale_in3.p[e] : 0.0f;
-  }
-  const float scs1 = q.shared_scale != nullptr ? *q.shared_scale : 0.0f;
-  const float scs3 = q.shared_scale3 != nullptr ? *q.shared_scale3 : 0.0f;
+  ScaleValues<E> scales;
+  if constexpr (CAST) scales = request_scales<E>(q);
   if (!caster) {
 #pragma unroll
     for (int k = 0; k < FILL; ++k) {
-      const int i = threadIdx.x + k * ROLE_WAVES * 64;
+      const int i = threadIdx.x + k * RW * 64;
       if (i < E * ROW16) {
         const uint4 v = wpart[k];
         const int unit = i >> 6, l = i & 63;
@@ -619,74 +529,26 @@ __global__ __launch_bounds__(2 * ROLE_WAVES * 64, 2 * ROLES_BLOCKS_PER_CU) void 
     }
   }
   __syncthreads();
+  CastFacts<E> facts;
+  if constexpr (CAST) facts = cast_facts<E>(q, scales);
 
-  // decisions and checks on the scale values (see GateQuant); NULL pointer: the clamp rule's marker
-  auto inv_of = [](const float* p, float v) { return p == nullptr ? -1.0f : hdmoe_dev_round_bf16(__fdiv_rn(1.0f, v)); };
-  float inv_e[E];
-  bool ok13 = true, same = true;
-#pragma unroll
-  for (int e = 0; e < E; ++e) {
-    inv_e[e] = hdmoe_q_uniform(inv_of(q.scale_in.p[e], sc1[e]));
-    if (q.scale_in3.p[e] != q.scale_in.p[e]) ok13 = ok13 && inv_of(q.scale_in3.p[e], sc3[e]) == inv_e[e];
-  }
-  float invs = hdmoe_q_uniform(inv_of(q.shared_scale, scs1));
-  if (q.shared_scale3 != q.shared_scale) ok13 = ok13 && inv_of(q.shared_scale3, scs3) == invs;
-#pragma unroll
-  for (int e = 0; e < E; ++e) same = same && inv_e[e] == invs;
-  const bool one_row = q.decide ? same : q.xq_routed == nullptr;
-  const bool with_shared = q.decide ? q.with_shared != 0 : q.xq_shared != nullptr;
-  if (!ok13) {
-    invs = __builtin_nanf("");   // every product and so every byte written below is NaN
-#pragma unroll
-    for (int e = 0; e < E; ++e) inv_e[e] = invs;
-  }
-  if (blockIdx.x == 0 && threadIdx.x == 0) {
-    if (q.decide) *q.layout_flag = same ? 1 : 0;
-    if (!ok13 && q.scale_check != nullptr) *q.scale_check = 1;
-  }
   int cnt[E];
 #pragma unroll
   for (int e = 0; e < E; ++e) cnt[e] = 0;
   if (!caster) {
     for (; t0 < t_end; t0 += step) {
       const int tn = t0 + step;
-      if (tn < t_end) load_row(tn, nxt);
+      if (tn < t_end) load_row(tn, nxt);   // the next token's row, a trip ahead
+      if constexpr (LN) {
+        float m, r;
+        ln_stats<NCHUNK>(row, (float)(NCHUNK * 512), q.ln_eps, m, r);
+        const size_t b0 = (size_t)(t0 / q.tokens_per_batch) * ROW16;
+#pragma unroll
+        for (int c = 0; c < NCHUNK; ++c)
+          row[c] = modulate8(row[c], q.mod_scale[b0 + c * 64 + lane], q.mod_shift[b0 + c * 64 + lane], m, r);
+      }
       float acc[E];
-#pragma unroll
-      for (int e = 0; e < E; ++e) acc[e] = 0.0f;
-      // Step s = c * E + e multiplies chunk c with the weight unit of expert e. The LDS reads run WEIGHT_READAHEAD
-      // steps ahead of the arithmetic and no further: each step's empty statement defines the lane offset the next
-      // reads use and consumes the sum of the step before, so the compiler can neither gather the reads at the top
-      // of the trip (the whole slice in registers) nor hoist them out of the token loop.
-      constexpr int RA = WEIGHT_READAHEAD, STEPS = NCHUNK * E;
-      int wlane = lane;
-      asm volatile("" : "+v"(wlane));
-      float4 wlo[RA], whi[RA];
-#pragma unroll
-      for (int s = 0; s < RA && s < STEPS; ++s) {
-        const int u = (s % E) * NCHUNK + s / E;
-        wlo[s] = wf[(u * 2 + 0) * 64 + wlane];
-        whi[s] = wf[(u * 2 + 1) * 64 + wlane];
-      }
-#pragma unroll
-      for (int c = 0; c < NCHUNK; ++c) {
-        float xa[8];
-        unpack8(row[c], xa);
-#pragma unroll
-        for (int e = 0; e < E; ++e) {
-          const int st = c * E + e;
-          const float4 lo = wlo[st % RA], hi = whi[st % RA];
-          if (st + RA < STEPS) {
-            const int u = ((st + RA) % E) * NCHUNK + (st + RA) / E;
-            asm volatile("" : "+v"(wlane), "+v"(acc[e == 0 ? E - 1 : e - 1]));
-            wlo[st % RA] = wf[(u * 2 + 0) * 64 + wlane];
-            whi[st % RA] = wf[(u * 2 + 1) * 64 + wlane];
-          }
-          const float w8[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
-#pragma unroll
-          for (int j = 0; j < 8; ++j) acc[e] = __builtin_fmaf(xa[j], w8[j], acc[e]);
-        }
-      }
+      dot_rows<E, NCHUNK, RA>(row, wf, lane, acc);
       int i0, i1;
       float s0, s1;
       finish_rows<E>(expert_rows<E>(acc), i0, i1, s0, s1);
@@ -696,10 +558,11 @@ __global__ __launch_bounds__(2 * ROLE_WAVES * 64, 2 * ROLES_BLOCKS_PER_CU) void 
       }
 #pragma unroll
       for (int e = 0; e < E; ++e) cnt[e] += (i0 == e) + (i1 == e);
+      if constexpr (LN) cast_token<E, NCHUNK>(row, t0, i0, i1, facts, q, lane);
 #pragma unroll
       for (int c = 0; c < NCHUNK; ++c) row[c] = nxt[c];
     }
-  } else if (one_row) {
+  } else if (facts.one_row) {
     // two rows in flight: the cast itself is a few instructions, the wave's time is memory latency
     if (t0 + step < t_end) load_row(t0 + step, nxt);
     for (; t0 < t_end; t0 += 2 * step) {
@@ -707,7 +570,7 @@ __global__ __launch_bounds__(2 * ROLE_WAVES * 64, 2 * ROLES_BLOCKS_PER_CU) void 
         if (t >= t_end) return;
         uint2 o[NCHUNK];
 #pragma unroll
-        for (int c = 0; c < NCHUNK; ++c) o[c] = hdmoe_q_8(r[c], invs);
+        for (int c = 0; c < NCHUNK; ++c) o[c] = hdmoe_q_8(r[c], facts.invs);
         if (t + 2 * step < t_end) load_row(t + 2 * step, r);
 #pragma unroll
         for (int c = 0; c < NCHUNK; ++c) q.xq_shared[(size_t)t * ROW16 + c * 64 + lane] = o[c];
@@ -716,34 +579,20 @@ __global__ __launch_bounds__(2 * ROLE_WAVES * 64, 2 * ROLES_BLOCKS_PER_CU) void 
       cast_row(t0 + step, nxt);
     }
   }
-  if (!one_row) {
-    // a cast per slot: all eight waves, from the routing the first four have written (the barrier makes a block's
-    // own global stores visible to its waves)
-    __syncthreads();
-    for (int t = t_first + (wv / ROLE_WAVES) * step; t < t_end; t += 2 * step) {
-      load_row(t, row);
-      const int2 r = reinterpret_cast<const int2*>(idx)[t];
-      const int i0 = __builtin_amdgcn_readfirstlane(r.x), i1 = __builtin_amdgcn_readfirstlane(r.y);
-      float inv0 = inv_e[0], inv1 = inv_e[0];
-#pragma unroll
-      for (int e = 1; e < E; ++e) {
-        inv0 = i0 == e ? inv_e[e] : inv0;
-        inv1 = i1 == e ? inv_e[e] : inv1;
-      }
-      inv0 = hdmoe_q_uniform(inv0);
-      inv1 = hdmoe_q_uniform(inv1);
-      uint2* r0 = q.xq_routed + (size_t)(2 * t) * ROW16;
-      const bool same01 = inv0 == inv1, same0s = inv0 == invs;  // equal scales: cast once, store again
-#pragma unroll
-      for (int c = 0; c < NCHUNK; ++c) {
-        const uint2 v0 = hdmoe_q_8(row[c], inv0);
-        r0[c * 64 + lane] = v0;
-        r0[ROW16 + c * 64 + lane] = same01 ? v0 : hdmoe_q_8(row[c], inv1);
-        if (with_shared) q.xq_shared[(size_t)t * ROW16 + c * 64 + lane] = same0s ? v0 : hdmoe_q_8(row[c], invs);
+  if constexpr (SPLIT) {
+    if (!facts.one_row) {
+      // a cast per slot: all eight waves, from the routing the first four have written (the barrier makes a block's
+      // own global stores visible to its waves)
+      __syncthreads();
+      for (int t = t_first + (wv / RW) * step; t < t_end; t += 2 * step) {
+        load_row(t, row);
+        const int2 r = reinterpret_cast<const int2*>(idx)[t];
+        cast_token<E, NCHUNK>(row, t, __builtin_amdgcn_readfirstlane(r.x), __builtin_amdgcn_readfirstlane(r.y), facts,
+                              q, lane);
       }
     }
   }
-  write_block_hist<E, 2 * ROLE_WAVES>(cnt, block_hist);
+  write_block_hist<E, ROW_WAVES>(cnt, block_hist);
 }
 
 // Any D that is a multiple of 8: Wg is re-read through the cache hierarchy.
@@ -807,20 +656,30 @@ __global__ __launch_bounds__(WAVES_PER_BLOCK * 64) void gate_top2_generic_kernel
   write_block_hist<E>(cnt, block_hist);
 }
 
+// which kernel a launch gets, as a function of the sizes and of what the kernel has to do besides routing
+enum GateKernel { KERNEL_GENERIC, KERNEL_ROUTE, KERNEL_SPLIT, KERNEL_LN };
+GateKernel gate_kernel_of(int D, int E, bool f16, bool with_cast, bool with_ln) {
+  if (f16 || E > 4 || D != 2560) return KERNEL_GENERIC;
+  return !with_cast ? KERNEL_ROUTE : (with_ln ? KERNEL_LN : KERNEL_SPLIT);
+}
+// tokens a block takes per trip, and resident blocks per CU
+int gate_trip_tokens(GateKernel k) { return k == KERNEL_GENERIC ? WAVES_PER_BLOCK : (k == KERNEL_SPLIT ? ROW_WAVES / 2 : ROW_WAVES); }
+int gate_resident_blocks(GateKernel k) { return HDMOE_NUM_CU * (k == KERNEL_GENERIC ? 3 : ROW_BLOCKS_PER_CU); }
+
 template <int E>
 int launch_gate(const void* x, const void* wg, int T, int D, int32_t* idx, void* w, const GateQuant* quant,
                 int32_t* block_hist, hipStream_t s, const char* what, bool f16) {
-  // with histograms: block ranges; without: waves strided over the tokens (gate_top2_reg_kernel: over token pairs),
-  // at least two tokens per wave, and no more blocks than are resident at once
-  const bool reg_kernel = !f16 && E <= 4 && D == 2560;
   const bool ln = quant != nullptr && quant->mod_scale != nullptr;
-  const bool roles = !f16 && hdmoe_gate_splits_roles(D, E, quant != nullptr, ln);
+  const GateKernel kernel = gate_kernel_of(D, E, f16, quant != nullptr, ln);
+  if (ln && kernel != KERNEL_LN) return hdmoe_fail(HDMOE_E_SHAPE, "%s: the LayerNorm variant needs D = 2560 and E <= 4", what);
+  if (f16 && quant) return hdmoe_fail(HDMOE_E_SHAPE, "%s: the fp8 cast takes bf16 activations", what);
+  // with histograms: block ranges; without: waves strided over the tokens, at least two tokens per wave of the
+  // generic kernel, and no more blocks than are resident at once
   const int tpb = block_hist != nullptr ? hdmoe_gate_tokens_per_block(T, D, E, quant != nullptr, ln) : 0;
-  const int per_trip = roles ? ROLE_WAVES : 2 * WAVES_PER_BLOCK;
-  int blocks = tpb > 0 ? (T + tpb - 1) / tpb : (T + per_trip - 1) / per_trip;
-  const int resident = HDMOE_NUM_CU * (roles ? ROLES_BLOCKS_PER_CU : reg_kernel ? GATE_BLOCKS_PER_CU : 3);
-  if (tpb == 0 && blocks > resident) blocks = resident;
-  dim3 grid(blocks < 1 ? 1 : blocks), block((roles ? 2 * ROLE_WAVES : WAVES_PER_BLOCK) * 64);
+  const int per_block = kernel == KERNEL_GENERIC ? 2 * WAVES_PER_BLOCK : gate_trip_tokens(kernel);
+  int blocks = tpb > 0 ? (T + tpb - 1) / tpb : (T + per_block - 1) / per_block;
+  if (tpb == 0 && blocks > gate_resident_blocks(kernel)) blocks = gate_resident_blocks(kernel);
+  dim3 grid(blocks < 1 ? 1 : blocks), block((kernel == KERNEL_GENERIC ? WAVES_PER_BLOCK : ROW_WAVES) * 64);
   const uint4* xp = static_cast<const uint4*>(x);
   const uint4* wp = static_cast<const uint4*>(wg);
   uint16_t* wo = static_cast<uint16_t*>(w);
@@ -828,24 +687,25 @@ int launch_gate(const void* x, const void* wg, int T, int D, int32_t* idx, void*
   memset(&q, 0, sizeof(q));
   if (quant) q = *quant;
   constexpr int ER = E <= 4 ? E : 4;  // the register kernels are only instantiated for up to 4 experts
-  if (f16) {
-    if (quant) return hdmoe_fail(HDMOE_E_SHAPE, "%s: the fp8 cast takes bf16 activations", what);
-    hipLaunchKernelGGL((gate_top2_generic_kernel<E, false, GateF16>), grid, block, 0, s, xp, wp, T, D, tpb, idx, wo,
-                       block_hist, q);
-  } else if (roles) {
-    hipLaunchKernelGGL((gate_cast_roles_kernel<ER, 5>), grid, block, 0, s, xp, wp, T, tpb, idx, wo, block_hist, q);
-  } else if (reg_kernel) {
-    // the cast without the LayerNorm goes to gate_cast_roles_kernel
-    if (quant)
-      hipLaunchKernelGGL((gate_top2_reg_kernel<ER, 5, true, true>), grid, block, 0, s, xp, wp, T, tpb, idx, wo, block_hist, q);
-    else
-      hipLaunchKernelGGL((gate_top2_reg_kernel<ER, 5, false>), grid, block, 0, s, xp, wp, T, tpb, idx, wo, block_hist, q);
-  } else {
-    if (ln) return hdmoe_fail(HDMOE_E_SHAPE, "%s: the LayerNorm variant needs D = 2560 and E <= 4", what);
-    if (quant)
-      hipLaunchKernelGGL((gate_top2_generic_kernel<E, true>), grid, block, 0, s, xp, wp, T, D, tpb, idx, wo, block_hist, q);
-    else
-      hipLaunchKernelGGL((gate_top2_generic_kernel<E, false>), grid, block, 0, s, xp, wp, T, D, tpb, idx, wo, block_hist, q);
+  switch (kernel) {
+    case KERNEL_ROUTE:
+      hipLaunchKernelGGL((gate_row_kernel<ER, 5, GATE_ROUTE>), grid, block, 0, s, xp, wp, T, tpb, idx, wo, block_hist, q);
+      break;
+    case KERNEL_SPLIT:
+      hipLaunchKernelGGL((gate_row_kernel<ER, 5, GATE_SPLIT>), grid, block, 0, s, xp, wp, T, tpb, idx, wo, block_hist, q);
+      break;
+    case KERNEL_LN:
+      hipLaunchKernelGGL((gate_row_kernel<ER, 5, GATE_LN>), grid, block, 0, s, xp, wp, T, tpb, idx, wo, block_hist, q);
+      break;
+    case KERNEL_GENERIC:
+      if (f16)
+        hipLaunchKernelGGL((gate_top2_generic_kernel<E, false, GateF16>), grid, block, 0, s, xp, wp, T, D, tpb, idx, wo,
+                           block_hist, q);
+      else if (quant)
+        hipLaunchKernelGGL((gate_top2_generic_kernel<E, true>), grid, block, 0, s, xp, wp, T, D, tpb, idx, wo, block_hist, q);
+      else
+        hipLaunchKernelGGL((gate_top2_generic_kernel<E, false>), grid, block, 0, s, xp, wp, T, D, tpb, idx, wo, block_hist, q);
+      break;
   }
   return hdmoe_check_launch(what);
 }
@@ -943,23 +803,13 @@ extern "C" int hdmoe_gate_top2_f16(const void* x_f16, const void* gate_w_f16, in
                        static_cast<hipStream_t>(stream), "hdmoe_gate_top2_f16", true);
 }
 
-// Which of the gate + cast kernels a launch gets: the one with routing and cast waves takes the cast without the
-// LayerNorm at the register kernels' shape (with the LayerNorm both kinds of wave would compute it, and at 32768
-// tokens, where the kernel is bound by its arithmetic, that costs 20 us).
-bool hdmoe_gate_splits_roles(int D, int E, bool with_cast, bool with_ln) {
-  return E <= 4 && D == 2560 && with_cast && !with_ln;
-}
-
-// Tokens per block of the gate kernels of the one-call layer, a pure function of the sizes and of the kernel.
-// Register kernel (two tokens per wave and trip) and the kernel with routing and cast waves (one token per routing
-// wave and trip): two blocks per CU, all resident at once, each block a whole number of trips. Generic kernel: three
-// blocks per CU, at least one token per wave. Very large T gets more blocks instead of more than 1024 tokens each
-// (the dispatch's scatter pass handles one or several whole blocks per chunk, at most 1024 tokens).
+// Tokens per block of the gate kernels of the one-call layer, a pure function of the sizes and of the kernel
+// (with_cast: fp8 experts; with_ln: LayerNorm + modulation inside the kernel). All blocks resident at once, each a
+// whole number of trips. Very large T gets more blocks instead of more than 1024 tokens each (the dispatch's scatter
+// pass handles one or several whole blocks per chunk, at most 1024 tokens).
 int hdmoe_gate_tokens_per_block(int T, int D, int E, bool with_cast, bool with_ln) {
-  const bool reg_kernel = E <= 4 && D == 2560;
-  const bool roles = hdmoe_gate_splits_roles(D, E, with_cast, with_ln);
-  const int resident = HDMOE_NUM_CU * (roles ? ROLES_BLOCKS_PER_CU : reg_kernel ? GATE_BLOCKS_PER_CU : 3);
-  const int unit = roles ? ROLE_WAVES : (reg_kernel ? 2 * WAVES_PER_BLOCK : WAVES_PER_BLOCK);
+  const GateKernel kernel = gate_kernel_of(D, E, false, with_cast, with_ln);
+  const int resident = gate_resident_blocks(kernel), unit = gate_trip_tokens(kernel);
   int tpb = (T + resident - 1) / resident;
   tpb = (tpb + unit - 1) / unit * unit;
   if (tpb < unit) tpb = unit;
