@@ -22,6 +22,7 @@
 namespace {
 
 constexpr int WAVES_PER_BLOCK = 4;
+constexpr int GENERIC_TOKENS_PER_TRIP = 4;   // tokens a wave of the generic kernel takes together
 
 __device__ __forceinline__ float exp_neg(float x) {
   // exp(x), x <= 0: ln2 split range reduction, degree-5 polynomial, exponent
@@ -625,31 +626,51 @@ __global__ __launch_bounds__(WAVES_PER_BLOCK * 64) void gate_top2_generic_kernel
       if (!ok13 && q.scale_check != nullptr) *q.scale_check = 1;
     }
   }
-  for (int t = walk.first; t < t_end; t += walk.step) {
-    float logit[E];
+  // Up to TG tokens of the wave's walk per trip: one read of a weight slice serves them all, and the weight traffic
+  // through the caches, E * D * 2 bytes per token otherwise, is what bounds this kernel. Each token's sums are formed
+  // from the same operands in the same order as alone.
+  constexpr int TG = GENERIC_TOKENS_PER_TRIP;
+  for (int t = walk.first; t < t_end; t += TG * walk.step) {
+    float logit[TG][E];
 #pragma unroll
-    for (int e = 0; e < E; ++e) logit[e] = 0.0f;
+    for (int g = 0; g < TG; ++g)
+#pragma unroll
+      for (int e = 0; e < E; ++e) logit[g][e] = 0.0f;
     for (int u = lane; u < row16; u += 64) {
-      uint4 xv = x[(size_t)t * row16 + u];
+      uint4 xv[TG];
 #pragma unroll
-      for (int e = 0; e < E; ++e) logit[e] = dot8<A>(xv, wg[(size_t)e * row16 + u], logit[e]);
+      for (int g = 0; g < TG; ++g) {
+        const int tg = t + g * walk.step;
+        xv[g] = x[(size_t)(tg < t_end ? tg : t) * row16 + u];   // past the end: the first token again, result dropped
+      }
+#pragma unroll
+      for (int e = 0; e < E; ++e) {
+        const uint4 wv = wg[(size_t)e * row16 + u];
+#pragma unroll
+        for (int g = 0; g < TG; ++g) logit[g][e] = dot8<A>(xv[g], wv, logit[g][e]);
+      }
     }
-    int i0, i1;
-    finish_token<E, A>(logit, lane, t, idx, wout, i0, i1);
 #pragma unroll
-    for (int e = 0; e < E; ++e) cnt[e] += (i0 == e) + (i1 == e);
-    if constexpr (QUANT) {
-      const float bad = __builtin_nanf("");   // a cast that cannot serve w1 and w3 alike: NaN rows
-      const float inv0 = hdmoe_q_uniform(ok13 ? hdmoe_q_inv_scale(q.scale_in.p[i0]) : bad);
-      const float inv1 = hdmoe_q_uniform(ok13 ? hdmoe_q_inv_scale(q.scale_in.p[i1]) : bad);
-      const float invs = hdmoe_q_uniform(ok13 ? hdmoe_q_inv_scale(q.shared_scale) : bad);
-      for (int u = lane; u < row16; u += 64) {
-        const uint4 xv = x[(size_t)t * row16 + u];
-        if (!one_row) {
-          q.xq_routed[(size_t)(2 * t) * row16 + u] = hdmoe_q_8(xv, inv0);
-          q.xq_routed[(size_t)(2 * t + 1) * row16 + u] = hdmoe_q_8(xv, inv1);
+    for (int g = 0; g < TG; ++g) {
+      const int tg = t + g * walk.step;
+      if (tg >= t_end) break;
+      int i0, i1;
+      finish_token<E, A>(logit[g], lane, tg, idx, wout, i0, i1);
+#pragma unroll
+      for (int e = 0; e < E; ++e) cnt[e] += (i0 == e) + (i1 == e);
+      if constexpr (QUANT) {
+        const float bad = __builtin_nanf("");   // a cast that cannot serve w1 and w3 alike: NaN rows
+        const float inv0 = hdmoe_q_uniform(ok13 ? hdmoe_q_inv_scale(q.scale_in.p[i0]) : bad);
+        const float inv1 = hdmoe_q_uniform(ok13 ? hdmoe_q_inv_scale(q.scale_in.p[i1]) : bad);
+        const float invs = hdmoe_q_uniform(ok13 ? hdmoe_q_inv_scale(q.shared_scale) : bad);
+        for (int u = lane; u < row16; u += 64) {
+          const uint4 xv = x[(size_t)tg * row16 + u];
+          if (!one_row) {
+            q.xq_routed[(size_t)(2 * tg) * row16 + u] = hdmoe_q_8(xv, inv0);
+            q.xq_routed[(size_t)(2 * tg + 1) * row16 + u] = hdmoe_q_8(xv, inv1);
+          }
+          if (one_row || with_shared) q.xq_shared[(size_t)tg * row16 + u] = hdmoe_q_8(xv, invs);
         }
-        if (one_row || with_shared) q.xq_shared[(size_t)t * row16 + u] = hdmoe_q_8(xv, invs);
       }
     }
   }
@@ -674,7 +695,8 @@ int launch_gate(const void* x, const void* wg, int T, int D, int32_t* idx, void*
   if (ln && kernel != KERNEL_LN) return hdmoe_fail(HDMOE_E_SHAPE, "%s: the LayerNorm variant needs D = 2560 and E <= 4", what);
   if (f16 && quant) return hdmoe_fail(HDMOE_E_SHAPE, "%s: the fp8 cast takes bf16 activations", what);
   // with histograms: block ranges; without: waves strided over the tokens, at least two tokens per wave of the
-  // generic kernel, and no more blocks than are resident at once
+  // generic kernel (more waves with fewer tokens each beat fewer waves with a full group of four: 29 against 31 us
+  // at 8192 tokens, 8 experts, width 2048), and no more blocks than are resident at once
   const int tpb = block_hist != nullptr ? hdmoe_gate_tokens_per_block(T, D, E, quant != nullptr, ln) : 0;
   const int per_block = kernel == KERNEL_GENERIC ? 2 * WAVES_PER_BLOCK : gate_trip_tokens(kernel);
   int blocks = tpb > 0 ? (T + tpb - 1) / tpb : (T + per_block - 1) / per_block;
