@@ -414,7 +414,7 @@ def main():
     for n in stage_ms:
         stage_ms[n] /= stage_steps * n_layers     # per layer
     stage_ms["gemm_gate_up"] = dom_ms             # from the timed steps
-    for evs in ev_sets:
+    for evs in stage_sets:
         hip.destroy(evs)
 
     fp8 = cfg["weights"] == "fp8"
