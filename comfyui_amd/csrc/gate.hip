@@ -1,18 +1,18 @@
-// Gate kernel: logits = x . Wg^T, softmax, top-2 with lowest-index tie-break.
+// Gate kernels: logits = x . Wg^T, softmax, top-2 with lowest-index tie-break.
 // Replaces MoEGate.forward (/root/reference/comfy/ldm/hidream/model.py:263-283).
 //
 // One token per wavefront. Lane l owns the 8-element groups starting at element
 // l*8 + c*512 (c = 0, 1, ...): a 16-byte load per lane and chunk, so a wave reads
 // 1 KiB of the token row per load instruction, fully coalesced. A lane needs the
-// same slice of Wg for every token; the block keeps Wg in LDS (packed bf16) and a
-// lane re-reads its slice per token. The E dot products are
-// accumulated in fp32 with fma in ascending element order per lane and reduced
-// across the wave with an xor butterfly (32, 16, 8, 4, 2, 1). That order is fixed
-// on purpose: it is the order the CPU checker restates, which makes logits,
-// scores and therefore the routing reproducible bit for bit.
+// same slice of Wg for every token: the kernels for HiDream's shape keep Wg in LDS
+// as fp32, the generic kernel re-reads it through the caches for four tokens at a
+// time. The E dot products are accumulated in fp32 with fma in ascending element
+// order per lane and reduced across the wave with an xor butterfly (32, 16, 8, 4,
+// 2, 1). That order is fixed on purpose: it is the order the CPU checker restates,
+// which makes logits, scores and therefore the routing reproducible bit for bit.
 //
-// HBM traffic per token: D*2 bytes read, 12 bytes written; the kernel is
-// bandwidth bound (the E x D weight is 20 KiB and stays in LDS / L2).
+// HBM traffic per token: D*2 bytes read, 12 bytes written (plus D bytes where the
+// kernel also casts the token to fp8 for the expert GEMMs).
 #include "common.h"
 #include "numfmt.h"
 #include "quant.h"
@@ -230,8 +230,7 @@ struct GateQuant {
 //     first pass of the dispatch's counting sort: block b writes its E counts to block_hist[b * E ..] and the
 //     dispatch needs no counting launch of its own;
 //   tpb == 0: the waves of the grid stride over the tokens (wave g: g, g + waves in the grid, ...), so that at any
-//     moment the grid reads one contiguous stretch of x: 1.5 us (8192 tokens) to 9 us (32768 tokens with the
-//     LayerNorm) faster than the block ranges, without histograms.
+//     moment the grid reads one contiguous stretch of x; no histograms (the stage entry points).
 struct TokenWalk { int first, end, step; };
 __device__ __forceinline__ TokenWalk token_walk(int T, int tpb) {
   const int wv = threadIdx.x >> 6;

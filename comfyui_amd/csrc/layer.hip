@@ -67,7 +67,8 @@ extern "C" int hdmoe_layer_layout_get(int T, int D, int H, int Hs, int E, int we
   out->offsets = take((size_t)(E + 1) * 4);
   out->perm = take(n * 4);
   out->inv_perm = take(n * 4);
-  // per-block expert histograms of the gate kernel (the first pass of the dispatch)
+  // per-block expert histograms of the gate kernel (the first pass of the dispatch); large enough for hdmoe_dispatch
+  // too, for a caller that composes the layer from the stages inside this workspace
   {
     const size_t a = hdmoe_gate_hist_bytes(T, D, E, fp8), b = hdmoe_dispatch_workspace_bytes(T, E);
     out->dispatch_ws = take(a > b ? a : b);
@@ -136,10 +137,8 @@ extern "C" int hdmoe_moe_ffn(const hdmoe_layer_args* p, hdmoe_stream_t stream) {
   int32_t* offsets = reinterpret_cast<int32_t*>(ws + l.offsets);
   int32_t* perm = reinterpret_cast<int32_t*>(ws + l.perm);
   int32_t* inv_perm = reinterpret_cast<int32_t*>(ws + l.inv_perm);
-  // Up to 16384 tokens the gate kernel also counts (one expert histogram per block) and the dispatch is its scatter
-  // pass alone; above, the gate kernel's faster token order without histograms and the two-pass dispatch win.
-  int32_t* const dispatch_ws = reinterpret_cast<int32_t*>(ws + l.dispatch_ws);
-  int32_t* const hist = T <= 16384 ? dispatch_ws : nullptr;
+  // The gate kernel also counts (one expert histogram per block of tokens), so the dispatch is its scatter pass alone.
+  int32_t* const hist = reinterpret_cast<int32_t*>(ws + l.dispatch_ws);
   uint8_t* a_routed = ws + l.a;
   uint8_t* a_shared = a_routed + (size_t)n * D * eb;  // fp8 only
   uint8_t* h_routed = ws + l.h;
@@ -232,15 +231,9 @@ extern "C" int hdmoe_moe_ffn(const hdmoe_layer_args* p, hdmoe_stream_t stream) {
     if (int rc = hdmoe_launch_gate(xin, p->gate_w, T, D, E, idx, tw, hist, s, "hdmoe_moe_ffn (gate)")) return rc;
   }
   mark();
-  if (hist != nullptr) {
-    if (int rc = hdmoe_launch_dispatch_scatter(idx, T, E, counts, offsets, perm, inv_perm, hist,
-                                               hdmoe_gate_tokens_per_block(T, D, E, fp8, ln_in_gate), s, "hdmoe_moe_ffn (dispatch)"))
-      return rc;
-  } else {
-    if (int rc = hdmoe_dispatch(idx, T, E, counts, offsets, perm, inv_perm, dispatch_ws,
-                                hdmoe_dispatch_workspace_bytes(T, E), stream))
-      return rc;
-  }
+  if (int rc = hdmoe_launch_dispatch_scatter(idx, T, E, counts, offsets, perm, inv_perm, hist,
+                                             hdmoe_gate_tokens_per_block(T, D, E, fp8, ln_in_gate), s, "hdmoe_moe_ffn (dispatch)"))
+    return rc;
   mark();
 
   // bf16 weights: the GEMM reads the tokens themselves, the routed rows through the permutation (row perm[r] / 2
