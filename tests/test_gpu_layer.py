@@ -321,13 +321,14 @@ def test_layer_casts_activations_in_the_gate_kernel_bit_exactly(dev, dim, E, sca
 
 @pytest.mark.parametrize("weights", ["fp8", "bf16"])
 @pytest.mark.parametrize("dim,E,T", [(256, 4, 1), (256, 4, 7), (256, 3, 129), (2560, 4, 333), (256, 8, 4097),
-                                     (2560, 4, 8192), (256, 4, 33000)])
+                                     (2560, 4, 8192), (256, 4, 33000), (2560, 3, 3), (2560, 3, 20001), (2560, 2, 40000)])
 def test_layer_dispatch_from_gate_histograms(dev, weights, dim, E, T):
     """Inside the one-call layer the gate kernel counts (one expert histogram per block of tokens) and the dispatch
     runs its second pass alone. counts, offsets, perm and inv_perm in the layer's workspace: equal to the CPU
     checker's stable sort of the same routing, at token counts around the block and chunk sizes (one token, a
-    partial block, more than one chunk, the large-chunk form above 32768 tokens), with 3, 4 and 8 experts and both
-    gate kernels (row in registers at D = 2560, generic otherwise)."""
+    partial block, more than one chunk, the large-chunk form above 32768 tokens, blocks of more than one trip at
+    D = 2560), with 2, 3, 4 and 8 experts and both gate kernels (row in registers at D = 2560, generic otherwise);
+    the routing rows themselves against the fixed-order checker."""
     from comfyui_amd import functional as HF
     from comfyui_amd import _lib
     hidden_arg = 512
@@ -348,6 +349,8 @@ def test_layer_dispatch_from_gate_histograms(dev, weights, dim, E, T):
 
     def ints(off, n):
         return ws[off:off + 4 * n].cpu().view(torch.int32)
+    ref_idx, _, _, _ = O.gate_fixed_order(x.reshape(T, dim), sd["gate.weight"])
+    assert torch.equal(idx.cpu(), ref_idx.to(torch.int32))
     counts_r, offs_r, perm_r, inv_r = O.dispatch(idx.cpu(), E)
     assert torch.equal(ints(lay.counts, E), counts_r.to(torch.int32))
     assert torch.equal(ints(lay.offsets, E + 1), offs_r.to(torch.int32))
